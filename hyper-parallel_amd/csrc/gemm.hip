@@ -1,0 +1,357 @@
+// Scaled FP8 GEMMs for gfx950: c[m,n] = sum_kb sa(m,kb) * sb(n,kb) * (A_kb . B_kb^T).
+//
+// Layout of the work
+//   * Both operands are K-contiguous E4M3 codes, so a 16-row x 128-byte slab of either is exactly
+//     one operand of v_mfma_f32_16x16x128_f8f6f4: one matrix instruction consumes one whole
+//     128-wide scaling block, and its fp32 result is promoted into the running accumulator with
+//     one FMA per element (acc += partial * sa * sb).
+//   * The weight-like operand b feeds the MFMA "A" port and the activation-like operand a the
+//     "B" port: a lane then holds 4 consecutive n for one m, which makes the per-row scale
+//     sa(m,kb) a per-lane constant and the bf16 store 8 contiguous bytes.
+//   * Workgroup tile 256(m) x 256(n) x 128(k), 8 waves as 4(m) x 2(n), wave tile 64 x 128
+//     (128 fp32 accumulators per lane, 2 waves per SIMD so one wave's FMAs overlap the other's
+//     MFMAs).  Two LDS stages of 64 KB; tiles are DMA'd global -> LDS with 128-bit buffer loads
+//     (out-of-range rows read as zero), 16-byte chunks XOR-swizzled by row so that both the DMA
+//     writes and the ds_read_b128 fragment reads are bank-conflict free.
+//   * Workgroup ids are remapped so that each XCD (own L2) works on a contiguous run of tiles.
+#include "hpfp8_device.h"
+#include "hpfp8_host.h"
+
+namespace hpfp8 {
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int kGemmThreads = 512;
+constexpr int kTileBytes = 256 * BK;          // one operand tile in LDS
+constexpr int kStageBytes = 2 * kTileBytes;   // a tile then b tile
+constexpr int kXcds = 8;
+
+enum ScaleMode { kScaleTensor = 0, kScaleBlock = 1, kScaleRow = 2 };
+
+struct GemmParams {
+  const uint8_t* a;
+  const uint8_t* b;
+  const float* sa;
+  const float* sb;
+  int64_t sa_sm, sa_sk;   // element strides of sa over (row, k-block)
+  int64_t sb_sn, sb_sk;   // element strides of sb over (row or 128-row block, k-block)
+  int64_t sb_se;          // grouped: stride of sb between experts
+  void* c;
+  int64_t ldc;
+  const uint16_t* bias;
+  const int32_t* offs;    // grouped: inclusive prefix sums of rows per expert
+  int experts;
+  int M, N, K;            // M = total rows of a
+  int accumulate;
+};
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+__device__ __forceinline__ v4i lds_read16(const uint8_t* p) {
+  return *reinterpret_cast<const v4i*>(p);
+}
+
+__device__ __forceinline__ v8i frag_read(const uint8_t* row_base, int pc0) {
+  v4i lo = lds_read16(row_base + pc0 * 16);
+  v4i hi = lds_read16(row_base + (pc0 ^ 1) * 16);
+  v8i r;
+  r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+  r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+  return r;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  __bf16 x = (__bf16)a, y = (__bf16)b;
+  return (uint32_t)__builtin_bit_cast(uint16_t, x) | ((uint32_t)__builtin_bit_cast(uint16_t, y) << 16);
+}
+
+template <int MODE, bool GROUPED, bool OUT_F32>
+__global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageBytes];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int K = p.K, N = p.N;
+  const int kblocks = K / BK;
+  const int tiles_n = (N + BN - 1) / BN;
+
+  // ---- workgroup -> tile, XCD aware: ids congruent mod 8 share an XCD and get a contiguous run
+  int t;
+  {
+    const int nblk = gridDim.x, pid = blockIdx.x;
+    const int xcd = pid % kXcds, local = pid / kXcds;
+    const int base = nblk / kXcds, big = nblk % kXcds;
+    t = xcd * base + (xcd < big ? xcd : big) + local;
+  }
+  int row0, row_end, tn, expert = 0;
+  if (GROUPED) {
+    int total_mt = 0;
+    for (int e = 0, prev = 0; e < p.experts; ++e) {
+      int end = p.offs[e];
+      total_mt += (end - prev + BM - 1) / BM;
+      prev = end;
+    }
+    if (total_mt == 0 || t >= total_mt * tiles_n) return;
+    tn = t / total_mt;
+    int mt = t % total_mt;
+    int prev = 0;
+    row0 = 0;
+    row_end = 0;
+    for (int e = 0; e < p.experts; ++e) {
+      int end = p.offs[e];
+      int cnt = (end - prev + BM - 1) / BM;
+      if (mt < cnt) {
+        expert = e;
+        row0 = prev + mt * BM;
+        row_end = end < p.M ? end : p.M;
+        break;
+      }
+      mt -= cnt;
+      prev = end;
+    }
+  } else {
+    const int tiles_m = (p.M + BM - 1) / BM;
+    if (t >= tiles_m * tiles_n) return;
+    tn = t / tiles_m;
+    row0 = (t % tiles_m) * BM;
+    row_end = p.M;
+  }
+  const int n0 = tn * BN;
+
+  // ---- global -> LDS tile DMA.  One wave instruction moves 8 rows x 128 B (lane i -> LDS slot
+  // i); the lane picks the 16-byte global chunk whose swizzled home is its slot.
+  const uint8_t* bbase = p.b + (GROUPED ? (int64_t)expert * N * K : 0);
+  const __amdgpu_buffer_rsrc_t rsrc_a =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)((int64_t)p.M * K), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b =
+      __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, (int)((int64_t)N * K), 0x00020000);
+  uint32_t a_off[4], b_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int q = wave * 4 + i;                       // 8-row group inside the tile
+    const int r = q * 8 + (lane >> 3);                // row inside the tile
+    const int chunk = (lane & 7) ^ ((r >> 1) & 7);    // logical 16-byte chunk of that row
+    a_off[i] = (uint32_t)(row0 + r) * (uint32_t)K + chunk * 16;
+    b_off[i] = (uint32_t)(n0 + r) * (uint32_t)K + chunk * 16;
+  }
+  auto issue_tile_loads = [&](int kb, int stage) {
+    uint8_t* sbase = lds + stage * kStageBytes + wave * 4096;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sbase + i * 1024), 16, a_off[i],
+                                               kb * BK, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sbase + kTileBytes + i * 1024), 16,
+                                               b_off[i], kb * BK, 0, 0);
+    }
+  };
+
+  // ---- fragment addressing
+  const int wn = wave & 1, wm = wave >> 1;
+  const int l16 = lane & 15, g = lane >> 4;
+  const int pc0 = (2 * g) ^ (l16 >> 1);
+  const int a_frag_off = (wm * 64 + l16) * BK;               // + j * 16 rows
+  const int b_frag_off = kTileBytes + (wn * 128 + l16) * BK;  // + i * 16 rows
+
+  // ---- scales
+  int arow[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int r = row0 + wm * 64 + j * 16 + l16;
+    arow[j] = r < p.M ? r : p.M - 1;
+  }
+  const float* sbp = p.sb + (GROUPED ? (int64_t)expert * p.sb_se : 0);
+  int nblk_idx = (n0 + wn * 128) >> 7;
+  if (nblk_idx > (N >> 7) - 1) nblk_idx = (N >> 7) - 1;
+  auto load_scales = [&](int kb, float s[4]) {
+    if (MODE == kScaleBlock) {
+      const float sbv = sbp[(int64_t)nblk_idx * p.sb_sn + (int64_t)kb * p.sb_sk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[j] = p.sa[(int64_t)arow[j] * p.sa_sm + (int64_t)kb * p.sa_sk] * sbv;
+    } else if (MODE == kScaleRow) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[j] = p.sa[(int64_t)arow[j] * p.sa_sm + (int64_t)kb * p.sa_sk];
+    }
+  };
+
+  v4f acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_nxt[4] = {1.f, 1.f, 1.f, 1.f};
+  load_scales(0, s_cur);
+  issue_tile_loads(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+
+  for (int kb = 0; kb < kblocks; ++kb) {
+    const int stage = kb & 1;
+    if (kb + 1 < kblocks) {
+      issue_tile_loads(kb + 1, stage ^ 1);
+      load_scales(kb + 1, s_nxt);
+    }
+    const uint8_t* sbase = lds + stage * kStageBytes;
+    v8i xf[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const v8i wf = frag_read(sbase + b_frag_off + i * 16 * BK, pc0);
+      float sbr[4] = {1.f, 1.f, 1.f, 1.f};
+      if (MODE == kScaleRow) {
+        int n = n0 + wn * 128 + i * 16 + g * 4;
+        if (n > N - 4) n = N - 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sbr[r] = p.sb[(int64_t)(n + r) * p.sb_sn + (int64_t)kb * p.sb_sk];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (MODE == kScaleTensor) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+        } else {
+          const v4f zero = {0.f, 0.f, 0.f, 0.f};
+          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], zero, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            if (MODE == kScaleRow)
+              acc[i][j][r] = __builtin_fmaf(part[r], s_cur[j] * sbr[r], acc[i][j][r]);
+            else
+              acc[i][j][r] = __builtin_fmaf(part[r], s_cur[j], acc[i][j][r]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s_cur[j] = s_nxt[j];
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // own DMA for the next stage has landed
+    __syncthreads();                     // everyone's has, and everyone is done reading this stage
+  }
+
+  // ---- epilogue
+  float tensor_scale = 1.f;
+  if (MODE == kScaleTensor) tensor_scale = p.sa[0] * p.sb[0];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int n = n0 + wn * 128 + i * 16 + g * 4;
+    if (n >= N) continue;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+      const uint2 braw = *reinterpret_cast<const uint2*>(p.bias + n);
+      bv[0] = bf16lo(braw.x); bv[1] = bf16hi(braw.x); bv[2] = bf16lo(braw.y); bv[3] = bf16hi(braw.y);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = row0 + wm * 64 + j * 16 + l16;
+      if (m >= row_end) continue;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] = acc[i][j][r];
+        if (MODE == kScaleTensor) v[r] *= tensor_scale;
+        v[r] += bv[r];
+      }
+      if (OUT_F32) {
+        float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.c) + (int64_t)m * p.ldc + n);
+        float4 o = make_float4(v[0], v[1], v[2], v[3]);
+        if (p.accumulate) {
+          float4 old = *dst;
+          o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
+        }
+        *dst = o;
+      } else {
+        uint2 o;
+        o.x = pack_bf16x2(v[0], v[1]);
+        o.y = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + n) = o;
+      }
+    }
+  }
+}
+
+template <int MODE, bool GROUPED>
+static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
+  dim3 grid((unsigned)tiles), block(kGemmThreads);
+  if (out_type == HPFP8_OUT_F32)
+    gemm_kernel<MODE, GROUPED, true><<<grid, block, 0, stream>>>(p);
+  else
+    gemm_kernel<MODE, GROUPED, false><<<grid, block, 0, stream>>>(p);
+  return check_launch("gemm");
+}
+
+static int check_common(const char* what, const void* a, const void* b, const float* sa, const float* sb,
+                        int64_t M, int64_t N, int64_t K, const void* bias, const void* c, int64_t ldc,
+                        int out_type, int accumulate) {
+  HPFP8_REQUIRE(M >= 0 && N >= 0 && K >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
+  HPFP8_REQUIRE(K > 0 && K % BK == 0 && N % kBlock == 0, HPFP8_ERR_SHAPE,
+                "%s: K=%lld must be a positive multiple of 128 and N=%lld a multiple of 128", what, (long long)K,
+                (long long)N);
+  HPFP8_REQUIRE(out_type == HPFP8_OUT_BF16 || out_type == HPFP8_OUT_F32, HPFP8_ERR_ARG, "%s: bad out_type", what);
+  HPFP8_REQUIRE(!accumulate || out_type == HPFP8_OUT_F32, HPFP8_ERR_ARG, "%s: accumulate needs fp32 output", what);
+  HPFP8_REQUIRE(ldc >= N, HPFP8_ERR_SHAPE, "%s: ldc=%lld smaller than N=%lld", what, (long long)ldc, (long long)N);
+  HPFP8_REQUIRE(ldc % 4 == 0, HPFP8_ERR_ALIGN, "%s: ldc must be a multiple of 4", what);
+  if (M == 0 || N == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(a && b && sa && sb && c, HPFP8_ERR_ARG, "%s: null buffer", what);
+  HPFP8_REQUIRE(aligned16(a) && aligned16(b) && aligned16(c) && (!bias || aligned16(bias)), HPFP8_ERR_ALIGN,
+                "%s: buffers must be 16-byte aligned", what);
+  // 32-bit byte offsets inside the tile loader, including rows read past the end of a tile
+  HPFP8_REQUIRE((M + BM) * K < (int64_t)0x7FFFFFFF && (N + BN) * K < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
+                "%s: an operand exceeds 2 GiB", what);
+  return 1;
+}
+
+}  // namespace hpfp8
+
+using namespace hpfp8;
+
+extern "C" {
+
+int hpfp8_gemm_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                         const void* b, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+                         int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
+                         int64_t ldc, int out_type, int accumulate, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(sb_gran == 1 || sb_gran == 128, HPFP8_ERR_ARG, "gemm_blockwise: sb_gran must be 1 or 128");
+  int rc = check_common("gemm_blockwise", a, b, sa, sb, M, N, K, bias, c, ldc, out_type, accumulate);
+  if (rc <= 0) return rc;
+  GemmParams p{};
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb;
+  p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k; p.sb_sn = sb_stride_n; p.sb_sk = sb_stride_k;
+  p.c = c; p.ldc = ldc; p.bias = (const uint16_t*)bias;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.accumulate = accumulate;
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (sb_gran == 128) return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
+  return launch<kScaleRow, false>(p, out_type, tiles, (hipStream_t)stream);
+}
+
+int hpfp8_gemm_per_tensor(const void* a, const float* sa_inv, const void* b, const float* sb_inv,
+                          int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
+                          int out_type, hpfp8_stream_t stream) {
+  int rc = check_common("gemm_per_tensor", a, b, sa_inv, sb_inv, M, N, K, bias, c, ldc, out_type, 0);
+  if (rc <= 0) return rc;
+  GemmParams p{};
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa_inv; p.sb = sb_inv;
+  p.c = c; p.ldc = ldc; p.bias = (const uint16_t*)bias;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  return launch<kScaleTensor, false>(p, out_type, tiles, (hipStream_t)stream);
+}
+
+int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, const void* b, const float* sb,
+                                 const int32_t* offs, int experts, int64_t total_m, int64_t N,
+                                 int64_t K, void* c, int64_t ldc, int out_type, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "gemm_grouped: bad expert count %d", experts);
+  int rc = check_common("gemm_grouped", a, b, sa, sb, total_m, N, K, nullptr, c, ldc, out_type, 0);
+  if (rc <= 0) return rc;
+  if (experts == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(offs != nullptr, HPFP8_ERR_ARG, "gemm_grouped: null offs");
+  GemmParams p{};
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb;
+  p.sa_sm = K / BK; p.sa_sk = 1;
+  p.sb_sn = K / BK; p.sb_sk = 1; p.sb_se = (N / kBlock) * (K / BK);
+  p.c = c; p.ldc = ldc; p.offs = offs; p.experts = experts;
+  p.M = (int)total_m; p.N = (int)N; p.K = (int)K;
+  // upper bound on row tiles: every expert may add one partial tile
+  const int64_t tiles = (total_m / BM + experts) * ((N + BN - 1) / BN);
+  return launch<kScaleBlock, true>(p, out_type, tiles, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,100 @@
+// Device-side helpers shared by the quantize and GEMM kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hpfp8 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short v2u16 __attribute__((ext_vector_type(2)));
+
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Streaming (non-temporal) 64/128-bit accesses for data touched exactly once.
+__device__ __forceinline__ uint4 nt_load16(const void* p) {
+  u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void nt_store16(void* p, const uint4& v) {
+  u32x4 t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+}
+__device__ __forceinline__ void nt_store8(void* p, const uint2& v) {
+  u32x2 t = {v.x, v.y};
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x2*>(p));
+}
+
+constexpr float kFp8Max = 448.0f;
+constexpr float kAmaxEps = 1e-12f;
+constexpr int kBlock = 128;
+
+// DPP controls (gfx9 encoding)
+constexpr int kDppQuadXor1 = 0xB1;      // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;      // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+
+// Packed max of two 16-bit magnitudes per word (bf16 |x| compares like an unsigned integer).
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  v2u16 r = __builtin_elementwise_max(__builtin_bit_cast(v2u16, a), __builtin_bit_cast(v2u16, b));
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
+// Max over the 16 lanes of a DPP row; every lane of the row ends with the result.
+__device__ __forceinline__ uint32_t row16_max_u32(uint32_t v) {
+  v = umax(v, dpp_u32<kDppQuadXor1>(v));
+  v = umax(v, dpp_u32<kDppQuadXor2>(v));
+  v = umax(v, dpp_u32<kDppRowHalfMirror>(v));
+  v = umax(v, dpp_u32<kDppRowMirror>(v));
+  return v;
+}
+
+// |bf16| magnitudes of the 8 values in a uint4, reduced to one 16-bit magnitude (low half).
+__device__ __forceinline__ uint32_t mag8(const uint4& v) {
+  uint32_t m = pk_max_u16(pk_max_u16(v.x & 0x7FFF7FFFu, v.y & 0x7FFF7FFFu),
+                          pk_max_u16(v.z & 0x7FFF7FFFu, v.w & 0x7FFF7FFFu));
+  return umax(m & 0xFFFFu, m >> 16);
+}
+
+__device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+
+// amax -> quantize multiplier and its inverse: two IEEE fp32 divisions, never rcp * x.
+__device__ __forceinline__ void scales_from_amax(float amax, float& scale, float& scale_inv) {
+  float amc = fmaxf(amax, kAmaxEps);
+  scale = kFp8Max / amc;
+  scale_inv = amc / kFp8Max;
+}
+
+__device__ __forceinline__ float clamp448(float y) {
+  return __builtin_amdgcn_fmed3f(y, -kFp8Max, kFp8Max);
+}
+
+// Two bf16 in one word -> two E4M3 codes in the chosen half of `old`.
+template <bool HI>
+__device__ __forceinline__ uint32_t cvt2(uint32_t old, uint32_t w, float scale) {
+  float a = clamp448(bf16lo(w) * scale);
+  float b = clamp448(bf16hi(w) * scale);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, HI);
+}
+
+// 8 bf16 (uint4) -> 8 E4M3 codes (uint2), element order kept.
+__device__ __forceinline__ uint2 cvt8(const uint4& v, float scale) {
+  uint2 r;
+  r.x = cvt2<true>(cvt2<false>(0u, v.x, scale), v.y, scale);
+  r.y = cvt2<true>(cvt2<false>(0u, v.z, scale), v.w, scale);
+  return r;
+}
+
+}  // namespace hpfp8

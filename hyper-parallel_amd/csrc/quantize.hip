@@ -1,0 +1,465 @@
+// Quantize / dequantize kernels for the FP8 linear path (gfx950).
+//
+// All of them are HBM-bound streaming kernels: 128-bit coalesced loads, |x| compared as packed
+// 16-bit integers (exact for bf16), amax reduced across lanes with DPP, scale = 448/amax by a
+// full IEEE division, E4M3 conversion with the hardware packed converter after an explicit
+// clamp to +-448, 64/128-bit stores.
+#include "hpfp8_device.h"
+#include "hpfp8_host.h"
+
+namespace hpfp8 {
+
+// ---------------------------------------------------------------------------------------------
+// per-tensor amax
+// ---------------------------------------------------------------------------------------------
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// amax_bits receives the fp32 bit pattern of max|x| (non-negative floats order like integers).
+__global__ __launch_bounds__(256) void amax_bf16_kernel(const uint16_t* __restrict__ x, int64_t n,
+                                                        uint32_t* __restrict__ amax_bits) {
+  const uint4* xv = reinterpret_cast<const uint4*>(x);
+  const int64_t nvec = n >> 3;
+  uint32_t m = 0;
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {
+    uint4 a = xv[i], b = xv[i + stride], c = xv[i + 2 * stride], d = xv[i + 3 * stride];
+    m = umax(m, umax(umax(mag8(a), mag8(b)), umax(mag8(c), mag8(d))));
+  }
+  for (; i < nvec; i += stride) m = umax(m, mag8(xv[i]));
+  if (blockIdx.x == 0 && threadIdx.x < (n & 7)) m = umax(m, x[(nvec << 3) + threadIdx.x] & 0x7FFFu);
+  m = row16_max_u32(m);
+  __shared__ uint32_t part[16];
+  if ((threadIdx.x & 15) == 0) part[threadIdx.x >> 4] = m;
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    m = row16_max_u32(part[threadIdx.x]);
+    if (threadIdx.x == 0) atomicMax(amax_bits, m << 16);
+  }
+}
+
+// Cast with one scale for the whole tensor; the scale is derived from *amax on the device.
+__global__ __launch_bounds__(256) void cast_per_tensor_kernel(const uint16_t* __restrict__ x, int64_t n,
+                                                              const float* __restrict__ amax,
+                                                              uint8_t* __restrict__ q,
+                                                              float* __restrict__ scale_out,
+                                                              float* __restrict__ scale_inv_out) {
+  float scale, scale_inv;
+  scales_from_amax(*amax, scale, scale_inv);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (scale_out) *scale_out = scale;
+    if (scale_inv_out) *scale_inv_out = scale_inv;
+  }
+  const uint4* xv = reinterpret_cast<const uint4*>(x);
+  uint2* qv = reinterpret_cast<uint2*>(q);
+  const int64_t nvec = n >> 3;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += stride)
+    qv[i] = cvt8(xv[i], scale);
+  if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {
+    int64_t j = (nvec << 3) + threadIdx.x;
+    uint32_t r = cvt2<false>(0u, x[j], scale);
+    q[j] = (uint8_t)(r & 0xFF);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 1x128 groups along the contiguous dim (activations, gradient buckets)
+// ---------------------------------------------------------------------------------------------
+// One group = 128 bf16 = 16 lanes x 16 B.  A thread handles UNROLL groups-slices so several
+// 128-bit loads are in flight before the first reduction.
+template <int UNROLL>
+__global__ __launch_bounds__(256) void quant_1x128_kernel(const uint4* __restrict__ x,
+                                                          uint2* __restrict__ q,
+                                                          float* __restrict__ scale,
+                                                          float* __restrict__ scale_inv,
+                                                          int64_t nvec) {
+  const int64_t base = (int64_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  uint4 v[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    int64_t i = base + u * 256;
+    v[u] = i < nvec ? nt_load16(&x[i]) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    int64_t i = base + u * 256;
+    uint32_t m = row16_max_u32(mag8(v[u]));
+    float s, si;
+    scales_from_amax(__uint_as_float(m << 16), s, si);
+    if (i < nvec) {
+      nt_store8(&q[i], cvt8(v[u], s));
+      if ((threadIdx.x & 15) == 0) {
+        if (scale) scale[i >> 4] = s;
+        scale_inv[i >> 4] = si;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// shared by the two tile kernels below: 128x128 tile, 256 threads
+// ---------------------------------------------------------------------------------------------
+// Thread t owns column group cg = t%16 (8 columns) and row quad rq = t/16: tile rows
+// {4rq..4rq+3} and {64+4rq..64+4rq+3}, i.e. load slot p -> row (p/4)*64 + 4rq + p%4.  Four
+// vertically adjacent codes then pack into one 32-bit word of the transposed tile.
+__device__ __forceinline__ int tile_row(int rq, int p) { return (p >> 2) * 64 + 4 * rq + (p & 3); }
+
+// 4x4 byte transpose: out[j] byte r = in[r] byte j.
+__device__ __forceinline__ void byte_transpose4(const uint32_t in[4], uint32_t out[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    out[j] = ((in[0] >> (8 * j)) & 0xFFu) | (((in[1] >> (8 * j)) & 0xFFu) << 8) |
+             (((in[2] >> (8 * j)) & 0xFFu) << 16) | (((in[3] >> (8 * j)) & 0xFFu) << 24);
+}
+
+// Writes the thread's codes c[p] (8 codes of tile row tile_row(rq,p)) into the transposed LDS
+// tile (row = tile column, 128 B; 16-byte chunks XOR-swizzled by the column group), then the
+// workgroup streams the tile out as 128 rows of dst (row stride ld bytes) with 128-bit stores.
+__device__ __forceinline__ void store_tile_transposed(uint8_t* tile, const uint2 c[8], int cg, int rq,
+                                                      uint8_t* __restrict__ dst, int64_t ld) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint32_t lo[4] = {c[4 * h].x, c[4 * h + 1].x, c[4 * h + 2].x, c[4 * h + 3].x};
+    const uint32_t hi[4] = {c[4 * h].y, c[4 * h + 1].y, c[4 * h + 2].y, c[4 * h + 3].y};
+    uint32_t wcol[8];
+    byte_transpose4(lo, wcol);
+    byte_transpose4(hi, wcol + 4);
+    const int rword = h * 16 + rq;  // 32-bit word inside the 128-byte transposed row
+    const int pc = (rword >> 2) ^ (cg & 7);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      *reinterpret_cast<uint32_t*>(&tile[(cg * 8 + j) * 128 + pc * 16 + (rword & 3) * 4]) = wcol[j];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int col = pass * 32 + (threadIdx.x >> 3);
+    const int pc = threadIdx.x & 7;
+    const int chunk = pc ^ ((col >> 3) & 7);
+    uint4 o = *reinterpret_cast<const uint4*>(&tile[col * 128 + pc * 16]);
+    *reinterpret_cast<uint4*>(dst + (int64_t)col * ld + chunk * 16) = o;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 128x128 blocks (weights), optional transposed copy of the codes for dgrad
+// ---------------------------------------------------------------------------------------------
+template <bool WITH_T>
+__global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __restrict__ w, int rows,
+                                                            int cols, uint8_t* __restrict__ q,
+                                                            uint8_t* __restrict__ qt,
+                                                            float* __restrict__ scale,
+                                                            float* __restrict__ scale_inv) {
+  const int cb = cols >> 7;
+  const int bc = blockIdx.x % cb, br = blockIdx.x / cb;
+  const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
+  const int64_t tile_off = (int64_t)br * 128 * cols + bc * 128 + cg * 8;
+  uint4 v[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p)
+    v[p] = nt_load16(w + tile_off + (int64_t)tile_row(rq, p) * cols);
+  uint32_t m = 0;
+#pragma unroll
+  for (int p = 0; p < 8; ++p) m = umax(m, mag8(v[p]));
+  m = row16_max_u32(m);
+  __shared__ uint32_t part[16];
+  __shared__ float s_scale;
+  if (cg == 0) part[rq] = m;
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    m = row16_max_u32(part[threadIdx.x]);
+    if (threadIdx.x == 0) {
+      float s, si;
+      scales_from_amax(__uint_as_float(m << 16), s, si);
+      s_scale = s;
+      if (scale) scale[blockIdx.x] = s;
+      scale_inv[blockIdx.x] = si;
+    }
+  }
+  __syncthreads();
+  const float s = s_scale;
+  uint2 c[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    c[p] = cvt8(v[p], s);
+    *reinterpret_cast<uint2*>(q + tile_off + (int64_t)tile_row(rq, p) * cols) = c[p];
+  }
+  if (WITH_T) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
+    store_tile_transposed(tile, c, cg, rq, qt + (int64_t)bc * 128 * rows + br * 128, rows);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 128x1 groups, transposed output (wgrad operands): x[M,K] -> qt[K,M], scales [K, M/128]
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int m, int k,
+                                                            uint8_t* __restrict__ qt,
+                                                            float* __restrict__ scale_t,
+                                                            float* __restrict__ scale_inv_t) {
+  const int kb = k >> 7;
+  const int tc = blockIdx.x % kb, tr = blockIdx.x / kb;
+  const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
+  const int mb = m >> 7;
+  const int64_t tile_off = (int64_t)tr * 128 * k + tc * 128 + cg * 8;
+  uint4 v[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p)
+    v[p] = nt_load16(x + tile_off + (int64_t)tile_row(rq, p) * k);
+  // per-column magnitudes over this thread's 8 rows, two columns per word
+  uint32_t cm[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    cm[0] = pk_max_u16(cm[0], v[p].x & 0x7FFF7FFFu);
+    cm[1] = pk_max_u16(cm[1], v[p].y & 0x7FFF7FFFu);
+    cm[2] = pk_max_u16(cm[2], v[p].z & 0x7FFF7FFFu);
+    cm[3] = pk_max_u16(cm[3], v[p].w & 0x7FFF7FFFu);
+  }
+  // across the 4 row quads inside the wave (lanes differing in bits 4 and 5)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 16));
+    cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 32));
+  }
+  __shared__ uint32_t part[4][64];  // [wave][cg*4 + word]
+  __shared__ float s_scale[128];
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) < 16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][cg * 4 + i] = cm[i];
+  }
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    const int col = threadIdx.x, word = col >> 1;
+    uint32_t mw = pk_max_u16(pk_max_u16(part[0][word], part[1][word]), pk_max_u16(part[2][word], part[3][word]));
+    uint32_t mag = (col & 1) ? (mw >> 16) : (mw & 0xFFFFu);
+    float s, si;
+    scales_from_amax(__uint_as_float(mag << 16), s, si);
+    s_scale[col] = s;
+    int64_t o = ((int64_t)tc * 128 + col) * mb + tr;
+    if (scale_t) scale_t[o] = s;
+    scale_inv_t[o] = si;
+  }
+  __syncthreads();
+  float sc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) sc[j] = s_scale[cg * 8 + j];
+  uint2 c[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const uint32_t ws[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
+    uint32_t pk[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float a = clamp448(bf16lo(ws[i]) * sc[2 * i]);
+      float b = clamp448(bf16hi(ws[i]) * sc[2 * i + 1]);
+      pk[i] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
+    }
+    c[p].x = pk[0] | (pk[1] << 16);
+    c[p].y = pk[2] | (pk[3] << 16);
+  }
+  __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
+  store_tile_transposed(tile, c, cg, rq, qt + (int64_t)tc * 128 * m + tr * 128, m);
+}
+
+// ---------------------------------------------------------------------------------------------
+// dequantize 1x128 groups back to bf16 (gradient bucket round trip)
+// ---------------------------------------------------------------------------------------------
+// out = bf16(decode(q) * scale_inv); if grad_scale != 1 the bf16 value is multiplied by it and
+// rounded again, the order of the reference's cast-back site
+// (hyper_parallel/core/hsdp/hsdp_grad_buffer.py:121-125).
+__global__ __launch_bounds__(256) void dequant_1x128_kernel(const uint4* __restrict__ q,
+                                                            const float* __restrict__ scale_inv,
+                                                            uint4* __restrict__ out, int64_t nvec,
+                                                            float grad_scale, int apply_grad_scale) {
+  // nvec counts 16-code vectors; 8 of them per group.  One thread: 16 codes -> 2 x uint4 of bf16.
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  uint4 c = nt_load16(&q[i]);
+  const float si = scale_inv[i >> 3];
+  const uint32_t words[4] = {c.x, c.y, c.z, c.w};
+  uint32_t o[8];
+#pragma unroll
+  for (int wd = 0; wd < 4; ++wd) {
+    v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], false);
+    v2f hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], true);
+    float f[4] = {lo.x * si, lo.y * si, hi.x * si, hi.y * si};
+    __bf16 b[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      b[e] = (__bf16)f[e];
+      if (apply_grad_scale) b[e] = (__bf16)((float)b[e] * grad_scale);
+    }
+    o[2 * wd] = (uint32_t)__builtin_bit_cast(uint16_t, b[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, b[1]) << 16);
+    o[2 * wd + 1] = (uint32_t)__builtin_bit_cast(uint16_t, b[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, b[3]) << 16);
+  }
+  nt_store16(&out[2 * i], make_uint4(o[0], o[1], o[2], o[3]));
+  nt_store16(&out[2 * i + 1], make_uint4(o[4], o[5], o[6], o[7]));
+}
+
+// codes with one scale per 128x128 block (weights) -> bf16
+__global__ __launch_bounds__(256) void dequant_128x128_kernel(const uint8_t* __restrict__ q,
+                                                              const float* __restrict__ scale_inv,
+                                                              uint16_t* __restrict__ out, int rows, int cols) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one 16-code vector
+  const int64_t nvec = (int64_t)rows * cols / 16;
+  if (i >= nvec) return;
+  const int64_t e0 = i * 16;
+  const int r = (int)(e0 / cols), c = (int)(e0 % cols);
+  const float si = scale_inv[(int64_t)(r >> 7) * (cols >> 7) + (c >> 7)];
+  uint4 cd = *reinterpret_cast<const uint4*>(q + e0);
+  const uint32_t words[4] = {cd.x, cd.y, cd.z, cd.w};
+  uint32_t o[8];
+#pragma unroll
+  for (int wd = 0; wd < 4; ++wd) {
+    v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], false);
+    v2f hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], true);
+    __bf16 b0 = (__bf16)(lo.x * si), b1 = (__bf16)(lo.y * si), b2 = (__bf16)(hi.x * si), b3 = (__bf16)(hi.y * si);
+    o[2 * wd] = (uint32_t)__builtin_bit_cast(uint16_t, b0) | ((uint32_t)__builtin_bit_cast(uint16_t, b1) << 16);
+    o[2 * wd + 1] = (uint32_t)__builtin_bit_cast(uint16_t, b2) | ((uint32_t)__builtin_bit_cast(uint16_t, b3) << 16);
+  }
+  uint4* ov = reinterpret_cast<uint4*>(out + e0);
+  ov[0] = make_uint4(o[0], o[1], o[2], o[3]);
+  ov[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
+}  // namespace hpfp8
+
+using namespace hpfp8;
+
+// ---------------------------------------------------------------------------------------------
+// C-ABI
+// ---------------------------------------------------------------------------------------------
+extern "C" {
+
+int hpfp8_amax_bf16(const void* x, int64_t n, float* amax_out, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(n >= 0, HPFP8_ERR_SHAPE, "amax: negative element count");
+  HPFP8_REQUIRE(amax_out != nullptr, HPFP8_ERR_ARG, "amax: null output");
+  HPFP8_REQUIRE(n == 0 || (x && aligned16(x)), HPFP8_ERR_ALIGN, "amax: input must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  fill_u32_kernel<<<1, 64, 0, s>>>(reinterpret_cast<uint32_t*>(amax_out), 0u, 1);
+  if (n > 0) {
+    int64_t nvec = n >> 3;
+    int blocks = (int)((nvec + 256 * 8 - 1) / (256 * 8));
+    if (blocks < 1) blocks = 1;
+    if (blocks > 4096) blocks = 4096;
+    amax_bf16_kernel<<<blocks, 256, 0, s>>>((const uint16_t*)x, n, reinterpret_cast<uint32_t*>(amax_out));
+  }
+  return check_launch("amax");
+}
+
+int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void* q, float* scale,
+                               float* scale_inv, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(n >= 0, HPFP8_ERR_SHAPE, "cast_per_tensor: negative element count");
+  HPFP8_REQUIRE(amax != nullptr, HPFP8_ERR_ARG, "cast_per_tensor: null amax");
+  HPFP8_REQUIRE(n == 0 || (x && q && aligned16(x) && aligned16(q)), HPFP8_ERR_ALIGN,
+                "cast_per_tensor: buffers must be non-null and 16-byte aligned");
+  int64_t nvec = n >> 3;
+  int blocks = (int)((nvec + 256 * 4 - 1) / (256 * 4));
+  if (blocks < 1) blocks = 1;
+  if (blocks > 16384) blocks = 16384;
+  cast_per_tensor_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, n, amax, (uint8_t*)q,
+                                                                  scale, scale_inv);
+  return check_launch("cast_per_tensor");
+}
+
+int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
+                                   float* scale_inv, hpfp8_stream_t stream) {
+  int rc = hpfp8_amax_bf16(x, n, amax, stream);
+  if (rc != HPFP8_OK) return rc;
+  return hpfp8_cast_per_tensor_bf16(x, n, amax, q, scale, scale_inv, stream);
+}
+
+int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                              float* scale_inv, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_1x128: negative shape");
+  HPFP8_REQUIRE(cols % kBlock == 0, HPFP8_ERR_SHAPE, "quantize_1x128: last dim %lld is not a multiple of 128",
+                (long long)cols);
+  const int64_t nvec = rows * cols / 8;
+  if (nvec == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(x && q && scale_inv, HPFP8_ERR_ARG, "quantize_1x128: null buffer");
+  HPFP8_REQUIRE(aligned16(x) && aligned16(q), HPFP8_ERR_ALIGN, "quantize_1x128: buffers must be 16-byte aligned");
+  constexpr int UNROLL = 4;
+  const int64_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "quantize_1x128: tensor too large");
+  quant_1x128_kernel<UNROLL><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+      (const uint4*)x, (uint2*)q, scale, scale_inv, nvec);
+  return check_launch("quantize_1x128");
+}
+
+int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, float* scale,
+                                float* scale_inv, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_128x128: negative shape");
+  HPFP8_REQUIRE(rows % kBlock == 0 && cols % kBlock == 0, HPFP8_ERR_SHAPE,
+                "quantize_128x128: shape [%lld, %lld] is not a multiple of 128", (long long)rows, (long long)cols);
+  HPFP8_REQUIRE(rows < (1 << 30) && cols < (1 << 30), HPFP8_ERR_SHAPE, "quantize_128x128: dimension too large");
+  const int64_t blocks = (rows / kBlock) * (cols / kBlock);
+  if (blocks == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "quantize_128x128: tensor too large");
+  HPFP8_REQUIRE(w && q && scale_inv, HPFP8_ERR_ARG, "quantize_128x128: null buffer");
+  HPFP8_REQUIRE(aligned16(w) && aligned16(q) && (!q_t || aligned16(q_t)), HPFP8_ERR_ALIGN,
+                "quantize_128x128: buffers must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  if (q_t)
+    quant_128x128_kernel<true><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
+                                                                (uint8_t*)q, (uint8_t*)q_t, scale, scale_inv);
+  else
+    quant_128x128_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
+                                                                 (uint8_t*)q, nullptr, scale, scale_inv);
+  return check_launch("quantize_128x128");
+}
+
+int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
+                                float* scale_inv_t, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "quantize_128x1_t: negative shape");
+  HPFP8_REQUIRE(m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE,
+                "quantize_128x1_t: shape [%lld, %lld] is not a multiple of 128", (long long)m, (long long)k);
+  HPFP8_REQUIRE(m < (1 << 30) && k < (1 << 30), HPFP8_ERR_SHAPE, "quantize_128x1_t: dimension too large");
+  const int64_t blocks = (m / kBlock) * (k / kBlock);
+  if (blocks == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "quantize_128x1_t: tensor too large");
+  HPFP8_REQUIRE(x && q_t && scale_inv_t, HPFP8_ERR_ARG, "quantize_128x1_t: null buffer");
+  HPFP8_REQUIRE(aligned16(x) && aligned16(q_t), HPFP8_ERR_ALIGN, "quantize_128x1_t: buffers must be 16-byte aligned");
+  quant_128x1_t_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, (int)m, (int)k,
+                                                                          (uint8_t*)q_t, scale_t, scale_inv_t);
+  return check_launch("quantize_128x1_t");
+}
+
+int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,
+                                float grad_scale, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "dequantize_1x128: negative shape");
+  HPFP8_REQUIRE(cols % kBlock == 0, HPFP8_ERR_SHAPE, "dequantize_1x128: last dim %lld is not a multiple of 128",
+                (long long)cols);
+  const int64_t nvec = rows * cols / 16;
+  if (nvec == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(q && scale_inv && out, HPFP8_ERR_ARG, "dequantize_1x128: null buffer");
+  HPFP8_REQUIRE(aligned16(q) && aligned16(out), HPFP8_ERR_ALIGN, "dequantize_1x128: buffers must be 16-byte aligned");
+  const int64_t blocks = (nvec + 255) / 256;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "dequantize_1x128: tensor too large");
+  dequant_1x128_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+      (const uint4*)q, scale_inv, (uint4*)out, nvec, grad_scale, grad_scale != 1.0f ? 1 : 0);
+  return check_launch("dequantize_1x128");
+}
+
+int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,
+                                  hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "dequantize_128x128: negative shape");
+  HPFP8_REQUIRE(rows % kBlock == 0 && cols % kBlock == 0, HPFP8_ERR_SHAPE,
+                "dequantize_128x128: shape [%lld, %lld] is not a multiple of 128", (long long)rows, (long long)cols);
+  HPFP8_REQUIRE(rows < (1 << 30) && cols < (1 << 30), HPFP8_ERR_SHAPE, "dequantize_128x128: dimension too large");
+  const int64_t nvec = rows * cols / 16;
+  if (nvec == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(q && scale_inv && out, HPFP8_ERR_ARG, "dequantize_128x128: null buffer");
+  HPFP8_REQUIRE(aligned16(q) && aligned16(out), HPFP8_ERR_ALIGN, "dequantize_128x128: buffers must be 16-byte aligned");
+  const int64_t blocks = (nvec + 255) / 256;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "dequantize_128x128: tensor too large");
+  dequant_128x128_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, scale_inv,
+                                                                           (uint16_t*)out, (int)rows, (int)cols);
+  return check_launch("dequantize_128x128");
+}
+
+}  // extern "C"

@@ -1,0 +1,20 @@
+"""hpfp8: MI355X-native FP8 mixed-precision linear path (quantizers, scaled GEMMs, fp8_linear).
+
+Importing the package loads libhpfp8.so; it raises ImportError if the HIP extension is not built.
+"""
+from . import _lib
+
+_lib.load()
+
+from .ops import (amax, quantize_per_tensor, quantize_1x128, quantize_128x128, quantize_128x1_t,  # noqa: E402
+                  dequantize_1x128, dequantize_128x128, gemm_blockwise, gemm_per_tensor,
+                  gemm_grouped_blockwise)
+from .linear import fp8_linear, Fp8Linear, fp8_grouped_linear  # noqa: E402
+from .bucket import quantize_bucket, dequantize_bucket  # noqa: E402
+
+__all__ = [
+    "amax", "quantize_per_tensor", "quantize_1x128", "quantize_128x128", "quantize_128x1_t",
+    "dequantize_1x128", "dequantize_128x128", "gemm_blockwise", "gemm_per_tensor",
+    "gemm_grouped_blockwise", "fp8_linear", "Fp8Linear", "fp8_grouped_linear",
+    "quantize_bucket", "dequantize_bucket",
+]

@@ -1,0 +1,170 @@
+"""FP8 linear with the calling convention of torch.nn.functional.linear.
+
+`fp8_linear(input, weight, bias=None)` is what a model swaps in for `F.linear`: same argument
+order, weight [out_features, in_features], contraction over the last dim of both, output
+`input.shape[:-1] + (out_features,)` in bf16 -- the operator the reference registers in
+hyper_parallel/core/shard/ops/yaml/torch_mm.yaml:6-9 and type-checks in
+hyper_parallel/core/shard/ops/parallel_matmul.py:344-404.  Being a plain function on local
+tensors it also fits `custom_shard(func, ...)` (hyper_parallel/core/shard/local_func.py:26-128).
+
+Recipes
+  "blockwise"  : activations / output gradients 1x128, weights 128x128; wgrad operands are
+                 re-quantized 128x1 (transposed) from the bf16 sources.
+  "per_tensor" : one scale per tensor (amax -> 448/amax); backward also per tensor.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import ops
+
+RECIPES = ("blockwise", "per_tensor")
+
+
+def _flatten(x: torch.Tensor):
+    return x.reshape(-1, x.shape[-1])
+
+
+class _Fp8LinearBlockwise(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        x2 = _flatten(x)
+        xq, sx = ops.quantize_1x128(x2)
+        need_wgrad_inputs = x.requires_grad or weight.requires_grad
+        if x.requires_grad:
+            wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
+        else:
+            wq, sw = ops.quantize_128x128(weight)
+            wqt = None
+        y = ops.gemm_blockwise(xq, sx, wq, sw, bias=bias)
+        ctx.save_for_backward(x2 if weight.requires_grad else None, wqt, sw)
+        ctx.x_shape = x.shape
+        ctx.has_bias = bias is not None
+        ctx.need = (x.requires_grad, weight.requires_grad, need_wgrad_inputs)
+        return y.reshape(x.shape[:-1] + (weight.shape[0],))
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x2, wqt, sw = ctx.saved_tensors
+        need_dx, need_dw, _ = ctx.need
+        go = _flatten(grad_out)
+        if go.dtype != torch.bfloat16:
+            go = go.to(torch.bfloat16)
+        go = go.contiguous()
+        dx = dw = db = None
+        if need_dx:
+            # dx[M,K] = go[M,N] . W[N,K]: contraction over N, b operand = W^T codes [K,N] whose
+            # 128x128 scales are W's with the two strides swapped.
+            goq, sgo = ops.quantize_1x128(go)
+            dx = ops.gemm_blockwise(goq, sgo, wqt, sw.t()).reshape(ctx.x_shape)
+        if need_dw:
+            # dW[N,K] = go^T[N,M] . x[M,K]: contraction over tokens, both operands 1x128 along M
+            m = go.shape[0]
+            if m % ops.BLOCK:
+                raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
+            got, sgot = ops.quantize_128x1_t(go)
+            xt, sxt = ops.quantize_128x1_t(x2)
+            dw = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1)
+        if ctx.has_bias:
+            db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
+        return dx, dw, db
+
+
+class _Fp8LinearPerTensor(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        x2 = _flatten(x)
+        xq, _, sx = ops.quantize_per_tensor(x2)
+        wq, _, sw = ops.quantize_per_tensor(weight)
+        y = ops.gemm_per_tensor(xq, sx, wq, sw, bias=bias)
+        ctx.save_for_backward(x2, weight)
+        ctx.x_shape = x.shape
+        ctx.has_bias = bias is not None
+        ctx.need = (x.requires_grad, weight.requires_grad)
+        return y.reshape(x.shape[:-1] + (weight.shape[0],))
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x2, weight = ctx.saved_tensors
+        need_dx, need_dw = ctx.need
+        go = _flatten(grad_out)
+        if go.dtype != torch.bfloat16:
+            go = go.to(torch.bfloat16)
+        go = go.contiguous()
+        dx = dw = db = None
+        if need_dx:
+            goq, _, sgo = ops.quantize_per_tensor(go)
+            wtq, _, swt = ops.quantize_per_tensor(weight.t().contiguous())
+            dx = ops.gemm_per_tensor(goq, sgo, wtq, swt).reshape(ctx.x_shape)
+        if need_dw:
+            gotq, _, sgot = ops.quantize_per_tensor(go.t().contiguous())
+            xtq, _, sxt = ops.quantize_per_tensor(x2.t().contiguous())
+            dw = ops.gemm_per_tensor(gotq, sgot, xtq, sxt)
+        if ctx.has_bias:
+            db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
+        return dx, dw, db
+
+
+def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
+               recipe: str = "blockwise") -> torch.Tensor:
+    """y = input @ weight.T + bias computed through E4M3 operands with fp32 accumulation.
+
+    input [..., in_features] bf16, weight [out_features, in_features] bf16, bias [out_features] bf16
+    or None; returns bf16 [..., out_features].  in_features and out_features must be multiples of
+    128 (ragged tails are rejected, not padded).
+    """
+    if recipe not in RECIPES:
+        raise ValueError(f"recipe must be one of {RECIPES}, got {recipe!r}")
+    if weight.dim() != 2:
+        raise ValueError("weight must be [out_features, in_features]")
+    if input.shape[-1] != weight.shape[1]:
+        raise ValueError(f"input last dim {input.shape[-1]} != weight in_features {weight.shape[1]}")
+    for name, t in (("input", input), ("weight", weight), ("bias", bias)):
+        if t is not None and t.dtype != torch.bfloat16:
+            raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+    fn = _Fp8LinearBlockwise if recipe == "blockwise" else _Fp8LinearPerTensor
+    return fn.apply(input, weight, bias)
+
+
+class Fp8Linear(nn.Module):
+    """Drop-in for torch.nn.Linear (bf16 parameters) whose matmuls run through fp8_linear."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, *, recipe: str = "blockwise",
+                 device=None, dtype=torch.bfloat16):
+        super().__init__()
+        if recipe not in RECIPES:
+            raise ValueError(f"recipe must be one of {RECIPES}, got {recipe!r}")
+        if in_features % ops.BLOCK or out_features % ops.BLOCK:
+            raise ValueError("in_features and out_features must be multiples of 128")
+        self.in_features, self.out_features, self.recipe = in_features, out_features, recipe
+        self.weight = nn.Parameter(torch.empty((out_features, in_features), device=device, dtype=dtype))
+        self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=dtype)) if bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        ref = nn.Linear(self.in_features, self.out_features, bias=self.bias is not None)
+        with torch.no_grad():
+            self.weight.copy_(ref.weight)
+            if self.bias is not None:
+                self.bias.copy_(ref.bias)
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        return fp8_linear(input, self.weight, self.bias, recipe=self.recipe)
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, "
+                f"bias={self.bias is not None}, recipe={self.recipe}")
+
+
+def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
+    """MoE grouped linear, forward only: rows of input[total_m, K] are sorted by expert, offs[E] are
+    the inclusive int32 prefix sums of rows per expert, weight[E, N, K] -> bf16 [total_m, N]."""
+    if input.dim() != 2 or weight.dim() != 3 or input.shape[1] != weight.shape[2]:
+        raise ValueError("input must be [total_m, K] and weight [E, N, K]")
+    xq, sx = ops.quantize_1x128(input)
+    e, n, k = weight.shape
+    wq, sw = ops.quantize_128x128(weight.reshape(e * n, k))
+    return ops.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), offs)

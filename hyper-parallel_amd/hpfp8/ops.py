@@ -1,0 +1,281 @@
+"""Tensor-level wrappers over the C ABI: quantizers, dequantizers and scaled GEMMs.
+
+All functions take and return torch tensors that live on the GPU; they only check arguments,
+allocate outputs with torch and pass raw pointers plus the current HIP stream to libhpfp8.so.
+Weight tensors are [out_features, in_features] and the contraction runs over the last dim of both
+GEMM operands, the operand roles of the reference's linear operator
+(hyper_parallel/core/shard/ops/parallel_matmul.py:377-381).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+BLOCK = 128
+FP8 = torch.float8_e4m3fn
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _check_bf16(x: torch.Tensor, name: str) -> torch.Tensor:
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not x.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {x.device}); this path has no CPU fallback")
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16, got {x.dtype}")
+    return x if x.is_contiguous() else x.contiguous()
+
+
+def _check_fp8(x: torch.Tensor, name: str) -> torch.Tensor:
+    if not x.is_cuda:
+        raise ValueError(f"{name} must live on the GPU")
+    if x.dtype not in (FP8, torch.uint8):
+        raise TypeError(f"{name} must be float8_e4m3fn (or uint8 codes), got {x.dtype}")
+    if not x.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return x
+
+
+def _check_f32(x: torch.Tensor, name: str) -> torch.Tensor:
+    if not x.is_cuda or x.dtype != torch.float32:
+        raise TypeError(f"{name} must be a float32 GPU tensor")
+    return x
+
+
+# ------------------------------------------------------------------------------------------------
+# quantizers
+# ------------------------------------------------------------------------------------------------
+def amax(x: torch.Tensor) -> torch.Tensor:
+    """max |x| as a 0-dim fp32 tensor."""
+    x = _check_bf16(x, "x")
+    out = torch.empty((), dtype=torch.float32, device=x.device)
+    _lib.call("hpfp8_amax_bf16", _ptr(x), x.numel(), _ptr(out), _stream())
+    return out
+
+
+def quantize_per_tensor(x: torch.Tensor, amax_in: Optional[torch.Tensor] = None
+                        ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One scale for the whole tensor: returns (codes like x, scale, scale_inv).
+
+    scale = 448 / max(amax, 1e-12) and scale_inv = max(amax, 1e-12) / 448 are 0-dim fp32 tensors.
+    With ``amax_in`` (0-dim fp32 GPU tensor) the reduction is skipped and that value is used.
+    """
+    x = _check_bf16(x, "x")
+    q = torch.empty(x.shape, dtype=FP8, device=x.device)
+    scale = torch.empty((), dtype=torch.float32, device=x.device)
+    scale_inv = torch.empty((), dtype=torch.float32, device=x.device)
+    if amax_in is None:
+        am = torch.empty((), dtype=torch.float32, device=x.device)
+        _lib.call("hpfp8_quantize_per_tensor_bf16", _ptr(x), x.numel(), _ptr(q), _ptr(am), _ptr(scale),
+                  _ptr(scale_inv), _stream())
+    else:
+        am = _check_f32(amax_in, "amax_in")
+        _lib.call("hpfp8_cast_per_tensor_bf16", _ptr(x), x.numel(), _ptr(am), _ptr(q), _ptr(scale),
+                  _ptr(scale_inv), _stream())
+    return q, scale, scale_inv
+
+
+def quantize_1x128(x: torch.Tensor, want_scale: bool = False):
+    """x[..., C] -> (codes, scale_inv[..., C/128]) (plus scale when ``want_scale``)."""
+    x = _check_bf16(x, "x")
+    if x.dim() < 1:
+        raise ValueError("x must have at least one dimension")
+    cols = x.shape[-1]
+    if cols % BLOCK:
+        raise ValueError(f"last dim {cols} is not a multiple of {BLOCK}")
+    rows = x.numel() // cols if cols else 0
+    q = torch.empty(x.shape, dtype=FP8, device=x.device)
+    sshape = x.shape[:-1] + (cols // BLOCK,)
+    scale_inv = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    scale = torch.empty(sshape, dtype=torch.float32, device=x.device) if want_scale else None
+    _lib.call("hpfp8_quantize_1x128_bf16", _ptr(x), rows, cols, _ptr(q), _ptr(scale), _ptr(scale_inv), _stream())
+    return (q, scale, scale_inv) if want_scale else (q, scale_inv)
+
+
+def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: bool = False):
+    """w[R, C] -> (codes[R, C], scale_inv[R/128, C/128]) (+ codes_t[C, R]) (+ scale)."""
+    w = _check_bf16(w, "w")
+    if w.dim() != 2:
+        raise ValueError("w must be 2-D")
+    r, c = w.shape
+    if r % BLOCK or c % BLOCK:
+        raise ValueError(f"shape {tuple(w.shape)} is not a multiple of {BLOCK} in both dims")
+    q = torch.empty((r, c), dtype=FP8, device=w.device)
+    qt = torch.empty((c, r), dtype=FP8, device=w.device) if with_transpose else None
+    scale_inv = torch.empty((r // BLOCK, c // BLOCK), dtype=torch.float32, device=w.device)
+    scale = torch.empty_like(scale_inv) if want_scale else None
+    _lib.call("hpfp8_quantize_128x128_bf16", _ptr(w), r, c, _ptr(q), _ptr(qt), _ptr(scale), _ptr(scale_inv),
+              _stream())
+    out = (q, scale_inv)
+    if with_transpose:
+        out += (qt,)
+    if want_scale:
+        out += (scale,)
+    return out
+
+
+def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False):
+    """Transposed re-quantization for wgrad from the bf16 source.
+
+    x[M, K] -> (codes_t[K, M], scale_inv_t[K, M/128]); one scale per 128 consecutive rows of a column.
+    """
+    x = _check_bf16(x, "x")
+    if x.dim() != 2:
+        raise ValueError("x must be 2-D")
+    m, k = x.shape
+    if m % BLOCK or k % BLOCK:
+        raise ValueError(f"shape {tuple(x.shape)} is not a multiple of {BLOCK} in both dims")
+    qt = torch.empty((k, m), dtype=FP8, device=x.device)
+    scale_inv = torch.empty((k, m // BLOCK), dtype=torch.float32, device=x.device)
+    scale = torch.empty_like(scale_inv) if want_scale else None
+    _lib.call("hpfp8_quantize_128x1_t_bf16", _ptr(x), m, k, _ptr(qt), _ptr(scale), _ptr(scale_inv), _stream())
+    return (qt, scale, scale_inv) if want_scale else (qt, scale_inv)
+
+
+def dequantize_1x128(q: torch.Tensor, scale_inv: torch.Tensor, grad_scale: float = 1.0) -> torch.Tensor:
+    """codes[..., C] with scale_inv[..., C/128] -> bf16."""
+    q = _check_fp8(q, "q")
+    scale_inv = _check_f32(scale_inv, "scale_inv")
+    cols = q.shape[-1]
+    if cols % BLOCK:
+        raise ValueError(f"last dim {cols} is not a multiple of {BLOCK}")
+    rows = q.numel() // cols if cols else 0
+    if scale_inv.numel() != rows * (cols // BLOCK) or not scale_inv.is_contiguous():
+        raise ValueError("scale_inv must be contiguous with one entry per 128 codes")
+    out = torch.empty(q.shape, dtype=torch.bfloat16, device=q.device)
+    _lib.call("hpfp8_dequantize_1x128_bf16", _ptr(q), _ptr(scale_inv), rows, cols, _ptr(out), float(grad_scale),
+              _stream())
+    return out
+
+
+def dequantize_128x128(q: torch.Tensor, scale_inv: torch.Tensor) -> torch.Tensor:
+    q = _check_fp8(q, "q")
+    scale_inv = _check_f32(scale_inv, "scale_inv")
+    r, c = q.shape
+    if r % BLOCK or c % BLOCK:
+        raise ValueError(f"shape {tuple(q.shape)} is not a multiple of {BLOCK} in both dims")
+    if tuple(scale_inv.shape) != (r // BLOCK, c // BLOCK) or not scale_inv.is_contiguous():
+        raise ValueError("scale_inv must be contiguous [R/128, C/128]")
+    out = torch.empty((r, c), dtype=torch.bfloat16, device=q.device)
+    _lib.call("hpfp8_dequantize_128x128_bf16", _ptr(q), _ptr(scale_inv), r, c, _ptr(out), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# GEMMs
+# ------------------------------------------------------------------------------------------------
+def _out_code(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return _lib.OUT_BF16
+    if dtype == torch.float32:
+        return _lib.OUT_F32
+    raise TypeError(f"out_dtype must be bfloat16 or float32, got {dtype}")
+
+
+def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor,
+                   bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16,
+                   sb_gran: int = 128, out: Optional[torch.Tensor] = None, accumulate: bool = False
+                   ) -> torch.Tensor:
+    """c[M,N] = sum_kb sa[m,kb] * sb[n//sb_gran, kb] * (a[m, kb] . b[n, kb]) (+ bias).
+
+    a[M,K], b[N,K] codes; sa, sb 2-D fp32 views (any strides) of scale_inv values.
+    """
+    a = _check_fp8(a, "a")
+    b = _check_fp8(b, "b")
+    sa = _check_f32(sa, "sa")
+    sb = _check_f32(sb, "sb")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"a {tuple(a.shape)} and b {tuple(b.shape)} must be 2-D with equal last dim")
+    m, k = a.shape
+    n = b.shape[0]
+    if k % BLOCK or n % BLOCK or k == 0:
+        raise ValueError(f"K={k} must be a positive multiple of 128 and N={n} a multiple of 128")
+    kb = k // BLOCK
+    if tuple(sa.shape) != (m, kb):
+        raise ValueError(f"sa must be [{m}, {kb}], got {tuple(sa.shape)}")
+    want_sb = (n // BLOCK, kb) if sb_gran == 128 else (n, kb)
+    if sb_gran not in (1, 128) or tuple(sb.shape) != want_sb:
+        raise ValueError(f"sb must be {list(want_sb)} for sb_gran={sb_gran}, got {tuple(sb.shape)}")
+    if bias is not None:
+        bias = _check_bf16(bias, "bias")
+        if tuple(bias.shape) != (n,):
+            raise ValueError(f"bias must be [{n}]")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs an existing `out`")
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    else:
+        if tuple(out.shape) != (m, n) or out.stride(1) != 1 or not out.is_cuda:
+            raise ValueError("out must be a GPU tensor [M, N] with unit inner stride")
+        out_dtype = out.dtype
+    if accumulate and out_dtype != torch.float32:
+        raise ValueError("accumulate needs a float32 output")
+    _lib.call("hpfp8_gemm_blockwise", _ptr(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
+              sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
+              out.stride(0) if m > 1 else n, _out_code(out_dtype), int(accumulate), _stream())
+    return out
+
+
+def gemm_per_tensor(a: torch.Tensor, sa_inv: torch.Tensor, b: torch.Tensor, sb_inv: torch.Tensor,
+                    bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """c = (a . b^T) * (sa_inv * sb_inv) (+ bias); sa_inv / sb_inv are 0-dim (or 1-element) fp32."""
+    a = _check_fp8(a, "a")
+    b = _check_fp8(b, "b")
+    sa_inv = _check_f32(sa_inv, "sa_inv")
+    sb_inv = _check_f32(sb_inv, "sb_inv")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"a {tuple(a.shape)} and b {tuple(b.shape)} must be 2-D with equal last dim")
+    if sa_inv.numel() != 1 or sb_inv.numel() != 1:
+        raise ValueError("per-tensor scales must have exactly one element")
+    m, k = a.shape
+    n = b.shape[0]
+    if k % BLOCK or n % BLOCK or k == 0:
+        raise ValueError(f"K={k} must be a positive multiple of 128 and N={n} a multiple of 128")
+    if bias is not None:
+        bias = _check_bf16(bias, "bias")
+        if tuple(bias.shape) != (n,):
+            raise ValueError(f"bias must be [{n}]")
+    out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    _lib.call("hpfp8_gemm_per_tensor", _ptr(a), _ptr(sa_inv), _ptr(b), _ptr(sb_inv), m, n, k, _ptr(bias),
+              _ptr(out), n, _out_code(out_dtype), _stream())
+    return out
+
+
+def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor,
+                           offs: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """MoE grouped GEMM: rows of a[total_m, K] sorted by expert, offs[E] int32 inclusive prefix sums,
+    b[E, N, K], sb[E, N/128, K/128], sa[total_m, K/128] -> c[total_m, N].  Rows past offs[-1] are left
+    uninitialised (as torch's grouped matmul leaves them)."""
+    a = _check_fp8(a, "a")
+    b = _check_fp8(b, "b")
+    sa = _check_f32(sa, "sa")
+    sb = _check_f32(sb, "sb")
+    if a.dim() != 2 or b.dim() != 3 or a.shape[1] != b.shape[2]:
+        raise ValueError(f"a {tuple(a.shape)} must be [total_m, K] and b {tuple(b.shape)} [E, N, K]")
+    if not offs.is_cuda or offs.dtype != torch.int32 or offs.dim() != 1 or not offs.is_contiguous():
+        raise TypeError("offs must be a contiguous 1-D int32 GPU tensor")
+    total_m, k = a.shape
+    e, n, _ = b.shape
+    if offs.numel() != e:
+        raise ValueError(f"offs must have {e} entries")
+    if k % BLOCK or n % BLOCK or k == 0:
+        raise ValueError(f"K={k} must be a positive multiple of 128 and N={n} a multiple of 128")
+    kb = k // BLOCK
+    if tuple(sa.shape) != (total_m, kb) or not sa.is_contiguous():
+        raise ValueError(f"sa must be contiguous [{total_m}, {kb}]")
+    if tuple(sb.shape) != (e, n // BLOCK, kb) or not sb.is_contiguous():
+        raise ValueError(f"sb must be contiguous [{e}, {n // BLOCK}, {kb}]")
+    out = torch.empty((total_m, n), dtype=out_dtype, device=a.device)
+    _lib.call("hpfp8_gemm_grouped_blockwise", _ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(offs), e, total_m, n, k,
+              _ptr(out), n, _out_code(out_dtype), _stream())
+    return out

@@ -1,0 +1,137 @@
+/* hpfp8 -- C ABI of the MI355X (gfx950) FP8 mixed-precision linear path.
+ *
+ * Every entry point takes raw DEVICE pointers, sizes and a HIP stream, enqueues its kernels on
+ * that stream and returns without synchronizing.  Return value: HPFP8_OK (0) or a negative
+ * HPFP8_ERR_* code; hpfp8_last_error() then gives a human-readable message for the calling
+ * thread.  No exception crosses this boundary and no entry point allocates device memory.
+ *
+ * Data conventions
+ *   bf16 tensors   : uint16 bit patterns, row-major, 16-byte aligned base
+ *   E4M3 codes     : uint8 (OCP E4M3FN: bias 7, max 448, NaN = S.1111.111, no Inf)
+ *   scale          : fp32, quantize multiplier   448 / max(amax, 1e-12)
+ *   scale_inv      : fp32, dequantize multiplier max(amax, 1e-12) / 448   (what the GEMMs consume)
+ *   code           : e4m3_rne(clamp(float(x) * scale, -448, 448))
+ *
+ * What each entry point stands in for.  The reference (mindspore-ai/hyper-parallel) has no FP8
+ * kernels and no C/FFI boundary on its torch platform: a linear there is aten::linear called at
+ * hyper_parallel/core/shard/_op_dispatch.py:277-283 with the operand roles checked in
+ * hyper_parallel/core/shard/ops/parallel_matmul.py:344-404 (weight [out, in], contraction over
+ * the last dim of both), its backward is torch autograd of that op, and the gradient bucket
+ * cast sites are hyper_parallel/core/hsdp/hsdp_grad_buffer.py:95-108 (cast in) and :116-135
+ * (cast back, then * grad_scale).  Each declaration below names the site it replaces.
+ */
+#ifndef HPFP8_H_
+#define HPFP8_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* hpfp8_stream_t; /* a hipStream_t; NULL is the default stream */
+
+enum {
+  HPFP8_OK = 0,
+  HPFP8_ERR_ARG = -1,    /* null pointer / bad flag */
+  HPFP8_ERR_SHAPE = -2,  /* shape not supported (not a multiple of 128, too large, negative) */
+  HPFP8_ERR_ALIGN = -3,  /* pointer not 16-byte aligned */
+  HPFP8_ERR_LAUNCH = -4, /* HIP reported a launch error */
+  HPFP8_ERR_DEVICE = -5  /* not a gfx950 device */
+};
+
+/* Output element type of the GEMMs. */
+enum { HPFP8_OUT_BF16 = 0, HPFP8_OUT_F32 = 1 };
+
+/* Library version (major*10000 + minor*100 + patch). */
+int hpfp8_version(void);
+/* Message of the last failing call made by this thread ("" if none). */
+const char* hpfp8_last_error(void);
+/* HPFP8_OK if the current HIP device is gfx950. */
+int hpfp8_check_device(void);
+
+/* ---- amax and per-tensor cast ----------------------------------------------------------------
+ * Stand in for the dtype cast hooks of the torch platform, TorchPlatform.cast_fp_tensor
+ * (hyper_parallel/platform/torch/platform.py:587-597), for the FP8 target type that hook cannot
+ * express (a cast plus a scale). */
+
+/* amax_out[0] = max |x[i]| as fp32 over n bf16 values (0 for n == 0). */
+int hpfp8_amax_bf16(const void* x, int64_t n, float* amax_out, hpfp8_stream_t stream);
+
+/* q[i] = code(x[i]) with the scale derived on the device from amax[0]; scale / scale_inv
+ * (each may be NULL) receive the two multipliers. */
+int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void* q, float* scale,
+                               float* scale_inv, hpfp8_stream_t stream);
+
+/* amax followed by cast: amax (fp32[1], required) is written then consumed. */
+int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
+                                   float* scale_inv, hpfp8_stream_t stream);
+
+/* ---- blockwise quantizers --------------------------------------------------------------------
+ * Operand preparation for the linear of hyper_parallel/core/shard/_op_dispatch.py:277-283. */
+
+/* Activations / gradient buckets: x[rows, cols] bf16, one scale per 128 contiguous values.
+ * q[rows, cols]; scale (may be NULL) and scale_inv are [rows, cols/128]. */
+int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                              float* scale_inv, hpfp8_stream_t stream);
+
+/* Weights: w[rows, cols] bf16, one scale per 128x128 block.  q[rows, cols]; q_t (may be NULL)
+ * receives the transposed codes [cols, rows] that dgrad consumes; scale (may be NULL) and
+ * scale_inv are [rows/128, cols/128]. */
+int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t,
+                                float* scale, float* scale_inv, hpfp8_stream_t stream);
+
+/* wgrad operands: x[m, k] bf16, one scale per 128 consecutive ROWS of a column, written
+ * transposed: q_t[k, m]; scale_t (may be NULL) and scale_inv_t are [k, m/128]. */
+int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
+                                float* scale_inv_t, hpfp8_stream_t stream);
+
+/* ---- dequantizers ----------------------------------------------------------------------------
+ * The cast-back site hyper_parallel/core/hsdp/hsdp_grad_buffer.py:116-125: out = bf16(decode(q)
+ * * scale_inv); when grad_scale != 1 the bf16 result is multiplied by it and rounded again. */
+int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
+                                void* out, float grad_scale, hpfp8_stream_t stream);
+int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
+                                  void* out, hpfp8_stream_t stream);
+
+/* ---- scaled FP8 GEMMs -------------------------------------------------------------------------
+ * Replace aten::linear (forward) and its autograd backward (dgrad, wgrad) as called from
+ * hyper_parallel/core/shard/_op_dispatch.py:277-283.
+ *
+ *   c[m, n] = sum_kb  sa(m, kb) * sb(n, kb) * ( sum_{k in block kb} a[m, k] * b[n, k] )  (+ bias[n])
+ *
+ * a[M, K] and b[N, K] are E4M3 codes with K contiguous (K, N multiples of 128); fp32
+ * accumulation, k-blocks ascending; one rounding to bf16 at the end (or fp32 output).
+ *   sa(m, kb) = sa[m * sa_stride_m + kb * sa_stride_k]
+ *   sb(n, kb) = sb[(n / sb_gran) * sb_stride_n + kb * sb_stride_k],  sb_gran = 128 or 1
+ * Uses:  forward  a = x codes (1x128),  b = W codes (128x128),            sb_gran = 128
+ *        dgrad    a = grad_out codes,   b = W^T codes, W's scales with swapped strides
+ *        wgrad    a = grad_out^T codes (128x1 requant), b = x^T codes,    sb_gran = 1
+ * bias: bf16[N] or NULL.  out_type HPFP8_OUT_BF16 / HPFP8_OUT_F32; ldc = row stride of c in
+ * elements.  accumulate != 0 (fp32 output only) adds into c instead of overwriting it, the fp32
+ * main-grad bookkeeping of hyper_parallel/platform/torch/fully_shard/param.py:134-167. */
+int hpfp8_gemm_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                         const void* b, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+                         int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
+                         int64_t ldc, int out_type, int accumulate, hpfp8_stream_t stream);
+
+/* Per-tensor scales: c = (a . b^T) * (sa_inv[0] * sb_inv[0]) (+ bias), accumulation over the whole
+ * K inside the matrix cores.  K a multiple of 128, N a multiple of 128. */
+int hpfp8_gemm_per_tensor(const void* a, const float* sa_inv, const void* b, const float* sb_inv,
+                          int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
+                          int out_type, hpfp8_stream_t stream);
+
+/* MoE grouped form (one rank's local experts; no counterpart in the reference, whose expert
+ * parallelism is unimplemented): rows of a[total_m, K] are sorted by expert; offs[e] (int32,
+ * device) is the inclusive prefix sum of per-expert row counts, a count may be 0, rows past
+ * offs[experts-1] are left untouched; b[experts, N, K]; sb[experts, N/128, K/128];
+ * sa[total_m, K/128]; c[total_m, N] bf16 or fp32. */
+int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, const void* b, const float* sb,
+                                 const int32_t* offs, int experts, int64_t total_m, int64_t N,
+                                 int64_t K, void* c, int64_t ldc, int out_type,
+                                 hpfp8_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HPFP8_H_ */

@@ -1,0 +1,326 @@
+"""CPU oracle for the FP8 mixed-precision linear path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing that ships may import this module: only tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py use it, and only as the checker.
+
+What it restates
+----------------
+The reference checkout (mindspore-ai/hyper-parallel) holds no FP8 arithmetic, so there is no
+reference quantizer or scaled GEMM to follow line by line.  The oracle therefore restates
+
+  * the numeric recipe the benchmark configuration text fixes ("amax->scale=448/amax, cast,
+    GEMM with fp32 accumulation, bf16 out"; "1x128 activation scales", "128x128 block scales",
+    "128x1 transposed requant", "1x128 group scales to E4M3 + fp32 scales"), and
+  * the calling conventions of the reference call sites the FP8 path slots into:
+      - linear operand roles, weight [out, in], contraction over the last dim of both:
+        hyper_parallel/core/shard/ops/parallel_matmul.py:377-381
+      - flat gradient bucket, cast -> (reduce) -> cast back -> * grad_scale:
+        hyper_parallel/core/hsdp/hsdp_grad_buffer.py:95-108 and :116-135
+
+Numeric conventions (all fp32, IEEE, round-to-nearest-even, denormals kept):
+  amax      = max(|x|) with x promoted bf16 -> fp32 (exact, order free)
+  amax_c    = max(amax, 1e-12f)
+  scale     = 448.0f / amax_c          (quantize multiplier, one correctly rounded division)
+  scale_inv = amax_c / 448.0f          (dequantize / GEMM-epilogue multiplier, one division)
+  code      = e4m3fn_rne( clamp(float(x) * scale, -448, 448) )
+  dequant   = bf16_rne( decode(code) * scale_inv )
+  gemm      = sum over 128-wide k-blocks, ascending, of
+              (sum_k decode(a)*decode(b)) * (sa_inv * sb_inv); bias added in fp32; one final
+              rounding to bf16.
+Inputs are required to be finite; NaN/Inf behaviour is left unspecified.
+
+How each function is pinned (tests/test_oracle_pins.py)
+-------------------------------------------------------
+  e4m3_decode / e4m3_encode : closed form of the OCP 8-bit format (1-4-3, bias 7, max 448,
+      NaN = S.1111.111, subnormals k*2^-9) checked against torch's float8_e4m3fn cast for all
+      256 codes, all 65536 bf16 bit patterns, every rounding midpoint and its fp32
+      neighbours, and a hand-written known-answer table.
+  amax, scales              : brute force on tiny inputs; special cases amax = 0 and
+      amax < 448/FLT_MAX.
+  quantize_*                : each blocked variant equals the per-tensor quantizer applied to
+      every block separately (pure-Python loops on small shapes); the transposed variant
+      equals quantize_1x128(x.T); the C restatement (fp8_oracle.c) is a second independent
+      implementation compared bit for bit.
+  gemm_*                    : torch._scaled_mm on CPU for per-tensor scales (library routine);
+      exact integer-valued inputs with unit scales reduce to an exact integer matmul; the
+      grouped variant equals a loop of dense calls; float64 dequant matmul bounds the rest.
+No function here is "parity unpinned" in the mathematical sense; what IS unpinned is parity
+with the reference, because the reference has no FP8 code to compare with.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+FP8_MAX = np.float32(448.0)
+AMAX_EPS = np.float32(1e-12)
+BLOCK = 128
+
+__all__ = [
+    "FP8_MAX", "AMAX_EPS", "BLOCK",
+    "bf16_bits_to_f32", "f32_to_bf16_bits", "e4m3_decode", "e4m3_encode",
+    "amax", "scales_from_amax", "quantize_per_tensor", "quantize_1x128",
+    "quantize_128x128", "quantize_128x1_t", "dequantize_per_tensor", "dequantize_1x128",
+    "dequantize_128x128", "quantize_bucket", "dequantize_bucket",
+    "gemm_per_tensor", "gemm_blockwise", "gemm_rowwise_both", "gemm_grouped_blockwise",
+    "gemm_dequant_f64",
+]
+
+
+# --------------------------------------------------------------------------------------
+# bf16 <-> fp32 (bit level).  Tensors travel as uint16 bit patterns so numpy can hold them.
+# --------------------------------------------------------------------------------------
+def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    """bf16 bit patterns (uint16) -> fp32 values; exact (bf16 is the top half of fp32)."""
+    bits = np.ascontiguousarray(bits, dtype=np.uint16)
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit patterns, round-to-nearest-even; NaN stays NaN (quiet bit forced)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    rounded = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    is_nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    nan_bits = (u >> np.uint32(16)) | np.uint32(0x0040)
+    return np.where(is_nan, nan_bits, rounded).astype(np.uint16)
+
+
+# --------------------------------------------------------------------------------------
+# E4M3FN: sign(1) exponent(4, bias 7) mantissa(3).  No Inf.  0x7F / 0xFF are NaN.
+# --------------------------------------------------------------------------------------
+def e4m3_decode(codes: np.ndarray) -> np.ndarray:
+    """uint8 E4M3FN codes -> fp32 values (exact)."""
+    c = np.ascontiguousarray(codes, dtype=np.uint8).astype(np.int32)
+    sign = np.where(c & 0x80, np.float32(-1.0), np.float32(1.0))
+    e = (c >> 3) & 0xF
+    m = c & 0x7
+    normal = np.ldexp((8 + m).astype(np.float32), e - 10)      # (1 + m/8) * 2^(e-7)
+    subnormal = np.ldexp(m.astype(np.float32), -9)               # m * 2^-9
+    mag = np.where(e == 0, subnormal, normal).astype(np.float32)
+    out = (sign * mag).astype(np.float32)
+    out = np.where((c & 0x7F) == 0x7F, np.float32(np.nan), out)
+    return out.astype(np.float32)
+
+
+def e4m3_encode(x: np.ndarray) -> np.ndarray:
+    """fp32 -> E4M3FN code, round-to-nearest-even, NOT saturating.
+
+    |x| that rounds above 448 (i.e. |x| >= 464) and NaN give the NaN code 0x7F | sign, the
+    behaviour of torch's float8_e4m3fn cast.  Callers clamp to +-448 first.
+    """
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    sign = ((u >> np.uint32(24)) & np.uint32(0x80)).astype(np.uint32)
+    a = u & np.uint32(0x7FFFFFFF)
+    # normal target range |x| >= 2^-6: drop 20 mantissa bits with RNE, rebias 127 -> 7
+    lsb = (a >> np.uint32(20)) & np.uint32(1)
+    r = (a + np.uint32(0x7FFFF) + lsb) >> np.uint32(20)
+    normal_code = r.astype(np.int64) - ((127 - 7) << 3)
+    # subnormal target range |x| < 2^-6: code = rne(|x| * 2^9); 8 lands on the first normal
+    small = a < np.uint32(0x3C800000)                                   # |x| < 2^-6
+    mag = np.where(small, a, np.uint32(0)).view(np.float32).astype(np.float64)
+    sub_code = np.rint(mag * 512.0).astype(np.int64)
+    code = np.where(small, sub_code, normal_code)
+    overflow = (code > 0x7E) | (a > np.uint32(0x7F800000)) | (a == np.uint32(0x7F800000))
+    code = np.where(overflow, 0x7F, code).astype(np.uint32)
+    return (code | sign).astype(np.uint8)
+
+
+# --------------------------------------------------------------------------------------
+# amax / scales
+# --------------------------------------------------------------------------------------
+def amax(x_f32: np.ndarray, axis=None, keepdims=False) -> np.ndarray:
+    """max |x| in fp32."""
+    return np.max(np.abs(np.asarray(x_f32, dtype=np.float32)), axis=axis,
+                  keepdims=keepdims).astype(np.float32)
+
+
+def scales_from_amax(am: np.ndarray):
+    """amax -> (scale, scale_inv), two independent correctly rounded fp32 divisions."""
+    am = np.asarray(am, dtype=np.float32)
+    amc = np.maximum(am, AMAX_EPS).astype(np.float32)
+    with np.errstate(over="ignore"):
+        scale = (FP8_MAX / amc).astype(np.float32)
+        scale_inv = (amc / FP8_MAX).astype(np.float32)
+    return scale, scale_inv
+
+
+def _cast(x_f32: np.ndarray, scale: np.ndarray) -> np.ndarray:
+    y = (np.asarray(x_f32, dtype=np.float32) * np.asarray(scale, dtype=np.float32)).astype(np.float32)
+    y = np.clip(y, -FP8_MAX, FP8_MAX).astype(np.float32)
+    return e4m3_encode(y)
+
+
+# --------------------------------------------------------------------------------------
+# quantizers.  x_bits are bf16 bit patterns (uint16) unless stated otherwise.
+# --------------------------------------------------------------------------------------
+def quantize_per_tensor(x_bits: np.ndarray):
+    """One scale for the whole tensor.  Returns (codes u8 like x, scale f32[()], scale_inv)."""
+    x = bf16_bits_to_f32(x_bits)
+    am = amax(x) if x.size else np.float32(0.0)
+    scale, scale_inv = scales_from_amax(am)
+    return _cast(x, scale).reshape(x.shape), scale, scale_inv
+
+
+def quantize_1x128(x_bits: np.ndarray):
+    """Row-wise groups of 128 along the last (contraction) dim.
+
+    x[R, C], C % 128 == 0 -> codes[R, C], scale[R, C/128], scale_inv[R, C/128].
+    """
+    x = bf16_bits_to_f32(x_bits)
+    r, c = x.shape
+    if c % BLOCK:
+        raise ValueError(f"last dim {c} is not a multiple of {BLOCK}")
+    g = x.reshape(r, c // BLOCK, BLOCK)
+    am = amax(g, axis=2) if g.size else np.zeros((r, c // BLOCK), np.float32)
+    scale, scale_inv = scales_from_amax(am)
+    codes = _cast(g, scale[:, :, None]).reshape(r, c)
+    return codes, scale, scale_inv
+
+
+def quantize_128x128(w_bits: np.ndarray):
+    """128x128 blocks.  w[R, C] (both % 128 == 0) -> codes[R, C], scale/scale_inv[R/128, C/128]."""
+    w = bf16_bits_to_f32(w_bits)
+    r, c = w.shape
+    if r % BLOCK or c % BLOCK:
+        raise ValueError(f"shape {w.shape} is not a multiple of {BLOCK} in both dims")
+    g = w.reshape(r // BLOCK, BLOCK, c // BLOCK, BLOCK)
+    am = amax(g, axis=(1, 3)) if g.size else np.zeros((r // BLOCK, c // BLOCK), np.float32)
+    scale, scale_inv = scales_from_amax(am)
+    codes = _cast(g, scale[:, None, :, None]).reshape(r, c)
+    return codes, scale, scale_inv
+
+
+def quantize_128x1_t(x_bits: np.ndarray):
+    """Transposed re-quantization for wgrad, always from the bf16 source.
+
+    x[M, K] (M % 128 == 0) -> codes_t[K, M], scale_t/scale_inv_t[K, M/128], where each scale
+    covers 128 consecutive rows of one column of x.
+    """
+    x = bf16_bits_to_f32(x_bits)
+    m, k = x.shape
+    if m % BLOCK:
+        raise ValueError(f"row count {m} is not a multiple of {BLOCK}")
+    g = x.reshape(m // BLOCK, BLOCK, k)
+    am = amax(g, axis=1) if g.size else np.zeros((m // BLOCK, k), np.float32)   # [M/128, K]
+    scale, scale_inv = scales_from_amax(am)
+    codes = _cast(g, scale[:, None, :]).reshape(m, k)
+    return (np.ascontiguousarray(codes.T), np.ascontiguousarray(scale.T),
+            np.ascontiguousarray(scale_inv.T))
+
+
+def _to_bf16_bits_product(vals_f32: np.ndarray, mult: np.ndarray) -> np.ndarray:
+    return f32_to_bf16_bits((vals_f32 * np.asarray(mult, np.float32)).astype(np.float32))
+
+
+def dequantize_per_tensor(codes: np.ndarray, scale_inv) -> np.ndarray:
+    """codes * scale_inv -> bf16 bit patterns."""
+    return _to_bf16_bits_product(e4m3_decode(codes), np.float32(scale_inv)).reshape(codes.shape)
+
+
+def dequantize_1x128(codes: np.ndarray, scale_inv: np.ndarray) -> np.ndarray:
+    r, c = codes.shape
+    v = e4m3_decode(codes).reshape(r, c // BLOCK, BLOCK)
+    return _to_bf16_bits_product(v, scale_inv[:, :, None]).reshape(r, c)
+
+
+def dequantize_128x128(codes: np.ndarray, scale_inv: np.ndarray) -> np.ndarray:
+    r, c = codes.shape
+    v = e4m3_decode(codes).reshape(r // BLOCK, BLOCK, c // BLOCK, BLOCK)
+    return _to_bf16_bits_product(v, scale_inv[:, None, :, None]).reshape(r, c)
+
+
+def quantize_bucket(flat_bits: np.ndarray):
+    """Flat gradient bucket (1-D, numel % 128 == 0) -> codes[numel], scale_inv[numel/128].
+
+    Same arithmetic as quantize_1x128 on view(-1, 128); the flat contiguous layout is the one
+    the reference packs gradients into (hyper_parallel/core/hsdp/hsdp_grad_buffer.py:95-108).
+    """
+    flat_bits = np.asarray(flat_bits)
+    if flat_bits.ndim != 1 or flat_bits.size % BLOCK:
+        raise ValueError("bucket must be 1-D with numel a multiple of 128")
+    codes, scale, scale_inv = quantize_1x128(flat_bits.reshape(-1, BLOCK))
+    return codes.reshape(-1), scale.reshape(-1), scale_inv.reshape(-1)
+
+
+def dequantize_bucket(codes: np.ndarray, scale_inv: np.ndarray, grad_scale: float = 1.0) -> np.ndarray:
+    """Bucket back to bf16 bits; then `* grad_scale` in bf16 as the reference's cast-back site
+    does (hsdp_grad_buffer.py:121-125: buffer.to(dtype) first, then buffer * grad_scale)."""
+    bits = dequantize_1x128(codes.reshape(-1, BLOCK), scale_inv.reshape(-1, 1)).reshape(-1)
+    if grad_scale != 1.0:
+        v = (bf16_bits_to_f32(bits) * np.float32(grad_scale)).astype(np.float32)
+        bits = f32_to_bf16_bits(v)
+    return bits
+
+
+# --------------------------------------------------------------------------------------
+# GEMMs.  All return fp32 [M, N] before the final rounding plus the bf16 bit patterns.
+# a: codes [M, K]; b: codes [N, K]  (weight layout [out, in], contraction on the last dim of
+# both, hyper_parallel/core/shard/ops/parallel_matmul.py:377-381).
+# --------------------------------------------------------------------------------------
+def _finish(acc_f32: np.ndarray, bias_f32):
+    if bias_f32 is not None:
+        acc_f32 = (acc_f32 + np.asarray(bias_f32, np.float32)[None, :]).astype(np.float32)
+    return acc_f32, f32_to_bf16_bits(acc_f32)
+
+
+def gemm_per_tensor(a, sa_inv, b, sb_inv, bias_f32=None):
+    """y = (A . B^T) * (sa_inv * sb_inv); fp32 accumulation over the whole K."""
+    av, bv = e4m3_decode(a), e4m3_decode(b)
+    acc = (av @ bv.T).astype(np.float32)
+    s = np.float32(np.float32(sa_inv) * np.float32(sb_inv))
+    return _finish((acc * s).astype(np.float32), bias_f32)
+
+
+def gemm_blockwise(a, sa_inv, b, sb_inv, bias_f32=None):
+    """a[M,K] with sa_inv[M,K/128]; b[N,K] with sb_inv[N/128,K/128]."""
+    m, k = a.shape
+    n = b.shape[0]
+    av, bv = e4m3_decode(a), e4m3_decode(b)
+    acc = np.zeros((m, n), np.float32)
+    sb_rows = np.repeat(sb_inv, BLOCK, axis=0)                      # [N, K/128]
+    for kb in range(k // BLOCK):
+        sl = slice(kb * BLOCK, (kb + 1) * BLOCK)
+        part = (av[:, sl] @ bv[:, sl].T).astype(np.float32)
+        s = (sa_inv[:, kb].astype(np.float32)[:, None] * sb_rows[:, kb].astype(np.float32)[None, :])
+        acc = (acc + part * s.astype(np.float32)).astype(np.float32)
+    return _finish(acc, bias_f32)
+
+
+def gemm_rowwise_both(a, sa_inv, b, sb_inv, bias_f32=None):
+    """wgrad form: a[M,K] with sa_inv[M,K/128] and b[N,K] with sb_inv[N,K/128] (both 1x128)."""
+    m, k = a.shape
+    n = b.shape[0]
+    av, bv = e4m3_decode(a), e4m3_decode(b)
+    acc = np.zeros((m, n), np.float32)
+    for kb in range(k // BLOCK):
+        sl = slice(kb * BLOCK, (kb + 1) * BLOCK)
+        part = (av[:, sl] @ bv[:, sl].T).astype(np.float32)
+        s = sa_inv[:, kb].astype(np.float32)[:, None] * sb_inv[:, kb].astype(np.float32)[None, :]
+        acc = (acc + part * s.astype(np.float32)).astype(np.float32)
+    return _finish(acc, bias_f32)
+
+
+def gemm_grouped_blockwise(a, sa_inv, b, sb_inv, offs):
+    """MoE grouped form.  a[sumM, K] rows sorted by expert; b[E, N, K]; sb_inv[E, N/128, K/128];
+    offs[E] inclusive prefix sums of per-expert row counts (a count may be 0)."""
+    e_cnt, n, _ = b.shape
+    out = np.zeros((a.shape[0], n), np.float32)
+    start = 0
+    for e in range(e_cnt):
+        end = int(offs[e])
+        if end > start:
+            out[start:end], _ = gemm_blockwise(a[start:end], sa_inv[start:end], b[e], sb_inv[e])
+        start = end
+    return out, f32_to_bf16_bits(out)
+
+
+def gemm_dequant_f64(a, sa_rows_inv, b, sb_rows_inv):
+    """Dequantize-then-matmul in float64: the acceptance criterion's right-hand side.
+
+    sa_rows_inv[M, K/128] and sb_rows_inv[N, K/128] are per-row expansions of whatever block
+    geometry was used (np.repeat a 128x128 grid along axis 0, broadcast a scalar, ...).
+    """
+    av = e4m3_decode(a).astype(np.float64) * np.repeat(np.asarray(sa_rows_inv, np.float64), BLOCK, axis=1)
+    bv = e4m3_decode(b).astype(np.float64) * np.repeat(np.asarray(sb_rows_inv, np.float64), BLOCK, axis=1)
+    return av @ bv.T

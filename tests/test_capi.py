@@ -1,0 +1,80 @@
+"""The C-ABI library loads and exports every symbol include/hpfp8.h declares; argument checks that
+return before any kernel launch work without a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hpfp8.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hpfp8_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_functions()
+    for must in ("hpfp8_amax_bf16", "hpfp8_quantize_per_tensor_bf16", "hpfp8_quantize_1x128_bf16",
+                 "hpfp8_quantize_128x128_bf16", "hpfp8_quantize_128x1_t_bf16", "hpfp8_dequantize_1x128_bf16",
+                 "hpfp8_gemm_blockwise", "hpfp8_gemm_per_tensor", "hpfp8_gemm_grouped_blockwise"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from hpfp8 import _lib
+    lib = _lib.load()
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in include/hpfp8.h but not exported"
+    bound = set(_lib.SIGNATURES) | {"hpfp8_last_error"}
+    assert bound == set(declared_functions()), "python binding and header disagree"
+    assert lib.hpfp8_version() >= 100
+
+
+def test_argument_errors_are_reported_without_launching():
+    from hpfp8 import _lib
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.cast(buf, ctypes.c_void_p).value
+    p = (p + 15) & ~15
+    # last dim not a multiple of 128
+    rc = lib.hpfp8_quantize_1x128_bf16(p, 4, 100, p, None, p, None)
+    assert rc == -2 and b"multiple of 128" in lib.hpfp8_last_error()
+    # misaligned pointer
+    rc = lib.hpfp8_quantize_1x128_bf16(p + 2, 1, 128, p, None, p, None)
+    assert rc == -3
+    # null buffer
+    rc = lib.hpfp8_quantize_128x128_bf16(None, 128, 128, p, None, None, p, None)
+    assert rc == -1
+    # bad scale granularity, bad K
+    rc = lib.hpfp8_gemm_blockwise(p, p, 1, 1, p, p, 1, 1, 7, 128, 128, 128, None, p, 128, 0, 0, None)
+    assert rc == -1
+    rc = lib.hpfp8_gemm_blockwise(p, p, 1, 1, p, p, 1, 1, 128, 128, 128, 100, None, p, 128, 0, 0, None)
+    assert rc == -2
+    # accumulate needs fp32 output
+    rc = lib.hpfp8_gemm_blockwise(p, p, 1, 1, p, p, 1, 1, 128, 128, 128, 128, None, p, 128, 0, 1, None)
+    assert rc == -1
+    # empty problems succeed without touching the device
+    assert lib.hpfp8_quantize_1x128_bf16(None, 0, 128, None, None, None, None) == 0
+    assert lib.hpfp8_gemm_per_tensor(None, None, None, None, 0, 128, 128, None, None, 128, 0, None) == 0
+
+
+def test_python_wrappers_reject_cpu_tensors_and_bad_shapes():
+    import torch
+    import hpfp8
+    x = torch.zeros(4, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="no CPU fallback"):
+        hpfp8.quantize_1x128(x)
+    with pytest.raises(TypeError):
+        hpfp8.fp8_linear(torch.zeros(4, 128), torch.zeros(128, 128, dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        hpfp8.fp8_linear(x, torch.zeros(128, 256, dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        hpfp8.fp8_linear(x, torch.zeros(128, 128, dtype=torch.bfloat16), recipe="nope")
+    with pytest.raises(ValueError):
+        hpfp8.Fp8Linear(100, 128)
+    with pytest.raises(ValueError):
+        hpfp8.quantize_bucket(torch.zeros(100, dtype=torch.bfloat16))

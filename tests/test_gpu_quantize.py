@@ -1,0 +1,167 @@
+"""GPU parity of the quantize / dequantize kernels through the C ABI: codes byte-exact and fp32
+scales bit-exact against the CPU oracle on the same seeded inputs and on the golden fixtures."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from oracle import c_oracle as C
+import _util as U
+
+pytestmark = pytest.mark.gpu
+G = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fp8_path_golden.npz"))
+
+
+def eq_f32(gpu_t, ref):
+    return np.array_equal(U.f32_bits(U.f32(gpu_t)), U.f32_bits(ref))
+
+
+def test_hardware_cast_all_bf16_patterns(gpu):
+    """Every finite bf16 bit pattern through the cast with scale 1 (amax = 448) and with a scale that
+    makes results land in the subnormal range: the hardware converter must agree with the oracle."""
+    import hpfp8
+    b = np.arange(65536, dtype=np.uint16)
+    f = O.bf16_bits_to_f32(b)
+    keep = np.isfinite(f)
+    b = b[keep]
+    pad = (-b.size) % 128
+    b = np.concatenate([b, np.zeros(pad, np.uint16)])
+    x = U.from_bits(b, gpu)
+    for amax_val in (448.0, 448.0 * 64, 448.0 * 2 ** 20, 1.0, 2.0 ** -100, 3.0 / 7.0):
+        am = torch.tensor(amax_val, dtype=torch.float32, device=gpu)
+        q, s, si = hpfp8.quantize_per_tensor(x, amax_in=am)
+        scale, scale_inv = O.scales_from_amax(np.float32(amax_val))
+        want = O._cast(O.bf16_bits_to_f32(b), scale)
+        assert eq_f32(s, scale) and eq_f32(si, scale_inv)
+        got = U.codes(q)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, (amax_val, [(hex(b[i]), got[i], want[i]) for i in bad[:8]])
+
+
+def test_golden_fixtures(gpu):
+    import hpfp8
+    x = U.from_bits(G["x_bits"], gpu)
+    q, s, si = hpfp8.quantize_per_tensor(x)
+    assert np.array_equal(U.codes(q), G["pt_codes"]) and eq_f32(s, G["pt_scale"]) and eq_f32(si, G["pt_scale_inv"])
+    q, s, si = hpfp8.quantize_1x128(x, want_scale=True)
+    assert np.array_equal(U.codes(q), G["g1x128_codes"]) and eq_f32(s, G["g1x128_scale"]) and eq_f32(si, G["g1x128_scale_inv"])
+    d = hpfp8.dequantize_1x128(q, si)
+    assert np.array_equal(U.bits(d), G["g1x128_dequant_bits"])
+    q, si, qt, s = hpfp8.quantize_128x128(x, with_transpose=True, want_scale=True)
+    assert np.array_equal(U.codes(q), G["b128_codes"]) and eq_f32(s, G["b128_scale"]) and eq_f32(si, G["b128_scale_inv"])
+    assert np.array_equal(U.codes(qt), G["b128_codes"].T)
+    qt, s, si = hpfp8.quantize_128x1_t(x, want_scale=True)
+    assert np.array_equal(U.codes(qt), G["t128x1_codes"]) and eq_f32(s, G["t128x1_scale"]) and eq_f32(si, G["t128x1_scale_inv"])
+    c, si = hpfp8.quantize_bucket(U.from_bits(G["bucket_bits"], gpu))
+    assert np.array_equal(U.codes(c), G["bucket_codes"]) and eq_f32(si, G["bucket_scale_inv"])
+    back = hpfp8.dequantize_bucket(c, si, grad_scale=0.125)
+    assert np.array_equal(U.bits(back), G["bucket_back_bits"])
+
+
+@pytest.mark.parametrize("shape,seed,std,of,om", [
+    ((2048, 1024), 0, 1.0, 0.0, 1.0),          # cfg 1 activations
+    ((1024, 1024), 1, 0.02, 0.0, 1.0),         # cfg 1 weights
+    ((512, 7168), 2, 1.0, 0.001, 50.0),        # cfg 2 activations (row subset)
+    ((384, 640), 3, 0.006, 0.0, 1.0),
+    ((128, 128), 4, 1e-4, 1e-3, 1e3),
+])
+def test_seeded_parity_all_quantizers(gpu, shape, seed, std, of, om):
+    import hpfp8
+    x = U.randn_bf16(shape, seed, std, of, om)
+    xb = U.bits(x)
+    xg = x.to(gpu)
+    # per tensor (amax reduction + cast)
+    q, s, si = hpfp8.quantize_per_tensor(xg)
+    rq, rs, rsi = C.quantize_per_tensor(xb)
+    assert eq_f32(hpfp8.amax(xg), O.amax(O.bf16_bits_to_f32(xb)))
+    assert np.array_equal(U.codes(q), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    # 1x128
+    q, s, si = hpfp8.quantize_1x128(xg, want_scale=True)
+    rq, rs, rsi = C.quantize_1x128(xb)
+    assert np.array_equal(U.codes(q), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    assert np.array_equal(U.bits(hpfp8.dequantize_1x128(q, si)), C.dequantize_1x128(rq, rsi))
+    # 128x128 with transposed copy
+    q, si, qt, s = hpfp8.quantize_128x128(xg, with_transpose=True, want_scale=True)
+    rq, rs, rsi = C.quantize_128x128(xb)
+    assert np.array_equal(U.codes(q), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    assert np.array_equal(U.codes(qt), rq.T)
+    q2, si2 = hpfp8.quantize_128x128(xg)
+    assert np.array_equal(U.codes(q2), rq) and eq_f32(si2, rsi)
+    assert np.array_equal(U.bits(hpfp8.dequantize_128x128(q, si)), O.dequantize_128x128(rq, rsi))
+    # 128x1 transposed
+    qt, s, si = hpfp8.quantize_128x1_t(xg, want_scale=True)
+    rq, rs, rsi = C.quantize_128x1_t(xb)
+    assert np.array_equal(U.codes(qt), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+
+
+def test_laplace_gradients_and_transposed_identity(gpu):
+    import hpfp8
+    go = U.laplace_bf16((512, 896), seed=9, scale=1e-3)
+    gg = go.to(gpu)
+    qt, si = hpfp8.quantize_128x1_t(gg)
+    q, si2 = hpfp8.quantize_1x128(gg.t().contiguous())
+    assert torch.equal(qt.view(torch.uint8), q.view(torch.uint8)) and torch.equal(si, si2)
+    rq, rs, rsi = C.quantize_128x1_t(U.bits(go))
+    assert np.array_equal(U.codes(qt), rq) and eq_f32(si, rsi)
+
+
+def test_special_values_and_edge_shapes(gpu):
+    import hpfp8
+    sp = U.special_bf16_rows(256)
+    q, s, si = hpfp8.quantize_1x128(sp.to(gpu), want_scale=True)
+    rq, rs, rsi = O.quantize_1x128(U.bits(sp))
+    assert np.array_equal(U.codes(q), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    # empty tensors
+    e = torch.empty((0, 128), dtype=torch.bfloat16, device=gpu)
+    q, si = hpfp8.quantize_1x128(e)
+    assert q.shape == (0, 128) and si.shape == (0, 1)
+    assert float(hpfp8.amax(torch.empty((0,), dtype=torch.bfloat16, device=gpu))) == 0.0
+    # per-tensor with a ragged tail (numel not a multiple of 8)
+    x = U.randn_bf16((1003,), 17)
+    q, s, si = hpfp8.quantize_per_tensor(x.to(gpu))
+    rq, rs, rsi = O.quantize_per_tensor(U.bits(x))
+    assert np.array_equal(U.codes(q), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    # one group, one row; 3-D input
+    x = U.randn_bf16((3, 5, 256), 18)
+    q, si = hpfp8.quantize_1x128(x.to(gpu))
+    rq, rs, rsi = O.quantize_1x128(U.bits(x).reshape(15, 256))
+    assert np.array_equal(U.codes(q).reshape(15, 256), rq) and eq_f32(si.reshape(15, 2), rsi)
+    with pytest.raises(ValueError):
+        hpfp8.quantize_1x128(torch.zeros((4, 100), dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(ValueError):
+        hpfp8.quantize_128x1_t(torch.zeros((100, 128), dtype=torch.bfloat16, device=gpu))
+
+
+def test_bucket_full_size_properties(gpu):
+    """2^29-element bucket (cfg 5): properties that do not need a CPU pass over 1 GiB:
+    a strided sample of groups against the oracle, idempotence of quantize(dequantize(.)) on the
+    codes, and the per-group error bound."""
+    import hpfp8
+    n = 1 << 29
+    g = torch.Generator(device=gpu).manual_seed(0)
+    flat = (torch.randn(n, generator=g, device=gpu, dtype=torch.float32) * 1e-4)
+    idx = torch.randint(0, n, (n // 10000,), generator=g, device=gpu)
+    flat[idx] *= 1e3
+    flat = flat.to(torch.bfloat16)
+    codes, si = hpfp8.quantize_bucket(flat)
+    assert codes.shape == (n,) and si.shape == (n // 128,)
+    # sample of groups vs the oracle
+    gsel = torch.arange(0, n // 128, 4099, device=gpu)
+    rows = flat.view(-1, 128)[gsel].cpu()
+    rq, rs, rsi = O.quantize_1x128(U.bits(rows))
+    assert np.array_equal(U.codes(codes.view(-1, 128)[gsel]), rq)
+    assert np.array_equal(U.f32_bits(U.f32(si[gsel])), U.f32_bits(rsi.reshape(-1)))
+    back = hpfp8.dequantize_bucket(codes, si)
+    rback = O.dequantize_1x128(rq, rsi)
+    assert np.array_equal(U.bits(back.view(-1, 128)[gsel]), rback)
+    # error bound per group: |x - back| <= amax/28 + amax/256
+    am = flat.view(-1, 128).float().abs().amax(dim=1, keepdim=True)
+    err = (back.view(-1, 128).float() - flat.view(-1, 128).float()).abs()
+    assert bool((err <= am / 28 + am / 256 + 1e-30).all())
+    del err, am
+    # no NaN codes, and every group uses the top of the range (its amax element maps to +-448)
+    c8 = codes.view(torch.uint8).view(-1, 128)
+    assert not bool(((c8 & 0x7F) == 0x7F).any())
+    assert bool((((c8 & 0x7F) == 0x7E).any(dim=1)).all())

@@ -1,0 +1,336 @@
+"""Pins the CPU oracle to facts it did not author: torch's float8_e4m3fn cast, the closed form of
+the OCP E4M3FN format, brute force on small inputs, algebraic identities and a second, independently
+written C implementation.  Every function of oracle/fp8_oracle.py is covered by at least one check
+that a plausible slip (dropped term, wrong index, transposed operand, wrong rounding) would fail."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from oracle import c_oracle as C
+import _util as U
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KAT = json.load(open(os.path.join(HERE, "golden", "e4m3_known_answers.json")))
+
+
+def torch_encode(x_f32: np.ndarray) -> np.ndarray:
+    return torch.from_numpy(np.ascontiguousarray(x_f32, np.float32)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+
+
+# ---------------------------------------------------------------- E4M3 format
+def test_decode_all_256_codes_against_torch_and_c():
+    codes = np.arange(256, dtype=np.uint8)
+    t = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fn).float().numpy()
+    d = O.e4m3_decode(codes)
+    c = C.e4m3_decode(codes)
+    nan = np.isnan(t)
+    assert nan.sum() == 2 and nan[0x7F] and nan[0xFF]
+    assert np.array_equal(np.isnan(d), nan) and np.array_equal(np.isnan(c), nan)
+    assert np.array_equal(d[~nan].view(np.uint32), t[~nan].view(np.uint32))
+    assert np.array_equal(c[~nan].view(np.uint32), t[~nan].view(np.uint32))
+
+
+def test_decode_known_answers():
+    for code, val in KAT["decode"].items():
+        got = O.e4m3_decode(np.array([int(code)], np.uint8))[0]
+        assert got == np.float32(val) and np.signbit(got) == np.signbit(np.float32(val)), (code, got, val)
+
+
+def test_encode_known_answers():
+    for val, code in KAT["encode"]:
+        assert O.e4m3_encode(np.array([val], np.float32))[0] == code, (val, code)
+        assert C.e4m3_encode(np.array([val], np.float32))[0] == code, (val, code)
+
+
+def test_encode_roundtrips_every_code():
+    codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], np.uint8)
+    assert np.array_equal(O.e4m3_encode(O.e4m3_decode(codes)), codes)
+
+
+def test_encode_all_bf16_patterns_against_torch():
+    b = np.arange(65536, dtype=np.uint16)
+    x = O.bf16_bits_to_f32(b)
+    assert np.array_equal(O.e4m3_encode(x), torch_encode(x))
+
+
+def test_encode_midpoints_and_neighbours_against_torch_and_c():
+    codes = np.arange(0, 0x7F, dtype=np.uint8)
+    v = O.e4m3_decode(codes).astype(np.float64)
+    mids = ((v[:-1] + v[1:]) / 2).astype(np.float32)          # exact in fp32
+    pts = [mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf)),
+           np.array([448.0, 463.99997, 464.0, 480.0, 1e30, np.inf, np.nan, 0.0, 2.0 ** -10, 2.0 ** -11], np.float32)]
+    x = np.concatenate(pts).astype(np.float32)
+    x = np.concatenate([x, -x])
+    ref = torch_encode(x)
+    assert np.array_equal(O.e4m3_encode(x), ref)
+    finite = np.isfinite(x)
+    assert np.array_equal(C.e4m3_encode(x[finite]), ref[finite])
+    # ties go to the even mantissa: the midpoint between codes c and c+1 lands on the even one
+    got = O.e4m3_encode(mids)
+    want = np.where(codes[:-1] % 2 == 0, codes[:-1], codes[1:])
+    assert np.array_equal(got, want)
+
+
+def test_encode_random_fp32_against_torch():
+    rng = np.random.default_rng(7)
+    u = rng.integers(0, 2 ** 32, size=2_000_000, dtype=np.uint64).astype(np.uint32)
+    x = u.view(np.float32)
+    assert np.array_equal(O.e4m3_encode(x), torch_encode(x))
+    sub = x[:20000]
+    sub = sub[np.isfinite(sub)]
+    assert np.array_equal(C.e4m3_encode(sub), torch_encode(sub))
+
+
+# ---------------------------------------------------------------- bf16 conversion
+def test_bf16_conversions_against_torch():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, 200000).astype(np.float32)
+    x = np.concatenate([x, np.array([0.0, -0.0, np.inf, -np.inf, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8], np.float32)])
+    want = U.bits(torch.from_numpy(x).to(torch.bfloat16))
+    assert np.array_equal(O.f32_to_bf16_bits(x), want)
+    assert np.array_equal(O.bf16_bits_to_f32(want).view(np.uint32), want.astype(np.uint32) << 16)
+
+
+# ---------------------------------------------------------------- amax / scales
+def test_scales_closed_form_and_special_cases():
+    am = np.array([0.0, 1e-13, 1e-12, 2e-12, 1.0, 448.0, 3.0, 1.2e-38, 3.3895e38], np.float32)
+    s, si = O.scales_from_amax(am)
+    for a, sv, siv in zip(am, s, si):
+        amc = max(np.float32(a), np.float32(1e-12))
+        assert sv == np.float32(np.float32(448.0) / amc) and siv == np.float32(amc / np.float32(448.0))
+    assert s[0] == s[1] == s[2] == np.float32(448.0) / np.float32(1e-12)   # eps clamp
+    assert np.isfinite(s).all() and np.isfinite(si).all() and (si > 0).all()
+    assert s[5] == 1.0 and si[5] == 1.0
+    # the two multipliers are separate divisions, not reciprocals of each other
+    assert si[6] == np.float32(np.float32(3.0) / np.float32(448.0))
+    a = np.float32(3.0) / np.float32(7.0)
+    s7, si7 = O.scales_from_amax(a)
+    assert si7 == np.float32(a / np.float32(448.0)) and si7 != np.float32(np.float32(1.0) / s7)
+
+
+def test_amax_brute_force():
+    x = U.randn_bf16((7, 33), seed=11)
+    xf = x.float().numpy()
+    best = 0.0
+    for v in xf.reshape(-1):
+        best = max(best, abs(float(v)))
+    assert O.amax(xf) == np.float32(best)
+
+
+# ---------------------------------------------------------------- quantizers
+def _scalar_quantize_block(vals_f32):
+    """Straight-line Python restatement used only on tiny blocks."""
+    am = np.float32(0.0)
+    for v in vals_f32:
+        am = max(am, np.float32(abs(v)))
+    amc = max(am, np.float32(1e-12))
+    scale = np.float32(np.float32(448.0) / amc)
+    scale_inv = np.float32(amc / np.float32(448.0))
+    out = []
+    for v in vals_f32:
+        y = np.float32(np.float32(v) * scale)
+        y = min(max(y, np.float32(-448.0)), np.float32(448.0))
+        out.append(int(torch.tensor([y], dtype=torch.float32).to(torch.float8_e4m3fn).view(torch.uint8)[0]))
+    return np.array(out, np.uint8), scale, scale_inv
+
+
+def test_quantize_1x128_equals_blockwise_loop_with_torch_cast():
+    x = U.randn_bf16((6, 256), seed=21, outlier_frac=0.01, outlier_mul=50.0)
+    x[:, :128] = U.special_bf16_rows(128)[:6]
+    xb = U.bits(x)
+    q, s, si = O.quantize_1x128(xb)
+    xf = x.float().numpy()
+    for r in range(6):
+        for gidx in range(2):
+            qq, ss, ssi = _scalar_quantize_block(xf[r, gidx * 128:(gidx + 1) * 128])
+            assert np.array_equal(q[r, gidx * 128:(gidx + 1) * 128], qq)
+            assert s[r, gidx] == ss and si[r, gidx] == ssi
+
+
+def test_special_rows_behave_as_documented():
+    sp = U.special_bf16_rows(128)
+    q, s, si = O.quantize_1x128(U.bits(sp))
+    assert (q[0] == 0).all() and s[0, 0] == np.float32(448.0) / np.float32(1e-12)       # zero group
+    assert q[3, 0] == 0xFE and q[3, -1] == 0x7E                                            # +-448 hit exactly
+    assert q[4, 0] == 0x7E and q[4, 1] == 0xFE and q[4, 2] == 88 and q[4, 3] == 90        # scale 1: 17->16, 19->20
+    assert q[6, 0] == 0x80 and q[6, 2] == 0x80 | O.e4m3_encode(np.float32([2.0 ** -10 * 448]))[0]
+    assert not ((q & 0x7F) == 0x7F).any()                                                   # never NaN codes
+    assert (q[9] == 0).sum() == 0 and s[9, 0] == np.float32(448.0) / np.float32(1e-12)    # below the clamp
+
+
+def test_block_variants_reduce_to_per_tensor_on_each_block():
+    x = U.randn_bf16((256, 256), seed=31, outlier_frac=0.002, outlier_mul=50.0)
+    xb = U.bits(x)
+    q, s, si = O.quantize_128x128(xb)
+    for br in range(2):
+        for bc in range(2):
+            blk = np.ascontiguousarray(xb[br * 128:(br + 1) * 128, bc * 128:(bc + 1) * 128])
+            qq, ss, ssi = O.quantize_per_tensor(blk)
+            assert np.array_equal(q[br * 128:(br + 1) * 128, bc * 128:(bc + 1) * 128], qq)
+            assert s[br, bc] == ss and si[br, bc] == ssi
+    q1, s1, si1 = O.quantize_1x128(xb)
+    for r in (0, 5, 255):
+        qq, ss, ssi = O.quantize_per_tensor(np.ascontiguousarray(xb[r, 128:256]))
+        assert np.array_equal(q1[r, 128:256], qq) and s1[r, 1] == ss and si1[r, 1] == ssi
+
+
+def test_transposed_requant_is_rowwise_quantize_of_the_transpose():
+    x = U.randn_bf16((256, 384), seed=41, outlier_frac=0.002, outlier_mul=50.0)
+    xb = U.bits(x)
+    qt, st, sit = O.quantize_128x1_t(xb)
+    q, s, si = O.quantize_1x128(np.ascontiguousarray(xb.T))
+    assert np.array_equal(qt, q) and np.array_equal(st, s) and np.array_equal(sit, si)
+
+
+def test_bucket_is_1x128_on_the_flat_view_and_roundtrip_bound():
+    g = U.randn_bf16((128 * 40,), seed=51, std=1e-4, outlier_frac=1e-3, outlier_mul=1e3)
+    gb = U.bits(g)
+    c, s, si = O.quantize_bucket(gb)
+    q, s2, si2 = O.quantize_1x128(gb.reshape(-1, 128))
+    assert np.array_equal(c, q.reshape(-1)) and np.array_equal(si, si2.reshape(-1))
+    back = O.bf16_bits_to_f32(O.dequantize_bucket(c, si)).reshape(-1, 128)
+    orig = O.bf16_bits_to_f32(gb).reshape(-1, 128)
+    am = np.abs(orig).max(axis=1, keepdims=True)
+    # half an E4M3 step in the top binade is amax/28; the bf16 rounding of the result adds at most
+    # 2^-9 of the magnitude (<= amax/512)
+    assert (np.abs(back - orig) <= am / 28 + am / 256 + 1e-30).all()
+    # grad_scale is applied after the cast back, on bf16 values, with its own rounding
+    scaled = O.dequantize_bucket(c, si, grad_scale=0.3)
+    want = O.f32_to_bf16_bits((O.bf16_bits_to_f32(O.dequantize_bucket(c, si)) * np.float32(0.3)).astype(np.float32))
+    assert np.array_equal(scaled, want)
+
+
+def test_dequantize_matches_definition():
+    x = U.randn_bf16((128, 256), seed=61)
+    q, s, si = O.quantize_128x128(U.bits(x))
+    d = O.bf16_bits_to_f32(O.dequantize_128x128(q, si))
+    want = torch.from_numpy(O.e4m3_decode(q) * np.repeat(np.repeat(si, 128, 0), 128, 1)).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(d, want)
+    qp, sp, sip = O.quantize_per_tensor(U.bits(x))
+    dp = O.bf16_bits_to_f32(O.dequantize_per_tensor(qp, sip))
+    wantp = torch.from_numpy(O.e4m3_decode(qp) * sip).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(dp, wantp)
+
+
+# ---------------------------------------------------------------- C restatement, bit for bit
+@pytest.mark.parametrize("name", ["quantize_1x128", "quantize_128x128", "quantize_128x1_t"])
+def test_c_restatement_bit_exact(name):
+    x = U.randn_bf16((256, 384), seed=71, outlier_frac=0.001, outlier_mul=50.0)
+    x[:10, :128] = U.special_bf16_rows(128)
+    xb = U.bits(x)
+    a = getattr(O, name)(xb)
+    b = getattr(C, name)(xb)
+    assert np.array_equal(a[0], b[0])
+    assert np.array_equal(U.f32_bits(a[1]), U.f32_bits(b[1])) and np.array_equal(U.f32_bits(a[2]), U.f32_bits(b[2]))
+
+
+def test_c_per_tensor_and_dequant_bit_exact():
+    x = U.randn_bf16((64, 256), seed=72)
+    xb = U.bits(x)
+    a, b = O.quantize_per_tensor(xb), C.quantize_per_tensor(xb)
+    assert np.array_equal(a[0], b[0]) and a[1] == b[1] and a[2] == b[2]
+    q, s, si = O.quantize_1x128(xb)
+    assert np.array_equal(O.dequantize_1x128(q, si), C.dequantize_1x128(q, si))
+
+
+# ---------------------------------------------------------------- GEMMs
+def test_gemm_per_tensor_against_torch_scaled_mm():
+    x = U.randn_bf16((64, 256), seed=81)
+    w = U.randn_bf16((128, 256), seed=82, std=0.02)
+    xq, _, sxi = O.quantize_per_tensor(U.bits(x))
+    wq, _, swi = O.quantize_per_tensor(U.bits(w))
+    y, yb = O.gemm_per_tensor(xq, sxi, wq, swi)
+    a = torch.from_numpy(xq).view(torch.float8_e4m3fn)
+    b = torch.from_numpy(wq).view(torch.float8_e4m3fn)
+    try:
+        ref = torch._scaled_mm(a, b.t(), scale_a=torch.tensor(float(sxi)), scale_b=torch.tensor(float(swi)),
+                               out_dtype=torch.float32)
+    except Exception as e:  # pragma: no cover - depends on the CPU build of torch
+        pytest.skip(f"torch._scaled_mm unavailable on this CPU build: {e}")
+    rel = np.linalg.norm(y - ref.numpy()) / np.linalg.norm(ref.numpy())
+    assert rel < 1e-5, rel
+
+
+def test_gemm_exact_on_integer_inputs_with_unit_scales():
+    """Small integers are exact in E4M3 and their dot products are exact in fp32: the oracle GEMMs
+    must then equal the int64 matmul exactly.  Catches transposed operands and wrong block indexing."""
+    rng = np.random.default_rng(5)
+    ai = rng.integers(-8, 9, size=(48, 384)).astype(np.float32)
+    bi = rng.integers(-8, 9, size=(256, 384)).astype(np.float32)
+    a, b = O.e4m3_encode(ai), O.e4m3_encode(bi)
+    assert np.array_equal(O.e4m3_decode(a), ai)
+    want = ai.astype(np.int64) @ bi.astype(np.int64).T
+    ones_a = np.ones((48, 3), np.float32)
+    y, _ = O.gemm_blockwise(a, ones_a, b, np.ones((2, 3), np.float32))
+    assert np.array_equal(y.astype(np.int64), want)
+    y, _ = O.gemm_rowwise_both(a, ones_a, b, np.ones((256, 3), np.float32))
+    assert np.array_equal(y.astype(np.int64), want)
+    y, _ = O.gemm_per_tensor(a, 1.0, b, 1.0)
+    assert np.array_equal(y.astype(np.int64), want)
+    yc, _ = C.gemm_blockwise(a, ones_a, b, np.ones((2, 3), np.float32))
+    assert np.array_equal(yc.astype(np.int64), want)
+    # distinct power-of-two scales per block stay exact and expose any mix-up of scale indices
+    sa = (2.0 ** rng.integers(-3, 4, size=(48, 3))).astype(np.float32)
+    sb = (2.0 ** rng.integers(-3, 4, size=(2, 3))).astype(np.float32)
+    want2 = np.zeros((48, 256))
+    for kb in range(3):
+        part = ai[:, kb * 128:(kb + 1) * 128].astype(np.float64) @ bi[:, kb * 128:(kb + 1) * 128].astype(np.float64).T
+        want2 += part * sa[:, kb][:, None] * np.repeat(sb[:, kb], 128)[None, :]
+    y, _ = O.gemm_blockwise(a, sa, b, sb)
+    assert np.array_equal(y.astype(np.float64), want2)
+    yc, _ = C.gemm_blockwise(a, sa, b, sb)
+    assert np.array_equal(yc.astype(np.float64), want2)
+
+
+def test_gemm_blockwise_against_float64_dequant_matmul_and_bias():
+    x = U.randn_bf16((96, 384), seed=91, outlier_frac=0.002, outlier_mul=50.0)
+    w = U.randn_bf16((256, 384), seed=92, std=0.02)
+    bias = U.randn_bf16((256,), seed=93, std=0.1).float().numpy()
+    xq, _, sxi = O.quantize_1x128(U.bits(x))
+    wq, _, swi = O.quantize_128x128(U.bits(w))
+    ref = O.gemm_dequant_f64(xq, sxi, wq, np.repeat(swi, 128, axis=0))
+    y, yb = O.gemm_blockwise(xq, sxi, wq, swi)
+    assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 1e-6
+    yb_f = O.bf16_bits_to_f32(yb)
+    assert np.linalg.norm(yb_f - ref) / np.linalg.norm(ref) < 3e-3      # one bf16 rounding
+    y2, _ = O.gemm_blockwise(xq, sxi, wq, swi, bias)
+    assert np.allclose(y2 - y, bias[None, :], rtol=0, atol=1e-5)
+    yc, _ = C.gemm_blockwise(xq, sxi, wq, swi, bias_f32=bias)
+    assert np.linalg.norm(yc - y2) / np.linalg.norm(y2) < 1e-6
+    # and the quantization error itself is small against the unquantized product
+    exact = x.double().numpy() @ w.double().numpy().T
+    assert np.linalg.norm(ref - exact) / np.linalg.norm(exact) < 0.05
+
+
+def test_gemm_rowwise_both_against_float64():
+    a = U.randn_bf16((128, 256), seed=94)
+    b = U.randn_bf16((256, 256), seed=95)
+    aq, _, asi = O.quantize_1x128(U.bits(a))
+    bq, _, bsi = O.quantize_1x128(U.bits(b))
+    ref = O.gemm_dequant_f64(aq, asi, bq, bsi)
+    y, _ = O.gemm_rowwise_both(aq, asi, bq, bsi)
+    assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 1e-6
+    yc, _ = C.gemm_blockwise(aq, asi, bq, bsi, sb_per_row=True)
+    assert np.linalg.norm(yc - ref) / np.linalg.norm(ref) < 1e-6
+
+
+def test_grouped_equals_loop_of_dense_with_empty_experts():
+    counts = [5, 0, 130, 0, 1]
+    offs = np.cumsum(counts).astype(np.int32)
+    total = int(offs[-1])
+    x = U.randn_bf16((total, 256), seed=96)
+    w = U.randn_bf16((5 * 128, 256), seed=97, std=0.02)
+    xq, _, sxi = O.quantize_1x128(U.bits(x))
+    wq, _, swi = O.quantize_128x128(U.bits(w))
+    wq3, swi3 = wq.reshape(5, 128, 256), swi.reshape(5, 1, 2)
+    y, _ = O.gemm_grouped_blockwise(xq, sxi, wq3, swi3, offs)
+    start = 0
+    for e, cnt in enumerate(counts):
+        if cnt:
+            ye, _ = O.gemm_blockwise(xq[start:start + cnt], sxi[start:start + cnt], wq3[e], swi3[e])
+            assert np.array_equal(y[start:start + cnt], ye)
+        start += cnt
