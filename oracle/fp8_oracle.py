@@ -146,7 +146,8 @@ def scales_from_amax(am: np.ndarray):
 
 
 def _cast(x_f32: np.ndarray, scale: np.ndarray) -> np.ndarray:
-    y = (np.asarray(x_f32, dtype=np.float32) * np.asarray(scale, dtype=np.float32)).astype(np.float32)
+    with np.errstate(over="ignore"):      # a product beyond fp32 range becomes +-Inf and is clamped next
+        y = (np.asarray(x_f32, dtype=np.float32) * np.asarray(scale, dtype=np.float32)).astype(np.float32)
     y = np.clip(y, -FP8_MAX, FP8_MAX).astype(np.float32)
     return e4m3_encode(y)
 

