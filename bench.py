@@ -1,0 +1,229 @@
+"""Benchmark of the FP8 linear hot path on one MI355X.
+
+A step is one blockwise-FP8 forward of the DeepSeekV3 dense-MLP gate/up projection
+(x[4096,7168] bf16 with 0.1% x50 outliers, W[36864,7168] bf16 ~ N(0,0.006)):
+    quantize x 1x128  ->  quantize W 128x128  ->  scaled FP8 GEMM (fp32 accumulation, bf16 out)
+with all inputs resident in HBM when the clock starts and every kernel launched through the C ABI
+on preallocated buffers.  One JSON line is printed:
+
+    value      = 2*M*N*K / step time, TFLOP/s (whole step, quantizers included)
+    roofline   = the dominant kernel (the GEMM) alone, timed with HIP events on its stream
+    quantize   = the HBM-bound kernels alone, GB/s of algorithmic bytes, same timing method
+    cpu_baseline = the CPU oracle's C restatement on a bounded sample of the same workload
+
+Usage: python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "hyper-parallel_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+M, N, K = 4096, 36864, 7168
+PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
+# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured
+GEMM_TRAFFIC_BYTES = None
+
+
+def make_inputs(dev):
+    import torch
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32)
+    k = round(0.001 * M * K)
+    idx = torch.randperm(M * K, generator=g, device=dev)[:k]
+    x.view(-1)[idx] *= 50.0
+    x = x.to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=g, device=dev, dtype=torch.float32) * 0.006).to(torch.bfloat16)
+    return x, w
+
+
+def event_ms(pairs):
+    return [s.elapsed_time(e) for s, e in pairs]
+
+
+def cpu_baseline(x_bits, w_bits, target_seconds=15.0):
+    """The C restatement of the oracle (OpenMP over the host cores) on a bounded sample of the same
+    step: quantize all of W (128x128), quantize the first `ms` rows of x (1x128), scaled GEMM of those
+    rows against all of W.  The whole-step time is extrapolated linearly in the row count."""
+    import numpy as np
+    from oracle import c_oracle as C
+    threads = C.num_threads()
+    t0 = time.perf_counter()
+    wq, _, swi = C.quantize_128x128(w_bits)
+    t_qw = time.perf_counter() - t0
+    xq8, _, sxi8 = C.quantize_1x128(np.ascontiguousarray(x_bits[:8]))
+    t0 = time.perf_counter()
+    C.gemm_blockwise(xq8, sxi8, wq, swi)
+    t8 = max(time.perf_counter() - t0, 1e-6)
+    ms = int(min(x_bits.shape[0], max(8, (target_seconds - t_qw) / t8 * 8))) // 8 * 8
+    ms = max(ms, 8)
+    xs = np.ascontiguousarray(x_bits[:ms])
+    t0 = time.perf_counter()
+    xq, _, sxi = C.quantize_1x128(xs)
+    t_qx = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    C.gemm_blockwise(xq, sxi, wq, swi)
+    t_g = time.perf_counter() - t0
+    step_seconds = t_qw + (t_qx + t_g) * (M / ms)
+    return {
+        "value": 2.0 * M * N * K / step_seconds / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"quantize W[{N},{K}] ({t_qw:.1f} s) + quantize x[:{ms}] ({t_qx:.2f} s) + scaled GEMM of those "
+                  f"{ms} rows against all of W ({t_g:.1f} s), {threads} OpenMP threads; whole step extrapolated "
+                  f"linearly in rows to {step_seconds:.0f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one GPU's share of the path; this build has no multi-GPU leg "
+                 "(run with --gpus 1).")
+
+    import torch
+    import hpfp8
+    from hpfp8 import _lib, ops
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    lib = _lib.load()
+    assert lib.hpfp8_check_device() == 0, lib.hpfp8_last_error().decode()
+    dev = torch.device("cuda:0")
+    x, w = make_inputs(dev)
+
+    # preallocated outputs: nothing is allocated inside the timed region
+    FP8 = torch.float8_e4m3fn
+    xq = torch.empty((M, K), dtype=FP8, device=dev)
+    sx = torch.empty((M, K // 128), dtype=torch.float32, device=dev)
+    wq = torch.empty((N, K), dtype=FP8, device=dev)
+    sw = torch.empty((N // 128, K // 128), dtype=torch.float32, device=dev)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def q_act():
+        _lib.call("hpfp8_quantize_1x128_bf16", x.data_ptr(), M, K, xq.data_ptr(), None, sx.data_ptr(), stream)
+
+    def q_wgt():
+        _lib.call("hpfp8_quantize_128x128_bf16", w.data_ptr(), N, K, wq.data_ptr(), None, None, sw.data_ptr(), stream)
+
+    def gemm():
+        _lib.call("hpfp8_gemm_blockwise", xq.data_ptr(), sx.data_ptr(), K // 128, 1, wq.data_ptr(), sw.data_ptr(),
+                  K // 128, 1, 128, M, N, K, None, y.data_ptr(), N, _lib.OUT_BF16, 0, stream)
+
+    def ev():
+        return torch.cuda.Event(enable_timing=True)
+
+    for _ in range(args.warmup):
+        q_act(); q_wgt(); gemm()
+    torch.cuda.synchronize()
+
+    marks = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        e = [ev() for _ in range(4)]
+        e[0].record(); q_act()
+        e[1].record(); q_wgt()
+        e[2].record(); gemm()
+        e[3].record()
+        marks.append(e)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    ms_step = wall * 1e3 / args.steps
+    t_g = sum(event_ms([(e[2], e[3]) for e in marks])) / args.steps
+
+    # HBM-bound kernels alone: back-to-back launches between one event pair; the activation buffers
+    # rotate over > 256 MB so that the Infinity Cache cannot serve the reads.
+    reps = max(args.steps, 12)
+    xs = [x] + [x.clone() for _ in range(5)]
+    xqs = [xq] + [torch.empty_like(xq) for _ in range(5)]
+    torch.cuda.synchronize()
+    s0, s1 = ev(), ev()
+    s0.record()
+    for i in range(reps):
+        _lib.call("hpfp8_quantize_1x128_bf16", xs[i % 6].data_ptr(), M, K, xqs[i % 6].data_ptr(), None,
+                  sx.data_ptr(), stream)
+    s1.record()
+    torch.cuda.synchronize()
+    t_qa = s0.elapsed_time(s1) / reps
+    s0, s1 = ev(), ev()
+    s0.record()
+    for i in range(reps):
+        q_wgt()
+    s1.record()
+    torch.cuda.synchronize()
+    t_qw = s0.elapsed_time(s1) / reps
+    del xs, xqs
+    flops = 2.0 * M * N * K
+    bytes_qa = M * K * 3 + M * (K // 128) * 4
+    bytes_qw = N * K * 3 + (N // 128) * (K // 128) * 4
+    gemm_tflops = flops / (t_g * 1e-3) / 1e12
+
+    # spot check inside the bench: the timed buffers hold the right answer (float64 reference on a slice)
+    lut = torch.tensor([float(v) for v in torch.arange(256, dtype=torch.uint8).view(FP8).float().nan_to_num()],
+                       dtype=torch.float64, device=dev)
+    a64 = lut[xq[:256].view(torch.uint8).long()] * sx[:256].double().repeat_interleave(128, dim=1)
+    b64 = lut[wq[:256].view(torch.uint8).long()] * sw[:2].double().repeat_interleave(128, dim=0).repeat_interleave(128, dim=1)
+    ref = a64 @ b64.t()
+    err = float((y[:256, :256].double() - ref).norm() / ref.norm())
+    assert err < 1e-2, f"GEMM output is wrong: rel Frobenius error {err}"
+
+    out = {
+        "metric": "FP8 linear TFLOP/s & % FP8 MFMA peak; quantize GB/s & % HBM peak (1 GPU)",
+        "value": flops / (ms_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)",
+        "data": "synthetic",
+        "config": {
+            "workload": "DeepSeekV3 dense-MLP blockwise FP8 forward: x[4096,7168] bf16 (0.1% x50 outliers) 1x128 "
+                        "scales, W_gate_up[36864,7168] bf16 N(0,0.006) 128x128 scales; step = quantize x + quantize W + "
+                        "scaled GEMM, bf16 out",
+            "M": M, "N": N, "K": K,
+        },
+        "roofline": {
+            "kernel": "gemm_kernel<block scales> (hpfp8_gemm_blockwise)",
+            "bound": "mfma",
+            "achieved": gemm_tflops,
+            "peak": PEAK_FP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": gemm_tflops / PEAK_FP8_TFLOPS,
+            "traffic": GEMM_TRAFFIC_BYTES,
+            "ms": t_g,
+        },
+        "quantize": {
+            "act_1x128": {"GB/s": bytes_qa / (t_qa * 1e-3) / 1e9, "frac_hbm": bytes_qa / (t_qa * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                          "ms": t_qa, "bytes": bytes_qa},
+            "weight_128x128": {"GB/s": bytes_qw / (t_qw * 1e-3) / 1e9,
+                               "frac_hbm": bytes_qw / (t_qw * 1e-3) / 1e9 / PEAK_HBM_GBS, "ms": t_qw, "bytes": bytes_qw},
+        },
+        "check": {"gemm_rel_frobenius_vs_f64_dequant_matmul": err},
+    }
+    if not args.no_cpu_baseline:
+        import numpy as np
+        xb = x[:1024].cpu().view(torch.int16).numpy().view(np.uint16)
+        wb = w.cpu().view(torch.int16).numpy().view(np.uint16)
+        out["cpu_baseline"] = cpu_baseline(xb, wb)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
