@@ -46,6 +46,15 @@ struct GemmParams {
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// XOR applied to the 16-byte chunk index of tile row r.  ds_read_b128 is served 16 lanes at a time
+// and the 16 are not consecutive: per half-wave the lane quads {0,3,5,6} go together and {1,2,4,7}
+// go together (measured with SQ_LDS_BANK_CONFLICT on pairs of active lanes).  With the fragment
+// mapping lane -> (row = lane%16, k-chunk pair = lane/16) each such group holds all 16 rows once,
+// rows 4..11 with one k-chunk and the other rows with the neighbouring one; shifting the usual
+// (r/2)%8 pattern by 6 sends those two row sets to disjoint chunk ranges, so the 16 lanes hit 16
+// different bank groups.
+__device__ __forceinline__ int row_swizzle(int r) { return (((r >> 1) & 7) + 6) & 7; }
+
 __device__ __forceinline__ v4i lds_read16(const uint8_t* p) {
   return *reinterpret_cast<const v4i*>(p);
 }
@@ -129,7 +138,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   for (int i = 0; i < 4; ++i) {
     const int q = wave * 4 + i;                       // 8-row group inside the tile
     const int r = q * 8 + (lane >> 3);                // row inside the tile
-    const int chunk = (lane & 7) ^ ((r >> 1) & 7);    // logical 16-byte chunk of that row
+    const int chunk = (lane & 7) ^ row_swizzle(r);    // logical 16-byte chunk of that row
     a_off[i] = (uint32_t)(row0 + r) * (uint32_t)K + chunk * 16;
     b_off[i] = (uint32_t)(n0 + r) * (uint32_t)K + chunk * 16;
   }
@@ -147,7 +156,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // ---- fragment addressing
   const int wn = wave & 1, wm = wave >> 1;
   const int l16 = lane & 15, g = lane >> 4;
-  const int pc0 = (2 * g) ^ (l16 >> 1);
+  const int pc0 = (2 * g) ^ row_swizzle(l16);
   const int a_frag_off = (wm * 64 + l16) * BK;               // + j * 16 rows
   const int b_frag_off = kTileBytes + (wn * 128 + l16) * BK;  // + i * 16 rows
 
@@ -194,29 +203,54 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     v8i xf[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
+    if (MODE == kScaleBlock) {
+      // Software pipeline over the 8 n-subtiles: the matrix instructions of subtile i are issued
+      // interleaved with the promotion FMAs of subtile i-1, whose partial sums left the matrix
+      // pipe four instructions earlier, so neither pipe waits for the other.
+      const v4f zero = {0.f, 0.f, 0.f, 0.f};
+      v4f part[2][4];
+      v8i wf = frag_read(sbase + b_frag_off, pc0);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const v8i wf = frag_read(sbase + b_frag_off + i * 16 * BK, pc0);
-      float sbr[4] = {1.f, 1.f, 1.f, 1.f};
-      if (MODE == kScaleRow) {
-        int n = n0 + wn * 128 + i * 16 + g * 4;
-        if (n > N - 4) n = N - 4;
+      for (int i = 0; i < 8; ++i) {
+        v8i wf_next = wf;
+        if (i + 1 < 8) wf_next = frag_read(sbase + b_frag_off + (i + 1) * 16 * BK, pc0);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sbr[r] = p.sb[(int64_t)(n + r) * p.sb_sn + (int64_t)kb * p.sb_sk];
+        for (int j = 0; j < 4; ++j) {
+          part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], zero, 0, 0, 0, 0, 0, 0);
+          if (i > 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              acc[i - 1][j][r] = __builtin_fmaf(part[(i - 1) & 1][j][r], s_cur[j], acc[i - 1][j][r]);
+          }
+          __builtin_amdgcn_sched_barrier(0);   // keep this (MFMA, 4 FMA) group together, in this order
+        }
+        wf = wf_next;
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (MODE == kScaleTensor) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
-        } else {
-          const v4f zero = {0.f, 0.f, 0.f, 0.f};
-          v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], zero, 0, 0, 0, 0, 0, 0);
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            if (MODE == kScaleRow)
+        for (int r = 0; r < 4; ++r) acc[7][j][r] = __builtin_fmaf(part[1][j][r], s_cur[j], acc[7][j][r]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const v8i wf = frag_read(sbase + b_frag_off + i * 16 * BK, pc0);
+        float sbr[4] = {1.f, 1.f, 1.f, 1.f};
+        if (MODE == kScaleRow) {
+          int n = n0 + wn * 128 + i * 16 + g * 4;
+          if (n > N - 4) n = N - 4;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sbr[r] = p.sb[(int64_t)(n + r) * p.sb_sn + (int64_t)kb * p.sb_sk];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (MODE == kScaleTensor) {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+          } else {
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+            v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], zero, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
               acc[i][j][r] = __builtin_fmaf(part[r], s_cur[j] * sbr[r], acc[i][j][r]);
-            else
-              acc[i][j][r] = __builtin_fmaf(part[r], s_cur[j], acc[i][j][r]);
           }
         }
       }
