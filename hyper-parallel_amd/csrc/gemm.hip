@@ -201,19 +201,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     }
     const uint8_t* sbase = lds + stage * kStageBytes;
     v8i xf[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
     if (MODE == kScaleBlock) {
       // Software pipeline over the 8 n-subtiles: the matrix instructions of subtile i are issued
       // interleaved with the promotion FMAs of subtile i-1, whose partial sums left the matrix
-      // pipe four instructions earlier, so neither pipe waits for the other.
+      // pipe four instructions earlier, so neither pipe waits for the other.  The LDS reads of
+      // subtile i+1 are issued before the MFMAs of subtile i (a full subtile of latency cover).
       const v4f zero = {0.f, 0.f, 0.f, 0.f};
       v4f part[2][4];
       v8i wf = frag_read(sbase + b_frag_off, pc0);
 #pragma unroll
+      for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
       for (int i = 0; i < 8; ++i) {
         v8i wf_next = wf;
         if (i + 1 < 8) wf_next = frag_read(sbase + b_frag_off + (i + 1) * 16 * BK, pc0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], zero, 0, 0, 0, 0, 0, 0);
@@ -231,6 +234,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[7][j][r] = __builtin_fmaf(part[1][j][r], s_cur[j], acc[7][j][r]);
     } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const v8i wf = frag_read(sbase + b_frag_off + i * 16 * BK, pc0);
@@ -369,9 +374,10 @@ int hpfp8_gemm_per_tensor(const void* a, const float* sa_inv, const void* b, con
   return launch<kScaleTensor, false>(p, out_type, tiles, (hipStream_t)stream);
 }
 
-int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, const void* b, const float* sb,
-                                 const int32_t* offs, int experts, int64_t total_m, int64_t N,
-                                 int64_t K, void* c, int64_t ldc, int out_type, hpfp8_stream_t stream) {
+int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                                 const void* b, const float* sb, const int32_t* offs, int experts,
+                                 int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
+                                 hpfp8_stream_t stream) {
   HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "gemm_grouped: bad expert count %d", experts);
   int rc = check_common("gemm_grouped", a, b, sa, sb, total_m, N, K, nullptr, c, ldc, out_type, 0);
   if (rc <= 0) return rc;
@@ -379,7 +385,7 @@ int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, const void* b, 
   HPFP8_REQUIRE(offs != nullptr, HPFP8_ERR_ARG, "gemm_grouped: null offs");
   GemmParams p{};
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb;
-  p.sa_sm = K / BK; p.sa_sk = 1;
+  p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k;
   p.sb_sn = K / BK; p.sb_sk = 1; p.sb_se = (N / kBlock) * (K / BK);
   p.c = c; p.ldc = ldc; p.offs = offs; p.experts = experts;
   p.M = (int)total_m; p.N = (int)N; p.K = (int)K;

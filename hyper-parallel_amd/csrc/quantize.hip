@@ -100,6 +100,49 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const uint4* __restric
   }
 }
 
+// Same arithmetic, scales written k-block-major: scale[g * rows + row] for group g of a row.  This
+// is the layout the GEMM reads with unit stride across the 16 rows of a fragment.  A workgroup owns
+// 16 rows x 4 consecutive groups so that its 64 scales leave as four 64-byte runs.
+__global__ __launch_bounds__(256) void quant_1x128_kmajor_kernel(const uint16_t* __restrict__ x,
+                                                                 uint8_t* __restrict__ q,
+                                                                 float* __restrict__ scale,
+                                                                 float* __restrict__ scale_inv, int rows,
+                                                                 int cols) {
+  const int groups = cols >> 7;
+  const int gtiles = (groups + 3) >> 2;
+  const int g0 = (blockIdx.x % gtiles) * 4, row0 = (blockIdx.x / gtiles) * 16;
+  const int r = threadIdx.x >> 4, l16 = threadIdx.x & 15;
+  const int row = row0 + r;
+  __shared__ float s_s[4][16], s_si[4][16];
+  uint4 v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const bool ok = row < rows && g0 + u < groups;
+    v[u] = ok ? nt_load16(x + (int64_t)row * cols + (g0 + u) * 128 + l16 * 8) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const bool ok = row < rows && g0 + u < groups;
+    uint32_t m = row16_max_u32(mag8(v[u]));
+    float s, si;
+    scales_from_amax(__uint_as_float(m << 16), s, si);
+    if (ok) nt_store8(q + (int64_t)row * cols + (g0 + u) * 128 + l16 * 8, cvt8(v[u], s));
+    if (l16 == 0) {
+      s_s[u][r] = s;
+      s_si[u][r] = si;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const int u = threadIdx.x >> 4, rr = threadIdx.x & 15;
+    if (row0 + rr < rows && g0 + u < groups) {
+      const int64_t o = (int64_t)(g0 + u) * rows + row0 + rr;
+      if (scale) scale[o] = s_s[u][rr];
+      scale_inv[o] = s_si[u][rr];
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // shared by the two tile kernels below: 128x128 tile, 256 threads
 // ---------------------------------------------------------------------------------------------
@@ -197,6 +240,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // ---------------------------------------------------------------------------------------------
 // 128x1 groups, transposed output (wgrad operands): x[M,K] -> qt[K,M], scales [K, M/128]
 // ---------------------------------------------------------------------------------------------
+template <bool KMAJOR>
 __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int m, int k,
                                                             uint8_t* __restrict__ qt,
                                                             float* __restrict__ scale_t,
@@ -240,7 +284,8 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
     float s, si;
     scales_from_amax(__uint_as_float(mag << 16), s, si);
     s_scale[col] = s;
-    int64_t o = ((int64_t)tc * 128 + col) * mb + tr;
+    // row-major [k, m/128], or block-major [m/128, k] (unit stride over the output rows)
+    int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
     if (scale_t) scale_t[o] = s;
     scale_inv_t[o] = si;
   }
@@ -391,6 +436,24 @@ int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q
   return check_launch("quantize_1x128");
 }
 
+int hpfp8_quantize_1x128_kmajor_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                                     float* scale_inv, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_1x128_kmajor: negative shape");
+  HPFP8_REQUIRE(cols % kBlock == 0, HPFP8_ERR_SHAPE,
+                "quantize_1x128_kmajor: last dim %lld is not a multiple of 128", (long long)cols);
+  HPFP8_REQUIRE(rows < (1 << 30) && cols < (1 << 30), HPFP8_ERR_SHAPE, "quantize_1x128_kmajor: dimension too large");
+  if (rows == 0 || cols == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(x && q && scale_inv, HPFP8_ERR_ARG, "quantize_1x128_kmajor: null buffer");
+  HPFP8_REQUIRE(aligned16(x) && aligned16(q), HPFP8_ERR_ALIGN,
+                "quantize_1x128_kmajor: buffers must be 16-byte aligned");
+  const int64_t groups = cols / kBlock;
+  const int64_t blocks = ((groups + 3) / 4) * ((rows + 15) / 16);
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "quantize_1x128_kmajor: tensor too large");
+  quant_1x128_kmajor_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)x, (uint8_t*)q, scale, scale_inv, (int)rows, (int)cols);
+  return check_launch("quantize_1x128_kmajor");
+}
+
 int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, float* scale,
                                 float* scale_inv, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_128x128: negative shape");
@@ -413,20 +476,35 @@ int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void*
   return check_launch("quantize_128x128");
 }
 
-int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
-                                float* scale_inv_t, hpfp8_stream_t stream) {
-  HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "quantize_128x1_t: negative shape");
+static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, int64_t m, int64_t k, void* q_t,
+                                 float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE,
-                "quantize_128x1_t: shape [%lld, %lld] is not a multiple of 128", (long long)m, (long long)k);
-  HPFP8_REQUIRE(m < (1 << 30) && k < (1 << 30), HPFP8_ERR_SHAPE, "quantize_128x1_t: dimension too large");
+                "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)m, (long long)k);
+  HPFP8_REQUIRE(m < (1 << 30) && k < (1 << 30), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
   const int64_t blocks = (m / kBlock) * (k / kBlock);
   if (blocks == 0) return HPFP8_OK;
-  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "quantize_128x1_t: tensor too large");
-  HPFP8_REQUIRE(x && q_t && scale_inv_t, HPFP8_ERR_ARG, "quantize_128x1_t: null buffer");
-  HPFP8_REQUIRE(aligned16(x) && aligned16(q_t), HPFP8_ERR_ALIGN, "quantize_128x1_t: buffers must be 16-byte aligned");
-  quant_128x1_t_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, (int)m, (int)k,
-                                                                          (uint8_t*)q_t, scale_t, scale_inv_t);
-  return check_launch("quantize_128x1_t");
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
+  HPFP8_REQUIRE(x && q_t && scale_inv_t, HPFP8_ERR_ARG, "%s: null buffer", what);
+  HPFP8_REQUIRE(aligned16(x) && aligned16(q_t), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
+  hipStream_t s = (hipStream_t)stream;
+  if (kmajor)
+    quant_128x1_t_kernel<true><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
+                                                                 scale_t, scale_inv_t);
+  else
+    quant_128x1_t_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
+                                                                  scale_t, scale_inv_t);
+  return check_launch(what);
+}
+
+int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
+                                float* scale_inv_t, hpfp8_stream_t stream) {
+  return quantize_128x1_t_impl("quantize_128x1_t", false, x, m, k, q_t, scale_t, scale_inv_t, stream);
+}
+
+int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
+                                       float* scale_inv_t, hpfp8_stream_t stream) {
+  return quantize_128x1_t_impl("quantize_128x1_t_kmajor", true, x, m, k, q_t, scale_t, scale_inv_t, stream);
 }
 
 int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,

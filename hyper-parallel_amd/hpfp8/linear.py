@@ -32,7 +32,7 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias):
         x2 = _flatten(x)
-        xq, sx = ops.quantize_1x128(x2)
+        xq, sx = ops.quantize_1x128(x2, kmajor=True)
         need_wgrad_inputs = x.requires_grad or weight.requires_grad
         if x.requires_grad:
             wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
@@ -58,15 +58,15 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
         if need_dx:
             # dx[M,K] = go[M,N] . W[N,K]: contraction over N, b operand = W^T codes [K,N] whose
             # 128x128 scales are W's with the two strides swapped.
-            goq, sgo = ops.quantize_1x128(go)
+            goq, sgo = ops.quantize_1x128(go, kmajor=True)
             dx = ops.gemm_blockwise(goq, sgo, wqt, sw.t()).reshape(ctx.x_shape)
         if need_dw:
             # dW[N,K] = go^T[N,M] . x[M,K]: contraction over tokens, both operands 1x128 along M
             m = go.shape[0]
             if m % ops.BLOCK:
                 raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
-            got, sgot = ops.quantize_128x1_t(go)
-            xt, sxt = ops.quantize_128x1_t(x2)
+            got, sgot = ops.quantize_128x1_t(go, kmajor=True)
+            xt, sxt = ops.quantize_128x1_t(x2, kmajor=True)
             dw = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
@@ -164,7 +164,7 @@ def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Te
     the inclusive int32 prefix sums of rows per expert, weight[E, N, K] -> bf16 [total_m, N]."""
     if input.dim() != 2 or weight.dim() != 3 or input.shape[1] != weight.shape[2]:
         raise ValueError("input must be [total_m, K] and weight [E, N, K]")
-    xq, sx = ops.quantize_1x128(input)
+    xq, sx = ops.quantize_1x128(input, kmajor=True)
     e, n, k = weight.shape
     wq, sw = ops.quantize_128x128(weight.reshape(e * n, k))
     return ops.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), offs)

@@ -85,8 +85,13 @@ def quantize_per_tensor(x: torch.Tensor, amax_in: Optional[torch.Tensor] = None
     return q, scale, scale_inv
 
 
-def quantize_1x128(x: torch.Tensor, want_scale: bool = False):
-    """x[..., C] -> (codes, scale_inv[..., C/128]) (plus scale when ``want_scale``)."""
+def quantize_1x128(x: torch.Tensor, want_scale: bool = False, kmajor: bool = False):
+    """x[..., C] -> (codes, scale_inv[..., C/128]) (plus scale when ``want_scale``).
+
+    With ``kmajor`` the scales are STORED k-block-major ([C/128, rows] in memory) and returned as the
+    transposed view, so they index exactly like the row-major result but the GEMM reads them with
+    unit stride across rows.  Values are identical in both layouts.
+    """
     x = _check_bf16(x, "x")
     if x.dim() < 1:
         raise ValueError("x must have at least one dimension")
@@ -96,9 +101,21 @@ def quantize_1x128(x: torch.Tensor, want_scale: bool = False):
     rows = x.numel() // cols if cols else 0
     q = torch.empty(x.shape, dtype=FP8, device=x.device)
     sshape = x.shape[:-1] + (cols // BLOCK,)
-    scale_inv = torch.empty(sshape, dtype=torch.float32, device=x.device)
-    scale = torch.empty(sshape, dtype=torch.float32, device=x.device) if want_scale else None
-    _lib.call("hpfp8_quantize_1x128_bf16", _ptr(x), rows, cols, _ptr(q), _ptr(scale), _ptr(scale_inv), _stream())
+    if kmajor:
+        store = (cols // BLOCK, rows)
+        scale_inv = torch.empty(store, dtype=torch.float32, device=x.device)
+        scale = torch.empty(store, dtype=torch.float32, device=x.device) if want_scale else None
+        _lib.call("hpfp8_quantize_1x128_kmajor_bf16", _ptr(x), rows, cols, _ptr(q), _ptr(scale), _ptr(scale_inv),
+                  _stream())
+        scale_inv = scale_inv.t()
+        scale = scale.t() if want_scale else None
+        if x.dim() != 2:
+            scale_inv = scale_inv.reshape(sshape)
+            scale = scale.reshape(sshape) if want_scale else None
+    else:
+        scale_inv = torch.empty(sshape, dtype=torch.float32, device=x.device)
+        scale = torch.empty(sshape, dtype=torch.float32, device=x.device) if want_scale else None
+        _lib.call("hpfp8_quantize_1x128_bf16", _ptr(x), rows, cols, _ptr(q), _ptr(scale), _ptr(scale_inv), _stream())
     return (q, scale, scale_inv) if want_scale else (q, scale_inv)
 
 
@@ -124,10 +141,11 @@ def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: 
     return out
 
 
-def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False):
+def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = False):
     """Transposed re-quantization for wgrad from the bf16 source.
 
     x[M, K] -> (codes_t[K, M], scale_inv_t[K, M/128]); one scale per 128 consecutive rows of a column.
+    With ``kmajor`` the scales are stored [M/128, K] in memory and returned as the transposed view.
     """
     x = _check_bf16(x, "x")
     if x.dim() != 2:
@@ -136,9 +154,14 @@ def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False):
     if m % BLOCK or k % BLOCK:
         raise ValueError(f"shape {tuple(x.shape)} is not a multiple of {BLOCK} in both dims")
     qt = torch.empty((k, m), dtype=FP8, device=x.device)
-    scale_inv = torch.empty((k, m // BLOCK), dtype=torch.float32, device=x.device)
+    sshape = (m // BLOCK, k) if kmajor else (k, m // BLOCK)
+    scale_inv = torch.empty(sshape, dtype=torch.float32, device=x.device)
     scale = torch.empty_like(scale_inv) if want_scale else None
-    _lib.call("hpfp8_quantize_128x1_t_bf16", _ptr(x), m, k, _ptr(qt), _ptr(scale), _ptr(scale_inv), _stream())
+    name = "hpfp8_quantize_128x1_t_kmajor_bf16" if kmajor else "hpfp8_quantize_128x1_t_bf16"
+    _lib.call(name, _ptr(x), m, k, _ptr(qt), _ptr(scale), _ptr(scale_inv), _stream())
+    if kmajor:
+        scale_inv = scale_inv.t()
+        scale = scale.t() if want_scale else None
     return (qt, scale, scale_inv) if want_scale else (qt, scale_inv)
 
 
@@ -271,11 +294,11 @@ def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, s
     if k % BLOCK or n % BLOCK or k == 0:
         raise ValueError(f"K={k} must be a positive multiple of 128 and N={n} a multiple of 128")
     kb = k // BLOCK
-    if tuple(sa.shape) != (total_m, kb) or not sa.is_contiguous():
-        raise ValueError(f"sa must be contiguous [{total_m}, {kb}]")
+    if tuple(sa.shape) != (total_m, kb):
+        raise ValueError(f"sa must be [{total_m}, {kb}]")
     if tuple(sb.shape) != (e, n // BLOCK, kb) or not sb.is_contiguous():
         raise ValueError(f"sb must be contiguous [{e}, {n // BLOCK}, {kb}]")
     out = torch.empty((total_m, n), dtype=out_dtype, device=a.device)
-    _lib.call("hpfp8_gemm_grouped_blockwise", _ptr(a), _ptr(sa), _ptr(b), _ptr(sb), _ptr(offs), e, total_m, n, k,
-              _ptr(out), n, _out_code(out_dtype), _stream())
+    _lib.call("hpfp8_gemm_grouped_blockwise", _ptr(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
+              _ptr(offs), e, total_m, n, k, _ptr(out), n, _out_code(out_dtype), _stream())
     return out

@@ -75,6 +75,12 @@ int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* ama
 int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
                               float* scale_inv, hpfp8_stream_t stream);
 
+/* Same codes; scale / scale_inv written k-block-major, [cols/128, rows]: element (row, g) at
+ * [g * rows + row].  This is the layout the GEMMs read with unit stride over a fragment's rows
+ * (pass sa_stride_m = 1, sa_stride_k = rows). */
+int hpfp8_quantize_1x128_kmajor_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                                     float* scale_inv, hpfp8_stream_t stream);
+
 /* Weights: w[rows, cols] bf16, one scale per 128x128 block.  q[rows, cols]; q_t (may be NULL)
  * receives the transposed codes [cols, rows] that dgrad consumes; scale (may be NULL) and
  * scale_inv are [rows/128, cols/128]. */
@@ -85,6 +91,11 @@ int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void*
  * transposed: q_t[k, m]; scale_t (may be NULL) and scale_inv_t are [k, m/128]. */
 int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
                                 float* scale_inv_t, hpfp8_stream_t stream);
+
+/* Same codes; scale_t / scale_inv_t written block-major, [m/128, k]: element (col, b) at
+ * [b * k + col]. */
+int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
+                                       float* scale_inv_t, hpfp8_stream_t stream);
 
 /* ---- dequantizers ----------------------------------------------------------------------------
  * The cast-back site hyper_parallel/core/hsdp/hsdp_grad_buffer.py:116-125: out = bf16(decode(q)
@@ -125,10 +136,10 @@ int hpfp8_gemm_per_tensor(const void* a, const float* sa_inv, const void* b, con
  * parallelism is unimplemented): rows of a[total_m, K] are sorted by expert; offs[e] (int32,
  * device) is the inclusive prefix sum of per-expert row counts, a count may be 0, rows past
  * offs[experts-1] are left untouched; b[experts, N, K]; sb[experts, N/128, K/128];
- * sa[total_m, K/128]; c[total_m, N] bf16 or fp32. */
-int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, const void* b, const float* sb,
-                                 const int32_t* offs, int experts, int64_t total_m, int64_t N,
-                                 int64_t K, void* c, int64_t ldc, int out_type,
+ * sa(m, kb) = sa[m * sa_stride_m + kb * sa_stride_k]; c[total_m, N] bf16 or fp32. */
+int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                                 const void* b, const float* sb, const int32_t* offs, int experts,
+                                 int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
                                  hpfp8_stream_t stream);
 
 #ifdef __cplusplus

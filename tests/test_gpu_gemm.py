@@ -140,6 +140,9 @@ def test_blockwise_forward_shapes(gpu, M, N, K, seed):
     if M * N * K <= 512 * 1024 * 1024:
         want, _ = O.gemm_blockwise(U.codes(xq), U.f32(sxi), U.codes(wq), U.f32(swi))
         assert rel(U.f32(y32), want) < TOL_F32
+    # k-major scale storage gives the same result bit for bit
+    xq2, sxk = hpfp8.quantize_1x128(x, kmajor=True)
+    assert torch.equal(hpfp8.gemm_blockwise(xq2, sxk, wq, swi, out_dtype=torch.float32), y32)
     # accumulate into an fp32 buffer
     acc = torch.full((M, N), 1.5, dtype=torch.float32, device=gpu)
     hpfp8.gemm_blockwise(xq, sxi, wq, swi, out=acc, accumulate=True)
@@ -245,6 +248,7 @@ def test_grouped_leaves_rows_past_the_last_offset_alone(gpu):
     offs = torch.tensor([100, 260], dtype=torch.int32, device=gpu)
     from hpfp8 import _lib, ops
     out = torch.full((300, N), 7.0, dtype=torch.float32, device=gpu)
-    _lib.call("hpfp8_gemm_grouped_blockwise", xq.data_ptr(), sxi.data_ptr(), wq.data_ptr(), swi.data_ptr(),
-              offs.data_ptr(), 2, 300, N, K, out.data_ptr(), N, _lib.OUT_F32, ops._stream())
+    _lib.call("hpfp8_gemm_grouped_blockwise", xq.data_ptr(), sxi.data_ptr(), sxi.stride(0), sxi.stride(1),
+              wq.data_ptr(), swi.data_ptr(), offs.data_ptr(), 2, 300, N, K, out.data_ptr(), N, _lib.OUT_F32,
+              ops._stream())
     assert bool((out[260:] == 7.0).all()) and not bool((out[:260] == 7.0).any())

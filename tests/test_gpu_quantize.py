@@ -96,6 +96,24 @@ def test_seeded_parity_all_quantizers(gpu, shape, seed, std, of, om):
     assert np.array_equal(U.codes(qt), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
 
 
+@pytest.mark.parametrize("shape", [(512, 7168), (100, 384), (16, 128), (33, 640)])
+def test_kmajor_scale_layouts_hold_the_same_values(gpu, shape):
+    import hpfp8
+    x = U.randn_bf16(shape, 77, 1.0, 0.001, 50.0)
+    xg = x.to(gpu)
+    q, s, si = hpfp8.quantize_1x128(xg, want_scale=True)
+    qk, sk, sik = hpfp8.quantize_1x128(xg, want_scale=True, kmajor=True)
+    assert sik.shape == si.shape and sik.stride(0) == 1            # stored [C/128, rows]
+    assert torch.equal(q.view(torch.uint8), qk.view(torch.uint8)) and torch.equal(si, sik) and torch.equal(s, sk)
+    rq, rs, rsi = C.quantize_1x128(U.bits(x))
+    assert np.array_equal(U.codes(qk), rq) and eq_f32(sik, rsi) and eq_f32(sk, rs)
+    if shape[0] % 128 == 0:
+        qt, st, sit = hpfp8.quantize_128x1_t(xg, want_scale=True)
+        qtk, stk, sitk = hpfp8.quantize_128x1_t(xg, want_scale=True, kmajor=True)
+        assert sitk.stride(0) == 1 and torch.equal(qt.view(torch.uint8), qtk.view(torch.uint8))
+        assert torch.equal(sit, sitk) and torch.equal(st, stk)
+
+
 def test_laplace_gradients_and_transposed_identity(gpu):
     import hpfp8
     go = U.laplace_bf16((512, 896), seed=9, scale=1e-3)
