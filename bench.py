@@ -106,20 +106,20 @@ def main():
     # preallocated outputs: nothing is allocated inside the timed region
     FP8 = torch.float8_e4m3fn
     xq = torch.empty((M, K), dtype=FP8, device=dev)
-    sx = torch.empty((M, K // 128), dtype=torch.float32, device=dev)
+    sx = torch.empty((K // 128, M), dtype=torch.float32, device=dev)   # k-block-major: element (m, kb) at [kb, m]
     wq = torch.empty((N, K), dtype=FP8, device=dev)
     sw = torch.empty((N // 128, K // 128), dtype=torch.float32, device=dev)
     y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
 
     def q_act():
-        _lib.call("hpfp8_quantize_1x128_bf16", x.data_ptr(), M, K, xq.data_ptr(), None, sx.data_ptr(), stream)
+        _lib.call("hpfp8_quantize_1x128_kmajor_bf16", x.data_ptr(), M, K, xq.data_ptr(), None, sx.data_ptr(), stream)
 
     def q_wgt():
         _lib.call("hpfp8_quantize_128x128_bf16", w.data_ptr(), N, K, wq.data_ptr(), None, None, sw.data_ptr(), stream)
 
     def gemm():
-        _lib.call("hpfp8_gemm_blockwise", xq.data_ptr(), sx.data_ptr(), K // 128, 1, wq.data_ptr(), sw.data_ptr(),
+        _lib.call("hpfp8_gemm_blockwise", xq.data_ptr(), sx.data_ptr(), 1, M, wq.data_ptr(), sw.data_ptr(),
                   K // 128, 1, 128, M, N, K, None, y.data_ptr(), N, _lib.OUT_BF16, 0, stream)
 
     def ev():
@@ -153,7 +153,7 @@ def main():
     s0, s1 = ev(), ev()
     s0.record()
     for i in range(reps):
-        _lib.call("hpfp8_quantize_1x128_bf16", xs[i % 6].data_ptr(), M, K, xqs[i % 6].data_ptr(), None,
+        _lib.call("hpfp8_quantize_1x128_kmajor_bf16", xs[i % 6].data_ptr(), M, K, xqs[i % 6].data_ptr(), None,
                   sx.data_ptr(), stream)
     s1.record()
     torch.cuda.synchronize()
@@ -174,7 +174,7 @@ def main():
     # spot check inside the bench: the timed buffers hold the right answer (float64 reference on a slice)
     lut = torch.tensor([float(v) for v in torch.arange(256, dtype=torch.uint8).view(FP8).float().nan_to_num()],
                        dtype=torch.float64, device=dev)
-    a64 = lut[xq[:256].view(torch.uint8).long()] * sx[:256].double().repeat_interleave(128, dim=1)
+    a64 = lut[xq[:256].view(torch.uint8).long()] * sx.t()[:256].double().repeat_interleave(128, dim=1)
     b64 = lut[wq[:256].view(torch.uint8).long()] * sw[:2].double().repeat_interleave(128, dim=0).repeat_interleave(128, dim=1)
     ref = a64 @ b64.t()
     err = float((y[:256, :256].double() - ref).norm() / ref.norm())
@@ -219,7 +219,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         import numpy as np
-        xb = x[:1024].cpu().view(torch.int16).numpy().view(np.uint16)
+        xb = x[:2048].cpu().view(torch.int16).numpy().view(np.uint16)
         wb = w.cpu().view(torch.int16).numpy().view(np.uint16)
         out["cpu_baseline"] = cpu_baseline(xb, wb)
     print(json.dumps(out))

@@ -24,6 +24,7 @@ constexpr int kGemmThreads = 512;
 constexpr int kTileBytes = 256 * BK;          // one operand tile in LDS
 constexpr int kStageBytes = 2 * kTileBytes;   // a tile then b tile
 constexpr int kXcds = 8;
+constexpr int kGroupM = 8, kGroupN = 4;   // tile rectangle one XCD works on at a time
 
 enum ScaleMode { kScaleTensor = 0, kScaleBlock = 1, kScaleRow = 2 };
 
@@ -120,8 +121,19 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   } else {
     const int tiles_m = (p.M + BM - 1) / BM;
     if (t >= tiles_m * tiles_n) return;
-    tn = t / tiles_m;
-    row0 = (t % tiles_m) * BM;
+    // Consecutive tile ids (one XCD's CUs at any moment) cover kGroupM x kGroupN rectangles of
+    // tiles, so the L2 of that XCD serves each activation / weight panel to several CUs.
+    const int per_ngroup = kGroupN * tiles_m;
+    const int ng = t / per_ngroup, rest = t % per_ngroup;
+    const int gn = (tiles_n - ng * kGroupN) < kGroupN ? (tiles_n - ng * kGroupN) : kGroupN;   // last group may be narrow
+    const int mg = rest / (kGroupM * gn), rest2 = rest % (kGroupM * gn);
+    const int gm = (tiles_m - mg * kGroupM) < kGroupM ? (tiles_m - mg * kGroupM) : kGroupM;
+    // inside a rectangle: n fastest
+    int tm_local, tn_local;
+    if (gm == kGroupM) { tm_local = rest2 / gn; tn_local = rest2 % gn; }
+    else { const int r3 = rest - mg * kGroupM * gn; tm_local = r3 / gn; tn_local = r3 % gn; }
+    tn = ng * kGroupN + tn_local;
+    row0 = (mg * kGroupM + tm_local) * BM;
     row_end = p.M;
   }
   const int n0 = tn * BN;
@@ -142,15 +154,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     a_off[i] = (uint32_t)(row0 + r) * (uint32_t)K + chunk * 16;
     b_off[i] = (uint32_t)(n0 + r) * (uint32_t)K + chunk * 16;
   }
-  auto issue_tile_loads = [&](int kb, int stage) {
-    uint8_t* sbase = lds + stage * kStageBytes + wave * 4096;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sbase + i * 1024), 16, a_off[i],
+  // One of a wave's 8 transfers for k-block kb: even idx -> a tile, odd idx -> b tile.
+  auto issue_tile_load = [&](int kb, int stage, int idx) {
+    uint8_t* sbase = lds + stage * kStageBytes + wave * 4096 + (idx >> 1) * 1024;
+    if (idx & 1)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sbase + kTileBytes), 16, b_off[idx >> 1],
                                                kb * BK, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sbase + kTileBytes + i * 1024), 16,
-                                               b_off[i], kb * BK, 0, 0);
-    }
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)sbase, 16, a_off[idx >> 1], kb * BK, 0, 0);
+  };
+  auto issue_tile_loads = [&](int kb, int stage) {
+#pragma unroll
+    for (int idx = 0; idx < 8; ++idx) issue_tile_load(kb, stage, idx);
   };
 
   // ---- fragment addressing
@@ -170,15 +185,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   const float* sbp = p.sb + (GROUPED ? (int64_t)expert * p.sb_se : 0);
   int nblk_idx = (n0 + wn * 128) >> 7;
   if (nblk_idx > (N >> 7) - 1) nblk_idx = (N >> 7) - 1;
-  auto load_scales = [&](int kb, float s[4]) {
-    if (MODE == kScaleBlock) {
-      const float sbv = sbp[(int64_t)nblk_idx * p.sb_sn + (int64_t)kb * p.sb_sk];
+  // Raw scale values for one k-block: the loads are issued at the top of the round before it and
+  // only combined (sa * sb) at its end, so nothing waits on global memory in between.
+  auto load_scales = [&](int kb, float raw[5]) {
+    if (MODE == kScaleBlock) raw[4] = sbp[(int64_t)nblk_idx * p.sb_sn + (int64_t)kb * p.sb_sk];
+    if (MODE != kScaleTensor) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[j] = p.sa[(int64_t)arow[j] * p.sa_sm + (int64_t)kb * p.sa_sk] * sbv;
-    } else if (MODE == kScaleRow) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) s[j] = p.sa[(int64_t)arow[j] * p.sa_sm + (int64_t)kb * p.sa_sk];
+      for (int j = 0; j < 4; ++j) raw[j] = p.sa[(int64_t)arow[j] * p.sa_sm + (int64_t)kb * p.sa_sk];
     }
+  };
+  auto combine_scales = [&](const float raw[5], float s[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s[j] = MODE == kScaleBlock ? raw[j] * raw[4] : raw[j];
   };
 
   v4f acc[8][4];
@@ -187,18 +205,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_nxt[4] = {1.f, 1.f, 1.f, 1.f};
-  load_scales(0, s_cur);
+  float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_raw[5] = {1.f, 1.f, 1.f, 1.f, 1.f};
+  load_scales(0, s_raw);
+  combine_scales(s_raw, s_cur);
   issue_tile_loads(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
 
   for (int kb = 0; kb < kblocks; ++kb) {
     const int stage = kb & 1;
-    if (kb + 1 < kblocks) {
-      issue_tile_loads(kb + 1, stage ^ 1);
-      load_scales(kb + 1, s_nxt);
-    }
+    // The 8 tile transfers for the next k-block are issued one per n-subtile inside the compute
+    // loop instead of as a burst here: a burst of 64 transfers per CU queues up in the texture
+    // path and holds every wave back before its first LDS read.
+    // They are issued for the round after the last one too (into the stage nobody reads again;
+    // addresses past the tensor read as zero), which keeps the loop body free of branches.
+    load_scales(kb + 1 < kblocks ? kb + 1 : kb, s_raw);
+    __builtin_amdgcn_sched_barrier(0);
     const uint8_t* sbase = lds + stage * kStageBytes;
     v8i xf[4];
     if (MODE == kScaleBlock) {
@@ -208,18 +230,21 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       // subtile i+1 are issued before the MFMAs of subtile i (a full subtile of latency cover).
       const v4f zero = {0.f, 0.f, 0.f, 0.f};
       v4f part[2][4];
-      v8i wf = frag_read(sbase + b_frag_off, pc0);
+      // weight fragments are read two subtiles ahead of their use (three live at a time)
+      v8i wf[3];
+      wf[0] = frag_read(sbase + b_frag_off, pc0);
 #pragma unroll
       for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
+      wf[1] = frag_read(sbase + b_frag_off + 16 * BK, pc0);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        v8i wf_next = wf;
-        if (i + 1 < 8) wf_next = frag_read(sbase + b_frag_off + (i + 1) * 16 * BK, pc0);
+        if (i + 2 < 8) wf[(i + 2) % 3] = frag_read(sbase + b_frag_off + (i + 2) * 16 * BK, pc0);
+        issue_tile_load(kb + 1, stage ^ 1, i);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], zero, 0, 0, 0, 0, 0, 0);
+          part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i % 3], xf[j], zero, 0, 0, 0, 0, 0, 0);
           if (i > 0) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -227,7 +252,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
           }
           __builtin_amdgcn_sched_barrier(0);   // keep this (MFMA, 4 FMA) group together, in this order
         }
-        wf = wf_next;
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j)
@@ -239,6 +263,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const v8i wf = frag_read(sbase + b_frag_off + i * 16 * BK, pc0);
+        issue_tile_load(kb + 1, stage ^ 1, i);
+        __builtin_amdgcn_sched_barrier(0);
         float sbr[4] = {1.f, 1.f, 1.f, 1.f};
         if (MODE == kScaleRow) {
           int n = n0 + wn * 128 + i * 16 + g * 4;
@@ -260,10 +286,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
         }
       }
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) s_cur[j] = s_nxt[j];
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // own DMA for the next stage has landed
-    __syncthreads();                     // everyone's has, and everyone is done reading this stage
+    __builtin_amdgcn_sched_barrier(0);
+    combine_scales(s_raw, s_cur);
+    // own DMA for the next stage has landed and own LDS reads of this stage are done; then everyone's
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
   }
 
   // ---- epilogue

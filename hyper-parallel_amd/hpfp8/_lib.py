@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libhpfp8.so")
+# HPFP8_LIBRARY points at another build of the same C ABI (e.g. an instrumented one)
+LIB_PATH = os.environ.get("HPFP8_LIBRARY") or os.path.join(_HERE, "libhpfp8.so")
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
