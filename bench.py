@@ -27,8 +27,10 @@ for p in (ROOT, os.path.join(ROOT, "hyper-parallel_amd")):
 M, N, K = 4096, 36864, 7168
 PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
-# HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured
-GEMM_TRAFFIC_BYTES = None
+# Bytes per GEMM launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 1.9992 calibration + WRITE_SIZE, profiles/bench_cfg2_gemm_blockwise_and_quantizers.md):
+# 1,608,055 KiB fetched + 397,811 KiB written.  Algorithmic operand + output bytes are 582,591 KiB.
+GEMM_TRAFFIC_BYTES = (1608055 + 397811) * 1024
 
 
 def make_inputs(dev):
