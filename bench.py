@@ -118,10 +118,10 @@ def main():
         _lib.call("hpfp8_quantize_1x128_kmajor_bf16", x.data_ptr(), M, K, xq.data_ptr(), None, sx.data_ptr(), stream)
 
     def q_wgt():
-        _lib.call("hpfp8_quantize_128x128_bf16", w.data_ptr(), N, K, wq.data_ptr(), None, None, sw.data_ptr(), stream)
+        _lib.call("hpfp8_quantize_128x128_bf16", w.data_ptr(), N, K, wq.data_ptr(), None, 0, None, sw.data_ptr(), stream)
 
     def gemm():
-        _lib.call("hpfp8_gemm_blockwise", xq.data_ptr(), sx.data_ptr(), 1, M, wq.data_ptr(), sw.data_ptr(),
+        _lib.call("hpfp8_gemm_blockwise", xq.data_ptr(), K, sx.data_ptr(), 1, M, wq.data_ptr(), K, sw.data_ptr(),
                   K // 128, 1, 128, M, N, K, None, y.data_ptr(), N, _lib.OUT_BF16, 0, stream)
 
     def ev():

@@ -41,6 +41,7 @@ struct GemmParams {
   const uint16_t* bias;
   const int32_t* offs;    // grouped: inclusive prefix sums of rows per expert
   int experts;
+  int64_t lda, ldb;       // row strides of a and b in bytes (>= K)
   int M, N, K;            // M = total rows of a
   int accumulate;
 };
@@ -77,6 +78,8 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 template <int MODE, bool GROUPED, bool OUT_F32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageBytes];
+  // per-row scales of the b operand for one k-block (wgrad form), two stages of 256 floats
+  __shared__ __attribute__((aligned(16))) float sb_lds[MODE == kScaleRow ? 2 * BN : 4];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -140,20 +143,29 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 
   // ---- global -> LDS tile DMA.  One wave instruction moves 8 rows x 128 B (lane i -> LDS slot
   // i); the lane picks the 16-byte global chunk whose swizzled home is its slot.
-  const uint8_t* bbase = p.b + (GROUPED ? (int64_t)expert * N * K : 0);
+  const uint8_t* bbase = p.b + (GROUPED ? (int64_t)expert * N * p.ldb : 0);
   const __amdgpu_buffer_rsrc_t rsrc_a =
-      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)((int64_t)p.M * K), 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)((int64_t)p.M * p.lda), 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b =
-      __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, (int)((int64_t)N * K), 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, (int)((int64_t)N * p.ldb), 0x00020000);
   uint32_t a_off[4], b_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int q = wave * 4 + i;                       // 8-row group inside the tile
     const int r = q * 8 + (lane >> 3);                // row inside the tile
     const int chunk = (lane & 7) ^ row_swizzle(r);    // logical 16-byte chunk of that row
-    a_off[i] = (uint32_t)(row0 + r) * (uint32_t)K + chunk * 16;
-    b_off[i] = (uint32_t)(n0 + r) * (uint32_t)K + chunk * 16;
+    a_off[i] = (uint32_t)(row0 + r) * (uint32_t)p.lda + chunk * 16;
+    b_off[i] = (uint32_t)(n0 + r) * (uint32_t)p.ldb + chunk * 16;
   }
+  // wgrad form: the 256 per-row scales of the b tile for one k-block are one more 1 KB transfer
+  // (wave 0), possible because that scale array is k-block-major (unit stride over rows).
+  const __amdgpu_buffer_rsrc_t rsrc_sb = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)p.sb, 0, MODE == kScaleRow ? (int)((((int64_t)kblocks - 1) * p.sb_sk + N) * 4) : 0, 0x00020000);
+  auto issue_sb_load = [&](int kb, int stage) {
+    if (MODE == kScaleRow && wave == 0)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sb, (lds_ptr_t)(sb_lds + stage * BN), 16,
+                                               (uint32_t)(n0 + lane * 4) * 4u, (int)(kb * p.sb_sk * 4), 0, 0);
+  };
   // One of a wave's 8 transfers for k-block kb: even idx -> a tile, odd idx -> b tile.
   auto issue_tile_load = [&](int kb, int stage, int idx) {
     uint8_t* sbase = lds + stage * kStageBytes + wave * 4096 + (idx >> 1) * 1024;
@@ -209,6 +221,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   load_scales(0, s_raw);
   combine_scales(s_raw, s_cur);
   issue_tile_loads(0, 0);
+  issue_sb_load(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
 
@@ -223,7 +236,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     __builtin_amdgcn_sched_barrier(0);
     const uint8_t* sbase = lds + stage * kStageBytes;
     v8i xf[4];
-    if (MODE == kScaleBlock) {
+    if (MODE != kScaleTensor) {
       // Software pipeline over the 8 n-subtiles: the matrix instructions of subtile i are issued
       // interleaved with the promotion FMAs of subtile i-1, whose partial sums left the matrix
       // pipe four instructions earlier, so neither pipe waits for the other.  The LDS reads of
@@ -236,10 +249,16 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
       for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
       wf[1] = frag_read(sbase + b_frag_off + 16 * BK, pc0);
+      // wgrad form: the four per-row b scales of subtile i for this lane's four n
+      const float* sb_row = sb_lds + stage * BN + wn * 128 + g * 4;
+      v4f sbv[2];
+      if (MODE == kScaleRow) sbv[0] = *reinterpret_cast<const v4f*>(sb_row);
+      if (MODE == kScaleRow && wave == 0) issue_sb_load(kb + 1 < kblocks ? kb + 1 : kb, stage ^ 1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if (i + 2 < 8) wf[(i + 2) % 3] = frag_read(sbase + b_frag_off + (i + 2) * 16 * BK, pc0);
+        if (MODE == kScaleRow && i > 0) sbv[i & 1] = *reinterpret_cast<const v4f*>(sb_row + i * 16);   // used by the FMAs of group i+1
         issue_tile_load(kb + 1, stage ^ 1, i);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -247,16 +266,23 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
           part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i % 3], xf[j], zero, 0, 0, 0, 0, 0, 0);
           if (i > 0) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              acc[i - 1][j][r] = __builtin_fmaf(part[(i - 1) & 1][j][r], s_cur[j], acc[i - 1][j][r]);
+            for (int r = 0; r < 4; ++r) {
+              float pv = part[(i - 1) & 1][j][r];
+              if (MODE == kScaleRow) pv *= sbv[(i - 1) & 1][r];
+              acc[i - 1][j][r] = __builtin_fmaf(pv, s_cur[j], acc[i - 1][j][r]);
+            }
           }
-          __builtin_amdgcn_sched_barrier(0);   // keep this (MFMA, 4 FMA) group together, in this order
+          __builtin_amdgcn_sched_barrier(0);   // keep this (MFMA, FMAs) group together, in this order
         }
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[7][j][r] = __builtin_fmaf(part[1][j][r], s_cur[j], acc[7][j][r]);
+        for (int r = 0; r < 4; ++r) {
+          float pv = part[1][j][r];
+          if (MODE == kScaleRow) pv *= sbv[1][r];
+          acc[7][j][r] = __builtin_fmaf(pv, s_cur[j], acc[7][j][r]);
+        }
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
@@ -265,25 +291,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
         const v8i wf = frag_read(sbase + b_frag_off + i * 16 * BK, pc0);
         issue_tile_load(kb + 1, stage ^ 1, i);
         __builtin_amdgcn_sched_barrier(0);
-        float sbr[4] = {1.f, 1.f, 1.f, 1.f};
-        if (MODE == kScaleRow) {
-          int n = n0 + wn * 128 + i * 16 + g * 4;
-          if (n > N - 4) n = N - 4;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) sbr[r] = p.sb[(int64_t)(n + r) * p.sb_sn + (int64_t)kb * p.sb_sk];
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (MODE == kScaleTensor) {
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
-          } else {
-            const v4f zero = {0.f, 0.f, 0.f, 0.f};
-            v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], zero, 0, 0, 0, 0, 0, 0);
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              acc[i][j][r] = __builtin_fmaf(part[r], s_cur[j] * sbr[r], acc[i][j][r]);
-          }
-        }
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -344,15 +354,18 @@ static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t 
   return check_launch("gemm");
 }
 
-static int check_common(const char* what, const void* a, const void* b, const float* sa, const float* sb,
-                        int64_t M, int64_t N, int64_t K, const void* bias, const void* c, int64_t ldc,
-                        int out_type, int accumulate) {
+static int check_common(const char* what, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                        const float* sb, int64_t M, int64_t N, int64_t K, const void* bias, const void* c,
+                        int64_t ldc, int out_type, int accumulate) {
   HPFP8_REQUIRE(M >= 0 && N >= 0 && K >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(K > 0 && K % BK == 0 && N % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: K=%lld must be a positive multiple of 128 and N=%lld a multiple of 128", what, (long long)K,
                 (long long)N);
   HPFP8_REQUIRE(out_type == HPFP8_OUT_BF16 || out_type == HPFP8_OUT_F32, HPFP8_ERR_ARG, "%s: bad out_type", what);
   HPFP8_REQUIRE(!accumulate || out_type == HPFP8_OUT_F32, HPFP8_ERR_ARG, "%s: accumulate needs fp32 output", what);
+  HPFP8_REQUIRE(lda >= K && ldb >= K && lda % 16 == 0 && ldb % 16 == 0, HPFP8_ERR_SHAPE,
+                "%s: lda=%lld and ldb=%lld must be multiples of 16 and at least K=%lld", what, (long long)lda,
+                (long long)ldb, (long long)K);
   HPFP8_REQUIRE(ldc >= N, HPFP8_ERR_SHAPE, "%s: ldc=%lld smaller than N=%lld", what, (long long)ldc, (long long)N);
   HPFP8_REQUIRE(ldc % 4 == 0, HPFP8_ERR_ALIGN, "%s: ldc must be a multiple of 4", what);
   if (M == 0 || N == 0) return HPFP8_OK;
@@ -360,7 +373,7 @@ static int check_common(const char* what, const void* a, const void* b, const fl
   HPFP8_REQUIRE(aligned16(a) && aligned16(b) && aligned16(c) && (!bias || aligned16(bias)), HPFP8_ERR_ALIGN,
                 "%s: buffers must be 16-byte aligned", what);
   // 32-bit byte offsets inside the tile loader, including rows read past the end of a tile
-  HPFP8_REQUIRE((M + BM) * K < (int64_t)0x7FFFFFFF && (N + BN) * K < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
+  HPFP8_REQUIRE((M + BM) * lda < (int64_t)0x7FFFFFFF && (N + BN) * ldb < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
                 "%s: an operand exceeds 2 GiB", what);
   return 1;
 }
@@ -371,47 +384,53 @@ using namespace hpfp8;
 
 extern "C" {
 
-int hpfp8_gemm_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
-                         const void* b, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                         const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
                          int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
                          int64_t ldc, int out_type, int accumulate, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(sb_gran == 1 || sb_gran == 128, HPFP8_ERR_ARG, "gemm_blockwise: sb_gran must be 1 or 128");
-  int rc = check_common("gemm_blockwise", a, b, sa, sb, M, N, K, bias, c, ldc, out_type, accumulate);
+  int rc = check_common("gemm_blockwise", a, lda, b, ldb, sa, sb, M, N, K, bias, c, ldc, out_type, accumulate);
   if (rc <= 0) return rc;
   GemmParams p{};
-  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb;
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = ldb;
   p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k; p.sb_sn = sb_stride_n; p.sb_sk = sb_stride_k;
   p.c = c; p.ldc = ldc; p.bias = (const uint16_t*)bias;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.accumulate = accumulate;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (sb_gran == 128) return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
+  // per-row b scales travel to LDS as one contiguous 1 KB piece per k-block
+  HPFP8_REQUIRE(sb_stride_n == 1 && sb_stride_k >= N && sb_stride_k % 4 == 0 && aligned16(sb), HPFP8_ERR_SHAPE,
+                "gemm_blockwise: with sb_gran=1 the b scales must be k-block-major (sb_stride_n = 1, sb_stride_k >= N, "
+                "16-byte aligned rows)");
+  HPFP8_REQUIRE(((K / BK - 1) * sb_stride_k + N) * 4 < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
+                "gemm_blockwise: b scale array too large");
   return launch<kScaleRow, false>(p, out_type, tiles, (hipStream_t)stream);
 }
 
-int hpfp8_gemm_per_tensor(const void* a, const float* sa_inv, const void* b, const float* sb_inv,
-                          int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
-                          int out_type, hpfp8_stream_t stream) {
-  int rc = check_common("gemm_per_tensor", a, b, sa_inv, sb_inv, M, N, K, bias, c, ldc, out_type, 0);
+int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,
+                          const float* sb_inv, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
+                          int64_t ldc, int out_type, hpfp8_stream_t stream) {
+  int rc = check_common("gemm_per_tensor", a, lda, b, ldb, sa_inv, sb_inv, M, N, K, bias, c, ldc, out_type, 0);
   if (rc <= 0) return rc;
   GemmParams p{};
-  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa_inv; p.sb = sb_inv;
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa_inv; p.sb = sb_inv; p.lda = lda; p.ldb = ldb;
   p.c = c; p.ldc = ldc; p.bias = (const uint16_t*)bias;
   p.M = (int)M; p.N = (int)N; p.K = (int)K;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   return launch<kScaleTensor, false>(p, out_type, tiles, (hipStream_t)stream);
 }
 
-int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                                  const void* b, const float* sb, const int32_t* offs, int experts,
                                  int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
                                  hpfp8_stream_t stream) {
   HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "gemm_grouped: bad expert count %d", experts);
-  int rc = check_common("gemm_grouped", a, b, sa, sb, total_m, N, K, nullptr, c, ldc, out_type, 0);
+  int rc = check_common("gemm_grouped", a, lda, b, K, sa, sb, total_m, N, K, nullptr, c, ldc, out_type, 0);
   if (rc <= 0) return rc;
   if (experts == 0) return HPFP8_OK;
   HPFP8_REQUIRE(offs != nullptr, HPFP8_ERR_ARG, "gemm_grouped: null offs");
   GemmParams p{};
-  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb;
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = K;
   p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k;
   p.sb_sn = K / BK; p.sb_sk = 1; p.sb_se = (N / kBlock) * (K / BK);
   p.c = c; p.ldc = ldc; p.offs = offs; p.experts = experts;

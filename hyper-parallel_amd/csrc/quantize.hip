@@ -191,49 +191,73 @@ __device__ __forceinline__ void store_tile_transposed(uint8_t* tile, const uint2
 // ---------------------------------------------------------------------------------------------
 // 128x128 blocks (weights), optional transposed copy of the codes for dgrad
 // ---------------------------------------------------------------------------------------------
+constexpr int kTilesPerBlock = 4;   // tiles a workgroup of the transposing kernels walks through
+
 template <bool WITH_T>
 __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __restrict__ w, int rows,
                                                             int cols, uint8_t* __restrict__ q,
-                                                            uint8_t* __restrict__ qt,
+                                                            uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale,
                                                             float* __restrict__ scale_inv) {
-  const int cb = cols >> 7;
-  const int bc = blockIdx.x % cb, br = blockIdx.x / cb;
+  const int cb = cols >> 7, rb = rows >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
-  const int64_t tile_off = (int64_t)br * 128 * cols + bc * 128 + cg * 8;
-  uint4 v[8];
-#pragma unroll
-  for (int p = 0; p < 8; ++p)
-    v[p] = nt_load16(w + tile_off + (int64_t)tile_row(rq, p) * cols);
-  uint32_t m = 0;
-#pragma unroll
-  for (int p = 0; p < 8; ++p) m = umax(m, mag8(v[p]));
-  m = row16_max_u32(m);
   __shared__ uint32_t part[16];
   __shared__ float s_scale;
-  if (cg == 0) part[rq] = m;
-  __syncthreads();
-  if (threadIdx.x < 16) {
-    m = row16_max_u32(part[threadIdx.x]);
-    if (threadIdx.x == 0) {
-      float s, si;
-      scales_from_amax(__uint_as_float(m << 16), s, si);
-      s_scale = s;
-      if (scale) scale[blockIdx.x] = s;
-      scale_inv[blockIdx.x] = si;
-    }
-  }
-  __syncthreads();
-  const float s = s_scale;
-  uint2 c[8];
+  __shared__ __attribute__((aligned(16))) uint8_t tile[WITH_T ? 128 * 128 : 16];
+  // Without a transposed copy: one tile per workgroup, row-major tile order.  With it: a workgroup
+  // walks kTilesPerBlock tiles down a block column, loading tile t+1 before the LDS phases of tile
+  // t, and its consecutive 128-byte pieces of each transposed row are neighbours in memory.
+  const int total = rb * cb;
+  const int t0 = WITH_T ? blockIdx.x * kTilesPerBlock : blockIdx.x;
+  const int t1 = WITH_T ? (t0 + kTilesPerBlock < total ? t0 + kTilesPerBlock : total) : t0 + 1;
+  auto tile_pos = [&](int t, int& br, int& bc) {
+    if (WITH_T) { bc = t / rb; br = t % rb; } else { bc = t % cb; br = t / cb; }
+  };
+  auto load_tile = [&](int t, uint4 v[8]) {
+    int br, bc;
+    tile_pos(t, br, bc);
+    const int64_t off = (int64_t)br * 128 * cols + bc * 128 + cg * 8;
 #pragma unroll
-  for (int p = 0; p < 8; ++p) {
-    c[p] = cvt8(v[p], s);
-    *reinterpret_cast<uint2*>(q + tile_off + (int64_t)tile_row(rq, p) * cols) = c[p];
-  }
-  if (WITH_T) {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
-    store_tile_transposed(tile, c, cg, rq, qt + (int64_t)bc * 128 * rows + br * 128, rows);
+    for (int p = 0; p < 8; ++p) v[p] = nt_load16(w + off + (int64_t)tile_row(rq, p) * cols);
+  };
+  uint4 v[8], vn[8];
+  load_tile(t0, v);
+  for (int t = t0; t < t1; ++t) {
+    if (WITH_T && t + 1 < t1) load_tile(t + 1, vn);
+    int br, bc;
+    tile_pos(t, br, bc);
+    const int sidx = br * cb + bc;
+    const int64_t tile_off = (int64_t)br * 128 * cols + bc * 128 + cg * 8;
+    uint32_t m = 0;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) m = umax(m, mag8(v[p]));
+    m = row16_max_u32(m);
+    if (cg == 0) part[rq] = m;
+    __syncthreads();
+    if (threadIdx.x < 16) {
+      m = row16_max_u32(part[threadIdx.x]);
+      if (threadIdx.x == 0) {
+        float s, si;
+        scales_from_amax(__uint_as_float(m << 16), s, si);
+        s_scale = s;
+        if (scale) scale[sidx] = s;
+        scale_inv[sidx] = si;
+      }
+    }
+    __syncthreads();
+    const float s = s_scale;
+    uint2 c[8];
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      c[p] = cvt8(v[p], s);
+      *reinterpret_cast<uint2*>(q + tile_off + (int64_t)tile_row(rq, p) * cols) = c[p];
+    }
+    if (WITH_T) {
+      store_tile_transposed(tile, c, cg, rq, qt + (int64_t)bc * 128 * ld_t + br * 128, ld_t);
+      __syncthreads();   // the LDS tile, part[] and s_scale are reused by the next tile
+#pragma unroll
+      for (int p = 0; p < 8; ++p) v[p] = vn[p];
+    }
   }
 }
 
@@ -242,73 +266,86 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // ---------------------------------------------------------------------------------------------
 template <bool KMAJOR>
 __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int m, int k,
-                                                            uint8_t* __restrict__ qt,
+                                                            uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale_t,
                                                             float* __restrict__ scale_inv_t) {
-  const int kb = k >> 7;
-  const int tc = blockIdx.x % kb, tr = blockIdx.x / kb;
+  const int kb = k >> 7, mb = m >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
-  const int mb = m >> 7;
-  const int64_t tile_off = (int64_t)tr * 128 * k + tc * 128 + cg * 8;
-  uint4 v[8];
-#pragma unroll
-  for (int p = 0; p < 8; ++p)
-    v[p] = nt_load16(x + tile_off + (int64_t)tile_row(rq, p) * k);
-  // per-column magnitudes over this thread's 8 rows, two columns per word
-  uint32_t cm[4] = {0, 0, 0, 0};
-#pragma unroll
-  for (int p = 0; p < 8; ++p) {
-    cm[0] = pk_max_u16(cm[0], v[p].x & 0x7FFF7FFFu);
-    cm[1] = pk_max_u16(cm[1], v[p].y & 0x7FFF7FFFu);
-    cm[2] = pk_max_u16(cm[2], v[p].z & 0x7FFF7FFFu);
-    cm[3] = pk_max_u16(cm[3], v[p].w & 0x7FFF7FFFu);
-  }
-  // across the 4 row quads inside the wave (lanes differing in bits 4 and 5)
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 16));
-    cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 32));
-  }
+  const int wave = threadIdx.x >> 6;
   __shared__ uint32_t part[4][64];  // [wave][cg*4 + word]
   __shared__ float s_scale[128];
-  const int wave = threadIdx.x >> 6;
-  if ((threadIdx.x & 63) < 16) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
+  // A workgroup walks kTilesPerBlock tiles down a tile column (tr fastest), loading tile t+1 before
+  // the LDS phases of tile t.
+  const int total = kb * mb;
+  const int t0 = blockIdx.x * kTilesPerBlock;
+  const int t1 = t0 + kTilesPerBlock < total ? t0 + kTilesPerBlock : total;
+  auto load_tile = [&](int t, uint4 v[8]) {
+    const int tc = t / mb, tr = t % mb;
+    const int64_t off = (int64_t)tr * 128 * k + tc * 128 + cg * 8;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) part[wave][cg * 4 + i] = cm[i];
-  }
-  __syncthreads();
-  if (threadIdx.x < 128) {
-    const int col = threadIdx.x, word = col >> 1;
-    uint32_t mw = pk_max_u16(pk_max_u16(part[0][word], part[1][word]), pk_max_u16(part[2][word], part[3][word]));
-    uint32_t mag = (col & 1) ? (mw >> 16) : (mw & 0xFFFFu);
-    float s, si;
-    scales_from_amax(__uint_as_float(mag << 16), s, si);
-    s_scale[col] = s;
-    // row-major [k, m/128], or block-major [m/128, k] (unit stride over the output rows)
-    int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
-    if (scale_t) scale_t[o] = s;
-    scale_inv_t[o] = si;
-  }
-  __syncthreads();
-  float sc[8];
+    for (int p = 0; p < 8; ++p) v[p] = nt_load16(x + off + (int64_t)tile_row(rq, p) * k);
+  };
+  uint4 v[8], vn[8];
+  load_tile(t0, v);
+  for (int t = t0; t < t1; ++t) {
+    if (t + 1 < t1) load_tile(t + 1, vn);
+    const int tc = t / mb, tr = t % mb;
+    // per-column magnitudes over this thread's 8 rows, two columns per word
+    uint32_t cm[4] = {0, 0, 0, 0};
 #pragma unroll
-  for (int j = 0; j < 8; ++j) sc[j] = s_scale[cg * 8 + j];
-  uint2 c[8];
-#pragma unroll
-  for (int p = 0; p < 8; ++p) {
-    const uint32_t ws[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
-    uint32_t pk[4];
+    for (int p = 0; p < 8; ++p) {
+      cm[0] = pk_max_u16(cm[0], v[p].x & 0x7FFF7FFFu);
+      cm[1] = pk_max_u16(cm[1], v[p].y & 0x7FFF7FFFu);
+      cm[2] = pk_max_u16(cm[2], v[p].z & 0x7FFF7FFFu);
+      cm[3] = pk_max_u16(cm[3], v[p].w & 0x7FFF7FFFu);
+    }
+    // across the 4 row quads inside the wave (lanes differing in bits 4 and 5)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float a = clamp448(bf16lo(ws[i]) * sc[2 * i]);
-      float b = clamp448(bf16hi(ws[i]) * sc[2 * i + 1]);
-      pk[i] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
+      cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 16));
+      cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 32));
     }
-    c[p].x = pk[0] | (pk[1] << 16);
-    c[p].y = pk[2] | (pk[3] << 16);
+    if ((threadIdx.x & 63) < 16) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[wave][cg * 4 + i] = cm[i];
+    }
+    __syncthreads();
+    if (threadIdx.x < 128) {
+      const int col = threadIdx.x, word = col >> 1;
+      uint32_t mw = pk_max_u16(pk_max_u16(part[0][word], part[1][word]), pk_max_u16(part[2][word], part[3][word]));
+      uint32_t mag = (col & 1) ? (mw >> 16) : (mw & 0xFFFFu);
+      float s, si;
+      scales_from_amax(__uint_as_float(mag << 16), s, si);
+      s_scale[col] = s;
+      // row-major [k, m/128], or block-major [m/128, k] (unit stride over the output rows)
+      int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
+      if (scale_t) scale_t[o] = s;
+      scale_inv_t[o] = si;
+    }
+    __syncthreads();
+    float sc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sc[j] = s_scale[cg * 8 + j];
+    uint2 c[8];
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const uint32_t ws[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
+      uint32_t pk[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float a = clamp448(bf16lo(ws[i]) * sc[2 * i]);
+        float b = clamp448(bf16hi(ws[i]) * sc[2 * i + 1]);
+        pk[i] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
+      }
+      c[p].x = pk[0] | (pk[1] << 16);
+      c[p].y = pk[2] | (pk[3] << 16);
+    }
+    store_tile_transposed(tile, c, cg, rq, qt + (int64_t)tc * 128 * ld_t + tr * 128, ld_t);
+    __syncthreads();   // the LDS tile, part[] and s_scale are reused by the next tile
+#pragma unroll
+    for (int p = 0; p < 8; ++p) v[p] = vn[p];
   }
-  __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
-  store_tile_transposed(tile, c, cg, rq, qt + (int64_t)tc * 128 * m + tr * 128, m);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -317,33 +354,45 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
 // out = bf16(decode(q) * scale_inv); if grad_scale != 1 the bf16 value is multiplied by it and
 // rounded again, the order of the reference's cast-back site
 // (hyper_parallel/core/hsdp/hsdp_grad_buffer.py:121-125).
-__global__ __launch_bounds__(256) void dequant_1x128_kernel(const uint4* __restrict__ q,
+template <int UNROLL>
+__global__ __launch_bounds__(256) void dequant_1x128_kernel(const uint2* __restrict__ q,
                                                             const float* __restrict__ scale_inv,
                                                             uint4* __restrict__ out, int64_t nvec,
                                                             float grad_scale, int apply_grad_scale) {
-  // nvec counts 16-code vectors; 8 of them per group.  One thread: 16 codes -> 2 x uint4 of bf16.
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= nvec) return;
-  uint4 c = nt_load16(&q[i]);
-  const float si = scale_inv[i >> 3];
-  const uint32_t words[4] = {c.x, c.y, c.z, c.w};
-  uint32_t o[8];
+  // nvec counts 8-code vectors (16 per group).  One thread: 8 codes -> one uint4 of bf16, so both the
+  // 64-bit loads and the 128-bit stores of a wave are contiguous.
+  const int64_t base = (int64_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  uint2 c[UNROLL];
+  float si[UNROLL];
 #pragma unroll
-  for (int wd = 0; wd < 4; ++wd) {
-    v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], false);
-    v2f hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], true);
-    float f[4] = {lo.x * si, lo.y * si, hi.x * si, hi.y * si};
-    __bf16 b[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      b[e] = (__bf16)f[e];
-      if (apply_grad_scale) b[e] = (__bf16)((float)b[e] * grad_scale);
-    }
-    o[2 * wd] = (uint32_t)__builtin_bit_cast(uint16_t, b[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, b[1]) << 16);
-    o[2 * wd + 1] = (uint32_t)__builtin_bit_cast(uint16_t, b[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, b[3]) << 16);
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t i = base + u * 256;
+    const bool ok = i < nvec;
+    u32x2 t = ok ? __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(&q[i])) : u32x2{0u, 0u};
+    c[u] = make_uint2(t.x, t.y);
+    si[u] = ok ? scale_inv[i >> 4] : 0.f;
   }
-  nt_store16(&out[2 * i], make_uint4(o[0], o[1], o[2], o[3]));
-  nt_store16(&out[2 * i + 1], make_uint4(o[4], o[5], o[6], o[7]));
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t i = base + u * 256;
+    const uint32_t words[2] = {c[u].x, c[u].y};
+    uint32_t o[4];
+#pragma unroll
+    for (int wd = 0; wd < 2; ++wd) {
+      v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], false);
+      v2f hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], true);
+      float f[4] = {lo.x * si[u], lo.y * si[u], hi.x * si[u], hi.y * si[u]};
+      __bf16 b[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        b[e] = (__bf16)f[e];
+        if (apply_grad_scale) b[e] = (__bf16)((float)b[e] * grad_scale);
+      }
+      o[2 * wd] = (uint32_t)__builtin_bit_cast(uint16_t, b[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, b[1]) << 16);
+      o[2 * wd + 1] = (uint32_t)__builtin_bit_cast(uint16_t, b[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, b[3]) << 16);
+    }
+    if (i < nvec) nt_store16(&out[i], make_uint4(o[0], o[1], o[2], o[3]));
+  }
 }
 
 // codes with one scale per 128x128 block (weights) -> bf16
@@ -454,8 +503,8 @@ int hpfp8_quantize_1x128_kmajor_bf16(const void* x, int64_t rows, int64_t cols, 
   return check_launch("quantize_1x128_kmajor");
 }
 
-int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, float* scale,
-                                float* scale_inv, hpfp8_stream_t stream) {
+int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
+                                float* scale, float* scale_inv, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_128x128: negative shape");
   HPFP8_REQUIRE(rows % kBlock == 0 && cols % kBlock == 0, HPFP8_ERR_SHAPE,
                 "quantize_128x128: shape [%lld, %lld] is not a multiple of 128", (long long)rows, (long long)cols);
@@ -466,18 +515,20 @@ int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void*
   HPFP8_REQUIRE(w && q && scale_inv, HPFP8_ERR_ARG, "quantize_128x128: null buffer");
   HPFP8_REQUIRE(aligned16(w) && aligned16(q) && (!q_t || aligned16(q_t)), HPFP8_ERR_ALIGN,
                 "quantize_128x128: buffers must be 16-byte aligned");
+  HPFP8_REQUIRE(!q_t || (ld_t >= rows && ld_t % 16 == 0), HPFP8_ERR_SHAPE,
+                "quantize_128x128: ld_t=%lld must be a multiple of 16 and at least rows", (long long)ld_t);
   hipStream_t s = (hipStream_t)stream;
   if (q_t)
-    quant_128x128_kernel<true><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
-                                                                (uint8_t*)q, (uint8_t*)q_t, scale, scale_inv);
+    quant_128x128_kernel<true><<<(unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock), 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
+                                                                (uint8_t*)q, (uint8_t*)q_t, ld_t, scale, scale_inv);
   else
     quant_128x128_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
-                                                                 (uint8_t*)q, nullptr, scale, scale_inv);
+                                                                 (uint8_t*)q, nullptr, 0, scale, scale_inv);
   return check_launch("quantize_128x128");
 }
 
 static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, int64_t m, int64_t k, void* q_t,
-                                 float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
+                                 int64_t ld_t, float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)m, (long long)k);
@@ -487,24 +538,26 @@ static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, i
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
   HPFP8_REQUIRE(x && q_t && scale_inv_t, HPFP8_ERR_ARG, "%s: null buffer", what);
   HPFP8_REQUIRE(aligned16(x) && aligned16(q_t), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
+  HPFP8_REQUIRE(ld_t >= m && ld_t % 16 == 0, HPFP8_ERR_SHAPE, "%s: ld_t=%lld must be a multiple of 16 and at least m",
+                what, (long long)ld_t);
   hipStream_t s = (hipStream_t)stream;
   if (kmajor)
-    quant_128x1_t_kernel<true><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
-                                                                 scale_t, scale_inv_t);
+    quant_128x1_t_kernel<true><<<(unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock), 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
+                                                                 ld_t, scale_t, scale_inv_t);
   else
-    quant_128x1_t_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
-                                                                  scale_t, scale_inv_t);
+    quant_128x1_t_kernel<false><<<(unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock), 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
+                                                                  ld_t, scale_t, scale_inv_t);
   return check_launch(what);
 }
 
-int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
+int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t, float* scale_t,
                                 float* scale_inv_t, hpfp8_stream_t stream) {
-  return quantize_128x1_t_impl("quantize_128x1_t", false, x, m, k, q_t, scale_t, scale_inv_t, stream);
+  return quantize_128x1_t_impl("quantize_128x1_t", false, x, m, k, q_t, ld_t, scale_t, scale_inv_t, stream);
 }
 
-int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
-                                       float* scale_inv_t, hpfp8_stream_t stream) {
-  return quantize_128x1_t_impl("quantize_128x1_t_kmajor", true, x, m, k, q_t, scale_t, scale_inv_t, stream);
+int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t,
+                                       float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
+  return quantize_128x1_t_impl("quantize_128x1_t_kmajor", true, x, m, k, q_t, ld_t, scale_t, scale_inv_t, stream);
 }
 
 int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,
@@ -512,14 +565,15 @@ int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t r
   HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "dequantize_1x128: negative shape");
   HPFP8_REQUIRE(cols % kBlock == 0, HPFP8_ERR_SHAPE, "dequantize_1x128: last dim %lld is not a multiple of 128",
                 (long long)cols);
-  const int64_t nvec = rows * cols / 16;
+  const int64_t nvec = rows * cols / 8;
   if (nvec == 0) return HPFP8_OK;
   HPFP8_REQUIRE(q && scale_inv && out, HPFP8_ERR_ARG, "dequantize_1x128: null buffer");
   HPFP8_REQUIRE(aligned16(q) && aligned16(out), HPFP8_ERR_ALIGN, "dequantize_1x128: buffers must be 16-byte aligned");
-  const int64_t blocks = (nvec + 255) / 256;
+  constexpr int UNROLL = 4;
+  const int64_t blocks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "dequantize_1x128: tensor too large");
-  dequant_1x128_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
-      (const uint4*)q, scale_inv, (uint4*)out, nvec, grad_scale, grad_scale != 1.0f ? 1 : 0);
+  dequant_1x128_kernel<UNROLL><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+      (const uint2*)q, scale_inv, (uint4*)out, nvec, grad_scale, grad_scale != 1.0f ? 1 : 0);
   return check_launch("dequantize_1x128");
 }
 

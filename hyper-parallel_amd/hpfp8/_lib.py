@@ -25,16 +25,16 @@ SIGNATURES = {
     "hpfp8_quantize_per_tensor_bf16": [_vp, _i64, _vp, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_1x128_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_1x128_kmajor_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
-    "hpfp8_quantize_128x1_t_kmajor_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
-    "hpfp8_quantize_128x128_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp],
-    "hpfp8_quantize_128x1_t_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
+    "hpfp8_quantize_128x1_t_kmajor_bf16": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp],
+    "hpfp8_quantize_128x128_bf16": [_vp, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
+    "hpfp8_quantize_128x1_t_bf16": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_dequantize_1x128_bf16": [_vp, _vp, _i64, _i64, _vp, _f32, _vp],
     "hpfp8_dequantize_128x128_bf16": [_vp, _vp, _i64, _i64, _vp, _vp],
-    "hpfp8_gemm_blockwise": [_vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp, _vp,
-                             _i64, _int, _int, _vp],
-    "hpfp8_gemm_per_tensor": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _int, _vp],
-    "hpfp8_gemm_grouped_blockwise": [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _i64, _int,
-                                     _vp],
+    "hpfp8_gemm_blockwise": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp,
+                             _vp, _i64, _int, _int, _vp],
+    "hpfp8_gemm_per_tensor": [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _int, _vp],
+    "hpfp8_gemm_grouped_blockwise": [_vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _i64,
+                                     _int, _vp],
 }
 
 OUT_BF16, OUT_F32 = 0, 1

@@ -46,6 +46,32 @@ def _check_fp8(x: torch.Tensor, name: str) -> torch.Tensor:
     return x
 
 
+def _check_codes_2d(x: torch.Tensor, name: str) -> torch.Tensor:
+    """A GEMM operand: 2-D codes with unit inner stride; the row stride may exceed the row length."""
+    if not x.is_cuda:
+        raise ValueError(f"{name} must live on the GPU")
+    if x.dtype not in (FP8, torch.uint8):
+        raise TypeError(f"{name} must be float8_e4m3fn (or uint8 codes), got {x.dtype}")
+    if x.dim() != 2 or (x.shape[1] > 1 and x.stride(1) != 1) or (x.shape[0] > 1 and x.stride(0) % 16):
+        raise ValueError(f"{name} must be 2-D with unit inner stride and a row stride that is a multiple of 16")
+    return x
+
+
+def _ld(x: torch.Tensor) -> int:
+    return x.stride(0) if x.shape[0] > 1 else max(x.shape[1], 16)
+
+
+def _padded_ld(n: int) -> int:
+    """Row stride for a transposed code tensor with n columns: an odd multiple of 128 bytes, so that
+    consecutive rows do not all fall on the same HBM channel (n itself is a multiple of 128)."""
+    return n if (n // BLOCK) % 2 == 1 else n + BLOCK
+
+
+def _empty_codes_t(rows: int, cols: int, device) -> torch.Tensor:
+    ld = _padded_ld(cols)
+    return torch.empty((rows, ld), dtype=FP8, device=device)[:, :cols]
+
+
 def _check_f32(x: torch.Tensor, name: str) -> torch.Tensor:
     if not x.is_cuda or x.dtype != torch.float32:
         raise TypeError(f"{name} must be a float32 GPU tensor")
@@ -128,11 +154,11 @@ def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: 
     if r % BLOCK or c % BLOCK:
         raise ValueError(f"shape {tuple(w.shape)} is not a multiple of {BLOCK} in both dims")
     q = torch.empty((r, c), dtype=FP8, device=w.device)
-    qt = torch.empty((c, r), dtype=FP8, device=w.device) if with_transpose else None
+    qt = _empty_codes_t(c, r, w.device) if with_transpose else None     # row stride padded, see _padded_ld
     scale_inv = torch.empty((r // BLOCK, c // BLOCK), dtype=torch.float32, device=w.device)
     scale = torch.empty_like(scale_inv) if want_scale else None
-    _lib.call("hpfp8_quantize_128x128_bf16", _ptr(w), r, c, _ptr(q), _ptr(qt), _ptr(scale), _ptr(scale_inv),
-              _stream())
+    _lib.call("hpfp8_quantize_128x128_bf16", _ptr(w), r, c, _ptr(q), _ptr(qt), _ld(qt) if with_transpose else 0,
+              _ptr(scale), _ptr(scale_inv), _stream())
     out = (q, scale_inv)
     if with_transpose:
         out += (qt,)
@@ -153,12 +179,12 @@ def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = F
     m, k = x.shape
     if m % BLOCK or k % BLOCK:
         raise ValueError(f"shape {tuple(x.shape)} is not a multiple of {BLOCK} in both dims")
-    qt = torch.empty((k, m), dtype=FP8, device=x.device)
+    qt = _empty_codes_t(k, m, x.device)                                  # row stride padded, see _padded_ld
     sshape = (m // BLOCK, k) if kmajor else (k, m // BLOCK)
     scale_inv = torch.empty(sshape, dtype=torch.float32, device=x.device)
     scale = torch.empty_like(scale_inv) if want_scale else None
     name = "hpfp8_quantize_128x1_t_kmajor_bf16" if kmajor else "hpfp8_quantize_128x1_t_bf16"
-    _lib.call(name, _ptr(x), m, k, _ptr(qt), _ptr(scale), _ptr(scale_inv), _stream())
+    _lib.call(name, _ptr(x), m, k, _ptr(qt), _ld(qt), _ptr(scale), _ptr(scale_inv), _stream())
     if kmajor:
         scale_inv = scale_inv.t()
         scale = scale.t() if want_scale else None
@@ -211,10 +237,11 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
                    ) -> torch.Tensor:
     """c[M,N] = sum_kb sa[m,kb] * sb[n//sb_gran, kb] * (a[m, kb] . b[n, kb]) (+ bias).
 
-    a[M,K], b[N,K] codes; sa, sb 2-D fp32 views (any strides) of scale_inv values.
+    a[M,K], b[N,K] codes (unit inner stride, any 16-byte-multiple row stride); sa, sb 2-D fp32 views
+    (any strides) of scale_inv values.
     """
-    a = _check_fp8(a, "a")
-    b = _check_fp8(b, "b")
+    a = _check_codes_2d(a, "a")
+    b = _check_codes_2d(b, "b")
     sa = _check_f32(sa, "sa")
     sb = _check_f32(sb, "sb")
     if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
@@ -229,6 +256,8 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
     want_sb = (n // BLOCK, kb) if sb_gran == 128 else (n, kb)
     if sb_gran not in (1, 128) or tuple(sb.shape) != want_sb:
         raise ValueError(f"sb must be {list(want_sb)} for sb_gran={sb_gran}, got {tuple(sb.shape)}")
+    if sb_gran == 1 and (sb.stride(0) != 1 or sb.stride(1) < n or sb.stride(1) % 4 or sb.data_ptr() % 16):
+        sb = sb.t().contiguous().t()        # the kernel wants per-row b scales k-block-major
     if bias is not None:
         bias = _check_bf16(bias, "bias")
         if tuple(bias.shape) != (n,):
@@ -243,8 +272,8 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
         out_dtype = out.dtype
     if accumulate and out_dtype != torch.float32:
         raise ValueError("accumulate needs a float32 output")
-    _lib.call("hpfp8_gemm_blockwise", _ptr(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
-              sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
+    _lib.call("hpfp8_gemm_blockwise", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ld(b),
+              _ptr(sb), sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
               out.stride(0) if m > 1 else n, _out_code(out_dtype), int(accumulate), _stream())
     return out
 
@@ -252,8 +281,8 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
 def gemm_per_tensor(a: torch.Tensor, sa_inv: torch.Tensor, b: torch.Tensor, sb_inv: torch.Tensor,
                     bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """c = (a . b^T) * (sa_inv * sb_inv) (+ bias); sa_inv / sb_inv are 0-dim (or 1-element) fp32."""
-    a = _check_fp8(a, "a")
-    b = _check_fp8(b, "b")
+    a = _check_codes_2d(a, "a")
+    b = _check_codes_2d(b, "b")
     sa_inv = _check_f32(sa_inv, "sa_inv")
     sb_inv = _check_f32(sb_inv, "sb_inv")
     if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
@@ -269,8 +298,8 @@ def gemm_per_tensor(a: torch.Tensor, sa_inv: torch.Tensor, b: torch.Tensor, sb_i
         if tuple(bias.shape) != (n,):
             raise ValueError(f"bias must be [{n}]")
     out = torch.empty((m, n), dtype=out_dtype, device=a.device)
-    _lib.call("hpfp8_gemm_per_tensor", _ptr(a), _ptr(sa_inv), _ptr(b), _ptr(sb_inv), m, n, k, _ptr(bias),
-              _ptr(out), n, _out_code(out_dtype), _stream())
+    _lib.call("hpfp8_gemm_per_tensor", _ptr(a), _ld(a), _ptr(sa_inv), _ptr(b), _ld(b), _ptr(sb_inv), m, n, k,
+              _ptr(bias), _ptr(out), n, _out_code(out_dtype), _stream())
     return out
 
 
@@ -279,7 +308,7 @@ def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, s
     """MoE grouped GEMM: rows of a[total_m, K] sorted by expert, offs[E] int32 inclusive prefix sums,
     b[E, N, K], sb[E, N/128, K/128], sa[total_m, K/128] -> c[total_m, N].  Rows past offs[-1] are left
     uninitialised (as torch's grouped matmul leaves them)."""
-    a = _check_fp8(a, "a")
+    a = _check_codes_2d(a, "a")
     b = _check_fp8(b, "b")
     sa = _check_f32(sa, "sa")
     sb = _check_f32(sb, "sb")
@@ -299,6 +328,6 @@ def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, s
     if tuple(sb.shape) != (e, n // BLOCK, kb) or not sb.is_contiguous():
         raise ValueError(f"sb must be contiguous [{e}, {n // BLOCK}, {kb}]")
     out = torch.empty((total_m, n), dtype=out_dtype, device=a.device)
-    _lib.call("hpfp8_gemm_grouped_blockwise", _ptr(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
+    _lib.call("hpfp8_gemm_grouped_blockwise", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
               _ptr(offs), e, total_m, n, k, _ptr(out), n, _out_code(out_dtype), _stream())
     return out

@@ -82,20 +82,22 @@ int hpfp8_quantize_1x128_kmajor_bf16(const void* x, int64_t rows, int64_t cols, 
                                      float* scale_inv, hpfp8_stream_t stream);
 
 /* Weights: w[rows, cols] bf16, one scale per 128x128 block.  q[rows, cols]; q_t (may be NULL)
- * receives the transposed codes [cols, rows] that dgrad consumes; scale (may be NULL) and
- * scale_inv are [rows/128, cols/128]. */
-int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t,
+ * receives the transposed codes [cols, rows] that dgrad consumes, with row stride ld_t bytes
+ * (>= rows, multiple of 16; a stride that is an odd multiple of 128 avoids HBM channel camping);
+ * scale (may be NULL) and scale_inv are [rows/128, cols/128]. */
+int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
                                 float* scale, float* scale_inv, hpfp8_stream_t stream);
 
 /* wgrad operands: x[m, k] bf16, one scale per 128 consecutive ROWS of a column, written
- * transposed: q_t[k, m]; scale_t (may be NULL) and scale_inv_t are [k, m/128]. */
-int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
+ * transposed: q_t[k, m] with row stride ld_t bytes (>= m, multiple of 16); scale_t (may be NULL)
+ * and scale_inv_t are [k, m/128]. */
+int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t, float* scale_t,
                                 float* scale_inv_t, hpfp8_stream_t stream);
 
 /* Same codes; scale_t / scale_inv_t written block-major, [m/128, k]: element (col, b) at
  * [b * k + col]. */
-int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, float* scale_t,
-                                       float* scale_inv_t, hpfp8_stream_t stream);
+int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t,
+                                       float* scale_t, float* scale_inv_t, hpfp8_stream_t stream);
 
 /* ---- dequantizers ----------------------------------------------------------------------------
  * The cast-back site hyper_parallel/core/hsdp/hsdp_grad_buffer.py:116-125: out = bf16(decode(q)
@@ -111,33 +113,35 @@ int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t
  *
  *   c[m, n] = sum_kb  sa(m, kb) * sb(n, kb) * ( sum_{k in block kb} a[m, k] * b[n, k] )  (+ bias[n])
  *
- * a[M, K] and b[N, K] are E4M3 codes with K contiguous (K, N multiples of 128); fp32
- * accumulation, k-blocks ascending; one rounding to bf16 at the end (or fp32 output).
+ * a[M, K] and b[N, K] are E4M3 codes with K contiguous and row strides lda / ldb bytes (>= K,
+ * multiples of 16); K, N multiples of 128; fp32 accumulation, k-blocks ascending; one rounding to
+ * bf16 at the end (or fp32 output).
  *   sa(m, kb) = sa[m * sa_stride_m + kb * sa_stride_k]
  *   sb(n, kb) = sb[(n / sb_gran) * sb_stride_n + kb * sb_stride_k],  sb_gran = 128 or 1
  * Uses:  forward  a = x codes (1x128),  b = W codes (128x128),            sb_gran = 128
  *        dgrad    a = grad_out codes,   b = W^T codes, W's scales with swapped strides
- *        wgrad    a = grad_out^T codes (128x1 requant), b = x^T codes,    sb_gran = 1
+ *        wgrad    a = grad_out^T codes (128x1 requant), b = x^T codes,    sb_gran = 1; the b scales must
+ *                 then be k-block-major: sb_stride_n = 1, sb_stride_k >= N (what the *_kmajor quantizers write)
  * bias: bf16[N] or NULL.  out_type HPFP8_OUT_BF16 / HPFP8_OUT_F32; ldc = row stride of c in
  * elements.  accumulate != 0 (fp32 output only) adds into c instead of overwriting it, the fp32
  * main-grad bookkeeping of hyper_parallel/platform/torch/fully_shard/param.py:134-167. */
-int hpfp8_gemm_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
-                         const void* b, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                         const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
                          int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
                          int64_t ldc, int out_type, int accumulate, hpfp8_stream_t stream);
 
 /* Per-tensor scales: c = (a . b^T) * (sa_inv[0] * sb_inv[0]) (+ bias), accumulation over the whole
  * K inside the matrix cores.  K a multiple of 128, N a multiple of 128. */
-int hpfp8_gemm_per_tensor(const void* a, const float* sa_inv, const void* b, const float* sb_inv,
-                          int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
-                          int out_type, hpfp8_stream_t stream);
+int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,
+                          const float* sb_inv, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
+                          int64_t ldc, int out_type, hpfp8_stream_t stream);
 
 /* MoE grouped form (one rank's local experts; no counterpart in the reference, whose expert
- * parallelism is unimplemented): rows of a[total_m, K] are sorted by expert; offs[e] (int32,
+ * parallelism is unimplemented): rows of a[total_m, K] (row stride lda) are sorted by expert; offs[e] (int32,
  * device) is the inclusive prefix sum of per-expert row counts, a count may be 0, rows past
  * offs[experts-1] are left untouched; b[experts, N, K]; sb[experts, N/128, K/128];
  * sa(m, kb) = sa[m * sa_stride_m + kb * sa_stride_k]; c[total_m, N] bf16 or fp32. */
-int hpfp8_gemm_grouped_blockwise(const void* a, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                                  const void* b, const float* sb, const int32_t* offs, int experts,
                                  int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
                                  hpfp8_stream_t stream);

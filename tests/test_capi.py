@@ -47,19 +47,19 @@ def test_argument_errors_are_reported_without_launching():
     rc = lib.hpfp8_quantize_1x128_bf16(p + 2, 1, 128, p, None, p, None)
     assert rc == -3
     # null buffer
-    rc = lib.hpfp8_quantize_128x128_bf16(None, 128, 128, p, None, None, p, None)
+    rc = lib.hpfp8_quantize_128x128_bf16(None, 128, 128, p, None, 0, None, p, None)
     assert rc == -1
     # bad scale granularity, bad K
-    rc = lib.hpfp8_gemm_blockwise(p, p, 1, 1, p, p, 1, 1, 7, 128, 128, 128, None, p, 128, 0, 0, None)
+    rc = lib.hpfp8_gemm_blockwise(p, 128, p, 1, 1, p, 128, p, 1, 1, 7, 128, 128, 128, None, p, 128, 0, 0, None)
     assert rc == -1
-    rc = lib.hpfp8_gemm_blockwise(p, p, 1, 1, p, p, 1, 1, 128, 128, 128, 100, None, p, 128, 0, 0, None)
+    rc = lib.hpfp8_gemm_blockwise(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 128, 128, 100, None, p, 128, 0, 0, None)
     assert rc == -2
     # accumulate needs fp32 output
-    rc = lib.hpfp8_gemm_blockwise(p, p, 1, 1, p, p, 1, 1, 128, 128, 128, 128, None, p, 128, 0, 1, None)
+    rc = lib.hpfp8_gemm_blockwise(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 128, 128, 128, None, p, 128, 0, 1, None)
     assert rc == -1
     # empty problems succeed without touching the device
     assert lib.hpfp8_quantize_1x128_bf16(None, 0, 128, None, None, None, None) == 0
-    assert lib.hpfp8_gemm_per_tensor(None, None, None, None, 0, 128, 128, None, None, 128, 0, None) == 0
+    assert lib.hpfp8_gemm_per_tensor(None, 128, None, None, 128, None, 0, 128, 128, None, None, 128, 0, None) == 0
 
 
 def test_python_wrappers_reject_cpu_tensors_and_bad_shapes():

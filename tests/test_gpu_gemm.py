@@ -248,7 +248,7 @@ def test_grouped_leaves_rows_past_the_last_offset_alone(gpu):
     offs = torch.tensor([100, 260], dtype=torch.int32, device=gpu)
     from hpfp8 import _lib, ops
     out = torch.full((300, N), 7.0, dtype=torch.float32, device=gpu)
-    _lib.call("hpfp8_gemm_grouped_blockwise", xq.data_ptr(), sxi.data_ptr(), sxi.stride(0), sxi.stride(1),
+    _lib.call("hpfp8_gemm_grouped_blockwise", xq.data_ptr(), K, sxi.data_ptr(), sxi.stride(0), sxi.stride(1),
               wq.data_ptr(), swi.data_ptr(), offs.data_ptr(), 2, 300, N, K, out.data_ptr(), N, _lib.OUT_F32,
               ops._stream())
     assert bool((out[260:] == 7.0).all()) and not bool((out[:260] == 7.0).any())
