@@ -21,8 +21,11 @@ namespace hpfp8 {
 
 constexpr int BM = 256, BN = 256, BK = 128;
 constexpr int kGemmThreads = 512;
-constexpr int kTileBytes = 256 * BK;          // one operand tile in LDS
-constexpr int kStageBytes = 2 * kTileBytes;   // a tile then b tile
+constexpr int kTileBytes = 256 * BK;          // one operand tile in LDS (32 KB)
+// LDS: two buffers for the a tile, then kBStages buffers for the b tile.  The b operand is the one
+// that streams from HBM (each weight panel is used by one XCD only), so where LDS allows it gets a
+// third buffer and its transfers run two k-blocks ahead; a's re-reads come from the Infinity Cache.
+__host__ __device__ constexpr int b_stages(int mode) { return mode == 2 /* kScaleRow: LDS also holds scales */ ? 2 : 3; }
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8, kGroupN = 4;   // tile rectangle one XCD works on at a time
 
@@ -77,7 +80,9 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 
 template <int MODE, bool GROUPED, bool OUT_F32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * kStageBytes];
+  constexpr int kBStages = b_stages(MODE);
+  constexpr int kBAhead = kBStages - 1;     // k-blocks between issuing a b transfer and using it
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[(2 + kBStages) * kTileBytes];
   // per-row scales of the b operand for one k-block (wgrad form), two stages of 256 floats
   __shared__ __attribute__((aligned(16))) float sb_lds[MODE == kScaleRow ? 2 * BN : 4];
 
@@ -166,18 +171,23 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sb, (lds_ptr_t)(sb_lds + stage * BN), 16,
                                                (uint32_t)(n0 + lane * 4) * 4u, (int)(kb * p.sb_sk * 4), 0, 0);
   };
-  // One of a wave's 8 transfers for k-block kb: even idx -> a tile, odd idx -> b tile.
-  auto issue_tile_load = [&](int kb, int stage, int idx) {
-    uint8_t* sbase = lds + stage * kStageBytes + wave * 4096 + (idx >> 1) * 1024;
-    if (idx & 1)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sbase + kTileBytes), 16, b_off[idx >> 1],
-                                               kb * BK, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)sbase, 16, a_off[idx >> 1], kb * BK, 0, 0);
-  };
-  auto issue_tile_loads = [&](int kb, int stage) {
-#pragma unroll
-    for (int idx = 0; idx < 8; ++idx) issue_tile_load(kb, stage, idx);
+  // idx 0..3 -> a tile of k-block kb_a into a buffer abuf; idx 4..7 -> b tile of k-block kb_b into b
+  // buffer bbuf.
+  auto issue_tile_load = [&](int kb_a, int abuf, int kb_b, int bbuf, int idx) {
+    // The four transfers of one operand share one LDS base (M0) and differ in the instruction's
+    // immediate offset, which the hardware adds to both the LDS and the memory address; the memory
+    // side is compensated in the lane offset.  This leaves two M0 updates per round instead of eight.
+    uint8_t* sbase = lds + wave * 4096 + ((idx & 4) ? (2 + bbuf) * kTileBytes : abuf * kTileBytes);
+    const __amdgpu_buffer_rsrc_t& rs = (idx & 4) ? rsrc_b : rsrc_a;
+    const int sub = idx & 3;
+    const int kb = (idx & 4) ? kb_b : kb_a;
+    const uint32_t voff = ((idx & 4) ? b_off[sub] : a_off[sub]) - sub * 1024;
+    switch (sub) {   // the immediate must be a literal; idx is a compile-time constant after unrolling
+      case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 0, 0); break;
+      case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 1024, 0); break;
+      case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 2048, 0); break;
+      default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 3072, 0); break;
+    }
   };
 
   // ---- fragment addressing
@@ -185,7 +195,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   const int l16 = lane & 15, g = lane >> 4;
   const int pc0 = (2 * g) ^ row_swizzle(l16);
   const int a_frag_off = (wm * 64 + l16) * BK;               // + j * 16 rows
-  const int b_frag_off = kTileBytes + (wn * 128 + l16) * BK;  // + i * 16 rows
+  const int b_frag_off = (wn * 128 + l16) * BK;               // + i * 16 rows, inside a b buffer
 
   // ---- scales
   int arow[4];
@@ -220,10 +230,16 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_raw[5] = {1.f, 1.f, 1.f, 1.f, 1.f};
   load_scales(0, s_raw);
   combine_scales(s_raw, s_cur);
-  issue_tile_loads(0, 0);
+#pragma unroll
+  for (int idx = 0; idx < 8; ++idx) issue_tile_load(0, 0, 0, 0, idx);
+  if (kBAhead == 2) {
+#pragma unroll
+    for (int idx = 4; idx < 8; ++idx) issue_tile_load(0, 0, 1, 1, idx);
+  }
   issue_sb_load(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
+  int bbuf = 0;                        // b buffer holding k-block kb
 
   for (int kb = 0; kb < kblocks; ++kb) {
     const int stage = kb & 1;
@@ -234,7 +250,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     // addresses past the tensor read as zero), which keeps the loop body free of branches.
     load_scales(kb + 1 < kblocks ? kb + 1 : kb, s_raw);
     __builtin_amdgcn_sched_barrier(0);
-    const uint8_t* sbase = lds + stage * kStageBytes;
+    const uint8_t* abase = lds + stage * kTileBytes;
+    const uint8_t* bbase_l = lds + (2 + bbuf) * kTileBytes;
+    int bbuf_issue = bbuf + kBAhead;   // b buffer the transfers of this round go to
+    if (bbuf_issue >= kBStages) bbuf_issue -= kBStages;
     v8i xf[4];
     if (MODE != kScaleTensor) {
       // Software pipeline over the 8 n-subtiles: the matrix instructions of subtile i are issued
@@ -245,10 +264,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       v4f part[2][4];
       // weight fragments are read two subtiles ahead of their use (three live at a time)
       v8i wf[3];
-      wf[0] = frag_read(sbase + b_frag_off, pc0);
+      wf[0] = frag_read(bbase_l + b_frag_off, pc0);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
-      wf[1] = frag_read(sbase + b_frag_off + 16 * BK, pc0);
+      for (int j = 0; j < 4; ++j) xf[j] = frag_read(abase + a_frag_off + j * 16 * BK, pc0);
+      wf[1] = frag_read(bbase_l + b_frag_off + 16 * BK, pc0);
       // wgrad form: the four per-row b scales of subtile i for this lane's four n
       const float* sb_row = sb_lds + stage * BN + wn * 128 + g * 4;
       v4f sbv[2];
@@ -257,9 +276,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        if (i + 2 < 8) wf[(i + 2) % 3] = frag_read(sbase + b_frag_off + (i + 2) * 16 * BK, pc0);
+        if (i + 2 < 8) wf[(i + 2) % 3] = frag_read(bbase_l + b_frag_off + (i + 2) * 16 * BK, pc0);
         if (MODE == kScaleRow && i > 0) sbv[i & 1] = *reinterpret_cast<const v4f*>(sb_row + i * 16);   // used by the FMAs of group i+1
-        issue_tile_load(kb + 1, stage ^ 1, i);
+        issue_tile_load(kb + 1, stage ^ 1, kb + kBAhead, bbuf_issue, i);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -285,11 +304,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
         }
     } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xf[j] = frag_read(sbase + a_frag_off + j * 16 * BK, pc0);
+      for (int j = 0; j < 4; ++j) xf[j] = frag_read(abase + a_frag_off + j * 16 * BK, pc0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const v8i wf = frag_read(sbase + b_frag_off + i * 16 * BK, pc0);
-        issue_tile_load(kb + 1, stage ^ 1, i);
+        const v8i wf = frag_read(bbase_l + b_frag_off + i * 16 * BK, pc0);
+        issue_tile_load(kb + 1, stage ^ 1, kb + kBAhead, bbuf_issue, i);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -298,10 +317,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     }
     __builtin_amdgcn_sched_barrier(0);
     combine_scales(s_raw, s_cur);
-    // own DMA for the next stage has landed and own LDS reads of this stage are done; then everyone's
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    // Own transfers needed by the next round have landed and own LDS reads of this round are done;
+    // then everyone's.  With three b buffers the four b transfers issued this round (the youngest
+    // vector-memory operations) are for the round after next and may still be in flight.
+    if (kBAhead == 2) __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0x0070);               // vmcnt(0) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
+    bbuf = bbuf + 1 == kBStages ? 0 : bbuf + 1;
   }
+
+  // Transfers issued for rounds past the end still target this workgroup's LDS: drain them before
+  // the LDS can be handed to another workgroup.
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
 
   // ---- epilogue
   float tensor_scale = 1.f;
