@@ -78,6 +78,19 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return (uint32_t)__builtin_bit_cast(uint16_t, x) | ((uint32_t)__builtin_bit_cast(uint16_t, y) << 16);
 }
 
+// Tile number -> (m tile, n tile).  Consecutive numbers (one XCD's CUs at any moment) cover
+// kGroupM x kGroupN rectangles of tiles, n fastest inside a rectangle, so the L2 of that XCD serves
+// each activation / weight panel to several CUs.  Rectangles at the right and bottom edges shrink.
+__device__ __forceinline__ void rect_map(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int per_ngroup = kGroupN * tiles_m;
+  const int ng = t / per_ngroup, rest = t % per_ngroup;
+  const int gn = (tiles_n - ng * kGroupN) < kGroupN ? (tiles_n - ng * kGroupN) : kGroupN;
+  const int mg = rest / (kGroupM * gn);
+  const int r3 = rest - mg * kGroupM * gn;
+  tm = mg * kGroupM + r3 / gn;
+  tn = ng * kGroupN + r3 % gn;
+}
+
 template <int MODE, bool GROUPED, bool OUT_F32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
   constexpr int kBStages = b_stages(MODE);
@@ -102,46 +115,30 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   }
   int row0, row_end, tn, expert = 0;
   if (GROUPED) {
-    int total_mt = 0;
-    for (int e = 0, prev = 0; e < p.experts; ++e) {
-      int end = p.offs[e];
-      total_mt += (end - prev + BM - 1) / BM;
-      prev = end;
-    }
-    if (total_mt == 0 || t >= total_mt * tiles_n) return;
-    tn = t / total_mt;
-    int mt = t % total_mt;
-    int prev = 0;
-    row0 = 0;
-    row_end = 0;
+    // Tiles are numbered expert by expert (an expert with no rows has none); inside an expert they
+    // form the same rectangles as in the dense case, so its weight panels are shared through L2.
+    int prev = 0, first = 0, tm = 0;
+    bool found = false;
     for (int e = 0; e < p.experts; ++e) {
-      int end = p.offs[e];
-      int cnt = (end - prev + BM - 1) / BM;
-      if (mt < cnt) {
+      const int end = p.offs[e];
+      const int cnt = (end - prev + BM - 1) / BM;
+      if (!found && t < first + cnt * tiles_n) {
+        rect_map(t - first, cnt, tiles_n, tm, tn);
         expert = e;
-        row0 = prev + mt * BM;
+        row0 = prev + tm * BM;
         row_end = end < p.M ? end : p.M;
-        break;
+        found = true;
       }
-      mt -= cnt;
+      first += cnt * tiles_n;
       prev = end;
     }
+    if (!found) return;
   } else {
     const int tiles_m = (p.M + BM - 1) / BM;
     if (t >= tiles_m * tiles_n) return;
-    // Consecutive tile ids (one XCD's CUs at any moment) cover kGroupM x kGroupN rectangles of
-    // tiles, so the L2 of that XCD serves each activation / weight panel to several CUs.
-    const int per_ngroup = kGroupN * tiles_m;
-    const int ng = t / per_ngroup, rest = t % per_ngroup;
-    const int gn = (tiles_n - ng * kGroupN) < kGroupN ? (tiles_n - ng * kGroupN) : kGroupN;   // last group may be narrow
-    const int mg = rest / (kGroupM * gn), rest2 = rest % (kGroupM * gn);
-    const int gm = (tiles_m - mg * kGroupM) < kGroupM ? (tiles_m - mg * kGroupM) : kGroupM;
-    // inside a rectangle: n fastest
-    int tm_local, tn_local;
-    if (gm == kGroupM) { tm_local = rest2 / gn; tn_local = rest2 % gn; }
-    else { const int r3 = rest - mg * kGroupM * gn; tm_local = r3 / gn; tn_local = r3 % gn; }
-    tn = ng * kGroupN + tn_local;
-    row0 = (mg * kGroupM + tm_local) * BM;
+    int tm;
+    rect_map(t, tiles_m, tiles_n, tm, tn);
+    row0 = tm * BM;
     row_end = p.M;
   }
   const int n0 = tn * BN;
