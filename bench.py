@@ -84,12 +84,109 @@ def cpu_baseline(x_bits, w_bits, target_seconds=15.0):
     }
 
 
+def _time(fn, iters=10, warm=2):
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s0.record()
+    for _ in range(iters):
+        fn()
+    s1.record()
+    torch.cuda.synchronize()
+    return s0.elapsed_time(s1) / iters
+
+
+def other_configs(dev):
+    """Kernel times of configurations 1, 3, 4 and 5 (HIP events, back-to-back launches)."""
+    import torch
+    import hpfp8
+    res = {}
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def tf(flops, ms):
+        return {"ms": ms, "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_FP8_TFLOPS}
+
+    def gb(nbytes, ms):
+        return {"ms": ms, "GB/s": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+
+    # cfg 1: per-tensor linear 2048x1024x1024
+    x = torch.randn((2048, 1024), generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn((1024, 1024), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    xq, _, sx = hpfp8.quantize_per_tensor(x)
+    wq, _, sw = hpfp8.quantize_per_tensor(w)
+    res["cfg1_per_tensor"] = {
+        "quantize_x": gb(x.numel() * 5, _time(lambda: hpfp8.quantize_per_tensor(x))),
+        "gemm": tf(2.0 * 2048 * 1024 * 1024, _time(lambda: hpfp8.gemm_per_tensor(xq, sx, wq, sw))),
+    }
+    # cfg 3: o_proj backward
+    m, n, k = 4096, 7168, 16384
+    x = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
+    u = torch.rand((m, n), generator=g, device=dev) - 0.5
+    go = (-(2 ** -0.5) * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999)) * 1e-3).to(torch.bfloat16)
+    w = (torch.randn((n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16)
+    wq, sw, wqt = hpfp8.quantize_128x128(w, with_transpose=True)
+    goq, sgo = hpfp8.quantize_1x128(go, kmajor=True)
+    got, sgot = hpfp8.quantize_128x1_t(go, kmajor=True)
+    xt, sxt = hpfp8.quantize_128x1_t(x, kmajor=True)
+    fl = 2.0 * m * n * k
+    res["cfg3_backward"] = {
+        "quantize_w_with_transpose": gb(n * k * 4 + (n // 128) * (k // 128) * 4,
+                                        _time(lambda: hpfp8.quantize_128x128(w, with_transpose=True))),
+        "requant_t_x": gb(m * k * 3 + k * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(x, kmajor=True))),
+        "requant_t_grad_out": gb(m * n * 3 + n * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(go, kmajor=True))),
+        "quantize_grad_out": gb(m * n * 3 + m * (n // 128) * 4, _time(lambda: hpfp8.quantize_1x128(go, kmajor=True))),
+        "dgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq, sgo, wqt, sw.t()))),
+        "wgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1))),
+    }
+    del x, go, w, wq, wqt, goq, got, xt
+    torch.cuda.empty_cache()
+    # cfg 4: MoE grouped, 32 experts, 131072 routed rows, Zipf(1.1) counts, two empty experts
+    e, n, k, total = 32, 4096, 7168, 131072
+    gc = torch.Generator(device="cpu").manual_seed(0)
+    perm = torch.randperm(e, generator=gc)
+    pz = (torch.arange(1, e + 1, dtype=torch.float64) ** -1.1)[perm]
+    pz = pz / pz.sum()
+    counts = torch.multinomial(pz, total, replacement=True, generator=gc).bincount(minlength=e)
+    order = torch.argsort(pz)
+    for z in order[:2]:
+        counts[order[-1]] += counts[z]
+        counts[z] = 0
+    offs = counts.cumsum(0).to(torch.int32).to(dev)
+    x = torch.randn((total, k), generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn((e * n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16)
+    xq, sx = hpfp8.quantize_1x128(x, kmajor=True)
+    wq, sw = hpfp8.quantize_128x128(w)
+    del x, w
+    ms = _time(lambda: hpfp8.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // 128, k // 128), offs), iters=5)
+    res["cfg4_moe_grouped"] = dict(tf(2.0 * total * n * k, ms), rows=total, experts=e,
+                                   min_rows=int(counts.min()), max_rows=int(counts.max()))
+    del xq, sx, wq, sw
+    torch.cuda.empty_cache()
+    # cfg 5: gradient bucket, 2^29 elements
+    nel = 1 << 29
+    flat = torch.randn(nel, generator=g, device=dev) * 1e-4
+    idx = torch.randint(0, nel, (nel // 10000,), generator=g, device=dev)
+    flat[idx] *= 1e3
+    flat = flat.to(torch.bfloat16)
+    nbytes = nel * 3 + (nel // 128) * 4
+    codes, si = hpfp8.quantize_bucket(flat)
+    res["cfg5_bucket"] = {
+        "quantize": gb(nbytes, _time(lambda: hpfp8.quantize_bucket(flat))),
+        "dequantize": gb(nbytes, _time(lambda: hpfp8.dequantize_bucket(codes, si))),
+    }
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--all", action="store_true",
+                    help="also time the kernels of the other benchmark configurations (adds an 'other_configs' key)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU's share of the path; this build has no multi-GPU leg "
@@ -219,6 +316,10 @@ def main():
         },
         "check": {"gemm_rel_frobenius_vs_f64_dequant_matmul": err},
     }
+    if args.all:
+        del x, w, xq, wq, y
+        torch.cuda.empty_cache()
+        out["other_configs"] = other_configs(dev)
     if not args.no_cpu_baseline:
         import numpy as np
         xb = x[:2048].cpu().view(torch.int16).numpy().view(np.uint16)
