@@ -84,7 +84,7 @@ def cpu_baseline(x_bits, w_bits, target_seconds=15.0):
     }
 
 
-def _time(fn, iters=10, warm=2):
+def _time(fn, iters=20, warm=20):
     import torch
     for _ in range(warm):
         fn()
@@ -182,8 +182,8 @@ def other_configs(dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=50)   # the clock needs ~25 ms of load to leave its idle state
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--all", action="store_true",
                     help="also time the kernels of the other benchmark configurations (adds an 'other_configs' key)")
@@ -316,15 +316,17 @@ def main():
         },
         "check": {"gemm_rel_frobenius_vs_f64_dequant_matmul": err},
     }
+    host_copies = None
+    if not args.no_cpu_baseline:
+        import numpy as np
+        host_copies = (x[:2048].cpu().view(torch.int16).numpy().view(np.uint16),
+                       w.cpu().view(torch.int16).numpy().view(np.uint16))
     if args.all:
         del x, w, xq, wq, y
         torch.cuda.empty_cache()
         out["other_configs"] = other_configs(dev)
-    if not args.no_cpu_baseline:
-        import numpy as np
-        xb = x[:2048].cpu().view(torch.int16).numpy().view(np.uint16)
-        wb = w.cpu().view(torch.int16).numpy().view(np.uint16)
-        out["cpu_baseline"] = cpu_baseline(xb, wb)
+    if host_copies is not None:
+        out["cpu_baseline"] = cpu_baseline(*host_copies)
     print(json.dumps(out))
 
 
