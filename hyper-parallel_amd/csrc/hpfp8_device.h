@@ -82,18 +82,27 @@ __device__ __forceinline__ float clamp448(float y) {
 }
 
 // Two bf16 in one word -> two E4M3 codes in the chosen half of `old`.
-template <bool HI>
+// CLAMP = false is for kernels whose scale was derived from the amax of the very values being
+// cast: then |x * scale| <= 448 * (1 + 2^-23), which rounds to 448 like the clamped value does, so
+// the explicit clamp to +-448 cannot change a code for finite inputs and is left out.  With a scale
+// that comes from elsewhere (a caller-supplied amax) the clamp is required.
+template <bool HI, bool CLAMP>
 __device__ __forceinline__ uint32_t cvt2(uint32_t old, uint32_t w, float scale) {
-  float a = clamp448(bf16lo(w) * scale);
-  float b = clamp448(bf16hi(w) * scale);
+  float a = bf16lo(w) * scale;
+  float b = bf16hi(w) * scale;
+  if (CLAMP) {
+    a = clamp448(a);
+    b = clamp448(b);
+  }
   return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, HI);
 }
 
 // 8 bf16 (uint4) -> 8 E4M3 codes (uint2), element order kept.
+template <bool CLAMP>
 __device__ __forceinline__ uint2 cvt8(const uint4& v, float scale) {
   uint2 r;
-  r.x = cvt2<true>(cvt2<false>(0u, v.x, scale), v.y, scale);
-  r.y = cvt2<true>(cvt2<false>(0u, v.z, scale), v.w, scale);
+  r.x = cvt2<true, CLAMP>(cvt2<false, CLAMP>(0u, v.x, scale), v.y, scale);
+  r.y = cvt2<true, CLAMP>(cvt2<false, CLAMP>(0u, v.z, scale), v.w, scale);
   return r;
 }
 
