@@ -96,8 +96,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   constexpr int kBStages = b_stages(MODE);
   constexpr int kBAhead = kBStages - 1;     // k-blocks between issuing a b transfer and using it
   __shared__ __attribute__((aligned(1024))) uint8_t lds[(2 + kBStages) * kTileBytes];
-  // per-row scales of the b operand for one k-block (wgrad form), two stages of 256 floats
-  __shared__ __attribute__((aligned(16))) float sb_lds[MODE == kScaleRow ? 2 * BN : 4];
+  // per-row scales of the b operand for one k-block (wgrad form), three stages of 256 floats: the
+  // stage of k-block kb+1 is filled while slower waves may still read that of kb-1
+  __shared__ __attribute__((aligned(16))) float sb_lds[MODE == kScaleRow ? 3 * BN : 4];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -168,24 +169,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sb, (lds_ptr_t)(sb_lds + stage * BN), 16,
                                                (uint32_t)(n0 + lane * 4) * 4u, (int)(kb * p.sb_sk * 4), 0, 0);
   };
-  // idx 0..3 -> a tile of k-block kb_a into a buffer abuf; idx 4..7 -> b tile of k-block kb_b into b
-  // buffer bbuf.
-  auto issue_tile_load = [&](int kb_a, int abuf, int kb_b, int bbuf, int idx) {
-    // The four transfers of one operand share one LDS base (M0) and differ in the instruction's
-    // immediate offset, which the hardware adds to both the LDS and the memory address; the memory
-    // side is compensated in the lane offset.  This leaves two M0 updates per round instead of eight.
-    uint8_t* sbase = lds + wave * 4096 + ((idx & 4) ? (2 + bbuf) * kTileBytes : abuf * kTileBytes);
-    const __amdgpu_buffer_rsrc_t& rs = (idx & 4) ? rsrc_b : rsrc_a;
-    const int sub = idx & 3;
-    const int kb = (idx & 4) ? kb_b : kb_a;
-    const uint32_t voff = ((idx & 4) ? b_off[sub] : a_off[sub]) - sub * 1024;
-    switch (sub) {   // the immediate must be a literal; idx is a compile-time constant after unrolling
+  // One transfer = 8 rows x 128 B per wave; `sub` (0..3) selects which of the wave's four 8-row groups
+  // of the 256-row tile.  The four transfers of one operand tile share one LDS base (M0) and differ
+  // in the instruction's immediate offset, which the hardware adds to both the LDS and the memory
+  // address; the memory side is compensated in the lane offset.
+  auto issue_tile = [&](const __amdgpu_buffer_rsrc_t& rs, const uint32_t (&off)[4], int buf, int kb, int sub) {
+    uint8_t* sbase = lds + wave * 4096 + buf * kTileBytes;
+    const uint32_t voff = off[sub] - sub * 1024;
+    switch (sub) {   // the immediate must be a literal; sub is a compile-time constant after unrolling
       case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 0, 0); break;
       case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 1024, 0); break;
       case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 2048, 0); break;
       default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 3072, 0); break;
     }
   };
+  auto issue_a = [&](int kb, int abuf, int sub) { issue_tile(rsrc_a, a_off, abuf, kb, sub); };
+  auto issue_b = [&](int kb, int bbuf, int sub) { issue_tile(rsrc_b, b_off, 2 + bbuf, kb, sub); };
 
   // ---- fragment addressing
   const int wn = wave & 1, wm = wave >> 1;
@@ -224,103 +223,162 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
+  // ---- prologue: k-block 0 of both operands (and k-block 1 of b where it has three buffers)
   float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_raw[5] = {1.f, 1.f, 1.f, 1.f, 1.f};
   load_scales(0, s_raw);
   combine_scales(s_raw, s_cur);
 #pragma unroll
-  for (int idx = 0; idx < 8; ++idx) issue_tile_load(0, 0, 0, 0, idx);
+  for (int sub = 0; sub < 4; ++sub) issue_a(0, 0, sub);
+#pragma unroll
+  for (int sub = 0; sub < 4; ++sub) issue_b(0, 0, sub);
   if (kBAhead == 2) {
 #pragma unroll
-    for (int idx = 4; idx < 8; ++idx) issue_tile_load(0, 0, 1, 1, idx);
+    for (int sub = 0; sub < 4; ++sub) issue_b(1, 1, sub);
   }
   issue_sb_load(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
+
+  // The synchronisation point of a round sits before its last two n-subtiles, not at its end: what
+  // follows the barrier (the weight fragments of the next round's first two subtiles, and the
+  // activation fragments re-read one by one as the last subtile releases their registers) is then
+  // covered by the matrix instructions still to be issued, and no round starts with every wave
+  // waiting on LDS at once.  Fragments that cross the round boundary are carried in registers.
+  v8i xf[4], wf_n0, wf_n1;
+  wf_n0 = frag_read(lds + 2 * kTileBytes + b_frag_off, pc0);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) xf[j] = frag_read(lds + a_frag_off + j * 16 * BK, pc0);
+  wf_n1 = frag_read(lds + 2 * kTileBytes + b_frag_off + 16 * BK, pc0);
+  // first two transfers of the next activation tile (normally issued after the previous barrier)
+  issue_a(1, 1, 0);
+  issue_a(1, 1, 1);
+
+  constexpr bool kCarry = MODE == kScaleBlock;   // promote subtile 7 inside the next round's first group
+  const v4f zero = {0.f, 0.f, 0.f, 0.f};
+  v4f part_c[4] = {zero, zero, zero, zero};
+  float s_old[4] = {0.f, 0.f, 0.f, 0.f};
   int bbuf = 0;                        // b buffer holding k-block kb
+  int sbuf = 0;                        // scale stage (wgrad form) holding k-block kb
 
   for (int kb = 0; kb < kblocks; ++kb) {
     const int stage = kb & 1;
-    // The 8 tile transfers for the next k-block are issued one per n-subtile inside the compute
-    // loop instead of as a burst here: a burst of 64 transfers per CU queues up in the texture
-    // path and holds every wave back before its first LDS read.
-    // They are issued for the round after the last one too (into the stage nobody reads again;
-    // addresses past the tensor read as zero), which keeps the loop body free of branches.
+    // Transfers run past the last k-block too (into buffers nobody reads again; addresses past the
+    // tensor read as zero), which keeps the loop body free of branches.
     load_scales(kb + 1 < kblocks ? kb + 1 : kb, s_raw);
-    __builtin_amdgcn_sched_barrier(0);
-    const uint8_t* abase = lds + stage * kTileBytes;
-    const uint8_t* bbase_l = lds + (2 + bbuf) * kTileBytes;
-    int bbuf_issue = bbuf + kBAhead;   // b buffer the transfers of this round go to
+    const uint8_t* bcur = lds + (2 + bbuf) * kTileBytes;
+    int bnext = bbuf + 1 == kBStages ? 0 : bbuf + 1;           // holds k-block kb + 1
+    int bbuf_issue = bbuf + kBAhead;                           // receives k-block kb + kBAhead
     if (bbuf_issue >= kBStages) bbuf_issue -= kBStages;
-    v8i xf[4];
+    const uint8_t* bnxt = lds + (2 + bnext) * kTileBytes;
+    const uint8_t* anxt = lds + (stage ^ 1) * kTileBytes;
+    int snext = sbuf + 1 == 3 ? 0 : sbuf + 1;
+    // Per round: the rest of a(kb+1) at subtiles 0,1; b(kb+kBAhead) at 2..5; after the barrier the
+    // first half of a(kb+2), into the buffer whose fragments every wave has just left behind.
+    // One transfer per subtile: a burst would queue up in the texture path ahead of the LDS reads.
+    auto issue_slot = [&](int i) {
+      if (i < 2) issue_a(kb + 1, stage ^ 1, i + 2);
+      else if (i < 6) issue_b(kb + kBAhead, bbuf_issue, i - 2);
+      else issue_a(kb + 2, stage, i - 6);
+    };
+    auto round_sync = [&]() {
+      // Own transfers for the next round have landed and own LDS reads of this round's buffers are
+      // done; then everyone's.  With three b buffers the four b transfers of this round (the
+      // youngest vector-memory operations) are for the round after next and may stay in flight.
+      if (kBAhead == 2) __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+      else __builtin_amdgcn_s_waitcnt(0x0070);               // vmcnt(0) lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+    };
+    // weight fragment of subtile i + 2 (the first two of the next round once past the barrier)
+    auto read_ahead = [&](int i) {
+      return i + 2 < 8 ? frag_read(bcur + b_frag_off + (i + 2) * 16 * BK, pc0)
+                       : frag_read(bnxt + b_frag_off + (i + 2 - 8) * 16 * BK, pc0);
+    };
     if (MODE != kScaleTensor) {
       // Software pipeline over the 8 n-subtiles: the matrix instructions of subtile i are issued
       // interleaved with the promotion FMAs of subtile i-1, whose partial sums left the matrix
-      // pipe four instructions earlier, so neither pipe waits for the other.  The LDS reads of
-      // subtile i+1 are issued before the MFMAs of subtile i (a full subtile of latency cover).
-      const v4f zero = {0.f, 0.f, 0.f, 0.f};
+      // pipe four instructions earlier, so neither pipe waits for the other.
       v4f part[2][4];
-      // weight fragments are read two subtiles ahead of their use (three live at a time)
       v8i wf[3];
-      wf[0] = frag_read(bbase_l + b_frag_off, pc0);
+      wf[0] = wf_n0;
+      wf[1] = wf_n1;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xf[j] = frag_read(abase + a_frag_off + j * 16 * BK, pc0);
-      wf[1] = frag_read(bbase_l + b_frag_off + 16 * BK, pc0);
+      for (int j = 0; j < 4; ++j) part[1][j] = part_c[j];
       // wgrad form: the four per-row b scales of subtile i for this lane's four n
-      const float* sb_row = sb_lds + stage * BN + wn * 128 + g * 4;
+      const float* sb_row = sb_lds + sbuf * BN + wn * 128 + g * 4;
       v4f sbv[2];
       if (MODE == kScaleRow) sbv[0] = *reinterpret_cast<const v4f*>(sb_row);
-      if (MODE == kScaleRow && wave == 0) issue_sb_load(kb + 1 < kblocks ? kb + 1 : kb, stage ^ 1);
+      if (MODE == kScaleRow) issue_sb_load(kb + 1 < kblocks ? kb + 1 : kb, snext);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        if (i + 2 < 8) wf[(i + 2) % 3] = frag_read(bbase_l + b_frag_off + (i + 2) * 16 * BK, pc0);
+        if (i == 6) round_sync();
+        wf[(i + 2) % 3] = read_ahead(i);
         if (MODE == kScaleRow && i > 0) sbv[i & 1] = *reinterpret_cast<const v4f*>(sb_row + i * 16);   // used by the FMAs of group i+1
-        issue_tile_load(kb + 1, stage ^ 1, kb + kBAhead, bbuf_issue, i);
+        issue_slot(i);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i % 3], xf[j], zero, 0, 0, 0, 0, 0, 0);
-          if (i > 0) {
+          if (i > 0 || kCarry) {
+            const int ip = (i + 7) & 7;     // subtile being promoted; for i = 0 the last one of the previous round
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               float pv = part[(i - 1) & 1][j][r];
               if (MODE == kScaleRow) pv *= sbv[(i - 1) & 1][r];
-              acc[i - 1][j][r] = __builtin_fmaf(pv, s_cur[j], acc[i - 1][j][r]);
+              acc[ip][j][r] = __builtin_fmaf(pv, i == 0 ? s_old[j] : s_cur[j], acc[ip][j][r]);
             }
           }
+          if (i == 7) xf[j] = frag_read(anxt + a_frag_off + j * 16 * BK, pc0);
           __builtin_amdgcn_sched_barrier(0);   // keep this (MFMA, FMAs) group together, in this order
         }
       }
+      if (kCarry) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float pv = part[1][j][r];
-          if (MODE == kScaleRow) pv *= sbv[1][r];
-          acc[7][j][r] = __builtin_fmaf(pv, s_cur[j], acc[7][j][r]);
-        }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xf[j] = frag_read(abase + a_frag_off + j * 16 * BK, pc0);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const v8i wf = frag_read(bbase_l + b_frag_off + i * 16 * BK, pc0);
-        issue_tile_load(kb + 1, stage ^ 1, kb + kBAhead, bbuf_issue, i);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < 4; ++j) part_c[j] = part[1][j];
+      } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float pv = part[1][j][r];
+            if (MODE == kScaleRow) pv *= sbv[1][r];
+            acc[7][j][r] = __builtin_fmaf(pv, s_cur[j], acc[7][j][r]);
+          }
       }
+      wf_n0 = wf[8 % 3];
+      wf_n1 = wf[9 % 3];
+    } else {
+      v8i wf[3];
+      wf[0] = wf_n0;
+      wf[1] = wf_n1;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (i == 6) round_sync();
+        wf[(i + 2) % 3] = read_ahead(i);
+        issue_slot(i);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i % 3], xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+          if (i == 7) xf[j] = frag_read(anxt + a_frag_off + j * 16 * BK, pc0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      wf_n0 = wf[8 % 3];
+      wf_n1 = wf[9 % 3];
     }
     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s_old[j] = s_cur[j];
     combine_scales(s_raw, s_cur);
-    // Own transfers needed by the next round have landed and own LDS reads of this round are done;
-    // then everyone's.  With three b buffers the four b transfers issued this round (the youngest
-    // vector-memory operations) are for the round after next and may still be in flight.
-    if (kBAhead == 2) __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
-    else __builtin_amdgcn_s_waitcnt(0x0070);               // vmcnt(0) lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    bbuf = bbuf + 1 == kBStages ? 0 : bbuf + 1;
+    bbuf = bnext;
+    sbuf = snext;
+  }
+  if (kCarry) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[7][j][r] = __builtin_fmaf(part_c[j][r], s_old[j], acc[7][j][r]);
   }
 
   // Transfers issued for rounds past the end still target this workgroup's LDS: drain them before
