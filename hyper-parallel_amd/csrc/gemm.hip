@@ -14,6 +14,8 @@
 //     (out-of-range rows read as zero), 16-byte chunks XOR-swizzled by row so that both the DMA
 //     writes and the ds_read_b128 fragment reads are bank-conflict free.
 //   * Workgroup ids are remapped so that each XCD (own L2) works on a contiguous run of tiles.
+#include <type_traits>
+
 #include "hpfp8_device.h"
 #include "hpfp8_host.h"
 
@@ -39,6 +41,7 @@ struct GemmParams {
   int64_t sa_sm, sa_sk;   // element strides of sa over (row, k-block)
   int64_t sb_sn, sb_sk;   // element strides of sb over (row or 128-row block, k-block)
   int64_t sb_se;          // grouped: stride of sb between experts
+  int sb_bytes;           // size of the sb array in bytes (block form)
   void* c;
   int64_t ldc;
   const uint16_t* bias;
@@ -46,6 +49,7 @@ struct GemmParams {
   int experts;
   int64_t lda, ldb;       // row strides of a and b in bytes (>= K)
   int M, N, K;            // M = total rows of a
+  int tiles;              // dense: number of output tiles
   int accumulate;
 };
 
@@ -91,6 +95,33 @@ __device__ __forceinline__ void rect_map(int t, int tiles_m, int tiles_n, int& t
   tn = ng * kGroupN + r3 % gn;
 }
 
+// One output tile of a workgroup's list.  A tile with no rows (row0 == row_end, n0 >= N) stands for
+// "past the end of the list": transfers addressed to it fetch nothing.
+struct TileInfo {
+  int row0, row_end;   // rows [row0, row_end) of a and c that exist (row_end - row0 may be < BM)
+  int n0;              // first row of b / column of c
+  int expert;
+};
+
+// Position `d` k-blocks after k-block kb of the current tile: how many tiles further (0..2, d <= 2)
+// and which k-block there.
+__device__ __forceinline__ int tiles_ahead(int kb, int d, int kblocks, int& kb_out) {
+  int pos = kb + d, q = 0;
+  if (pos >= kblocks) { pos -= kblocks; q = 1; }
+  if (pos >= kblocks) { pos -= kblocks; q = 2; }
+  kb_out = pos;
+  return q;
+}
+
+__device__ __forceinline__ TileInfo pick_tile(int q, TileInfo t0, TileInfo t1, TileInfo t2) {
+  TileInfo r;
+  r.row0 = q == 2 ? t2.row0 : (q == 1 ? t1.row0 : t0.row0);
+  r.row_end = q == 2 ? t2.row_end : (q == 1 ? t1.row_end : t0.row_end);
+  r.n0 = q == 2 ? t2.n0 : (q == 1 ? t1.n0 : t0.n0);
+  r.expert = q == 2 ? t2.expert : (q == 1 ? t1.expert : t0.expert);
+  return r;
+}
+
 template <int MODE, bool GROUPED, bool OUT_F32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
   constexpr int kBStages = b_stages(MODE);
@@ -106,68 +137,109 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   const int kblocks = K / BK;
   const int tiles_n = (N + BN - 1) / BN;
 
-  // ---- workgroup -> tile, XCD aware: ids congruent mod 8 share an XCD and get a contiguous run
-  int t;
-  {
-    const int nblk = gridDim.x, pid = blockIdx.x;
-    const int xcd = pid % kXcds, local = pid / kXcds;
-    const int base = nblk / kXcds, big = nblk % kXcds;
-    t = xcd * base + (xcd < big ? xcd : big) + local;
-  }
-  int row0, row_end, tn, expert = 0;
+  // ---- the tile list of this workgroup.  The grid is persistent (one workgroup per CU); tiles are
+  // numbered so that consecutive numbers cover kGroupM x kGroupN rectangles, each XCD (workgroup ids
+  // congruent mod 8, own L2) owns a contiguous run of numbers, and the workgroups of an XCD walk
+  // through that run side by side, so at any moment they work on one rectangle.
+  int total_tiles = p.tiles;
   if (GROUPED) {
-    // Tiles are numbered expert by expert (an expert with no rows has none); inside an expert they
-    // form the same rectangles as in the dense case, so its weight panels are shared through L2.
-    int prev = 0, first = 0, tm = 0;
-    bool found = false;
+    // tiles are numbered expert by expert; an expert with no rows has none
+    int prev = 0, mt = 0;
     for (int e = 0; e < p.experts; ++e) {
       const int end = p.offs[e];
-      const int cnt = (end - prev + BM - 1) / BM;
-      if (!found && t < first + cnt * tiles_n) {
-        rect_map(t - first, cnt, tiles_n, tm, tn);
-        expert = e;
-        row0 = prev + tm * BM;
-        row_end = end < p.M ? end : p.M;
-        found = true;
-      }
-      first += cnt * tiles_n;
+      mt += (end - prev + BM - 1) / BM;
       prev = end;
     }
-    if (!found) return;
-  } else {
-    const int tiles_m = (p.M + BM - 1) / BM;
-    if (t >= tiles_m * tiles_n) return;
-    int tm;
-    rect_map(t, tiles_m, tiles_n, tm, tn);
-    row0 = tm * BM;
-    row_end = p.M;
+    total_tiles = mt * tiles_n;
   }
-  const int n0 = tn * BN;
-
+  int my_tiles, t_first, t_step;
+  {
+    const int nwg = gridDim.x, pid = blockIdx.x;
+    const int xu = nwg < kXcds ? nwg : kXcds;        // the host launches a multiple of 8 workgroups, or fewer than 8
+    const int xcd = pid % xu, slot = pid / xu;
+    t_step = nwg / xu;
+    const int base = total_tiles / xu, big = total_tiles % xu;
+    const int cnt = base + (xcd < big ? 1 : 0);
+    t_first = xcd * base + (xcd < big ? xcd : big) + slot;
+    my_tiles = slot < cnt ? (cnt - slot + t_step - 1) / t_step : 0;
+  }
+  if (my_tiles == 0) return;
+  const int n_pad = tiles_n * BN;
+  // grouped: forward-only search state (tile numbers are asked for in increasing order)
+  int g_e = 0, g_prev = 0, g_first = 0;
+  auto lookup = [&](int k, TileInfo& ti) {
+    int row0 = p.M, row_end = p.M, n0 = n_pad, expert = 0;
+    if (k < my_tiles) {
+      const int t = t_first + k * t_step;
+      int tm, tn;
+      if (GROUPED) {
+        int end = 0, cnt = 0;
+        while (g_e < p.experts) {
+          end = p.offs[g_e];
+          cnt = (end - g_prev + BM - 1) / BM;
+          if (t < g_first + cnt * tiles_n) break;
+          g_first += cnt * tiles_n;
+          g_prev = end;
+          ++g_e;
+        }
+        if (g_e < p.experts) {
+          rect_map(t - g_first, cnt, tiles_n, tm, tn);
+          expert = g_e;
+          row0 = g_prev + tm * BM;
+          row_end = end < p.M ? end : p.M;
+          if (row0 + BM < row_end) row_end = row0 + BM;
+          n0 = tn * BN;
+        }
+      } else {
+        rect_map(t, (p.M + BM - 1) / BM, tiles_n, tm, tn);
+        row0 = tm * BM;
+        row_end = row0 + BM < p.M ? row0 + BM : p.M;
+        n0 = tn * BN;
+      }
+    }
+    // (values found through the expert search sit in vector registers; as scalars they keep the
+    // buffer resources built from them scalar too)
+    ti.row0 = __builtin_amdgcn_readfirstlane(row0);
+    ti.row_end = __builtin_amdgcn_readfirstlane(row_end);
+    ti.n0 = __builtin_amdgcn_readfirstlane(n0);
+    ti.expert = __builtin_amdgcn_readfirstlane(expert);
+  };
+  // T0 is the tile being accumulated; transfers and scale loads run up to two k-blocks ahead and
+  // so reach into T1 (and into T2 when K is a single k-block).
+  TileInfo T0, T1, T2;
+  lookup(0, T0);
+  lookup(1, T1);
+  lookup(2, T2);
   // ---- global -> LDS tile DMA.  One wave instruction moves 8 rows x 128 B (lane i -> LDS slot
-  // i); the lane picks the 16-byte global chunk whose swizzled home is its slot.
-  const uint8_t* bbase = p.b + (GROUPED ? (int64_t)expert * N * p.ldb : 0);
-  const __amdgpu_buffer_rsrc_t rsrc_a =
-      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)((int64_t)p.M * p.lda), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b =
-      __builtin_amdgcn_make_buffer_rsrc((void*)bbase, 0, (int)((int64_t)N * p.ldb), 0x00020000);
+  // i); the lane picks the 16-byte global chunk whose swizzled home is its slot.  The buffer
+  // resource of a transfer starts at the tile's first row and ends with the tensor (or the expert),
+  // so lane offsets do not depend on the tile and rows past the end read as zero.
+  auto rsrc_a_of = [&](const TileInfo& ti) {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(p.a + (int64_t)ti.row0 * p.lda), 0,
+                                             (int)((int64_t)(ti.row_end - ti.row0) * p.lda), 0x00020000);
+  };
+  auto rsrc_b_of = [&](const TileInfo& ti) {
+    const int rows = N - ti.n0 > 0 ? N - ti.n0 : 0;
+    const uint8_t* base = p.b + (GROUPED ? (int64_t)ti.expert * N * p.ldb : 0) + (int64_t)(rows ? ti.n0 : 0) * p.ldb;
+    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)((int64_t)rows * p.ldb), 0x00020000);
+  };
   uint32_t a_off[4], b_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int q = wave * 4 + i;                       // 8-row group inside the tile
     const int r = q * 8 + (lane >> 3);                // row inside the tile
     const int chunk = (lane & 7) ^ row_swizzle(r);    // logical 16-byte chunk of that row
-    a_off[i] = (uint32_t)(row0 + r) * (uint32_t)p.lda + chunk * 16;
-    b_off[i] = (uint32_t)(n0 + r) * (uint32_t)p.ldb + chunk * 16;
+    a_off[i] = (uint32_t)r * (uint32_t)p.lda + chunk * 16;
+    b_off[i] = (uint32_t)r * (uint32_t)p.ldb + chunk * 16;
   }
   // wgrad form: the 256 per-row scales of the b tile for one k-block are one more 1 KB transfer
   // (wave 0), possible because that scale array is k-block-major (unit stride over rows).
   const __amdgpu_buffer_rsrc_t rsrc_sb = __builtin_amdgcn_make_buffer_rsrc(
       (void*)p.sb, 0, MODE == kScaleRow ? (int)((((int64_t)kblocks - 1) * p.sb_sk + N) * 4) : 0, 0x00020000);
-  auto issue_sb_load = [&](int kb, int stage) {
+  auto issue_sb_load = [&](const TileInfo& ti, int kb, int stage) {
     if (MODE == kScaleRow && wave == 0)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sb, (lds_ptr_t)(sb_lds + stage * BN), 16,
-                                               (uint32_t)(n0 + lane * 4) * 4u, (int)(kb * p.sb_sk * 4), 0, 0);
+                                               (uint32_t)(ti.n0 + lane * 4) * 4u, (int)(kb * p.sb_sk * 4), 0, 0);
   };
   // One transfer = 8 rows x 128 B per wave; `sub` (0..3) selects which of the wave's four 8-row groups
   // of the 256-row tile.  The four transfers of one operand tile share one LDS base (M0) and differ
@@ -183,8 +255,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)sbase, 16, voff, kb * BK, 3072, 0); break;
     }
   };
-  auto issue_a = [&](int kb, int abuf, int sub) { issue_tile(rsrc_a, a_off, abuf, kb, sub); };
-  auto issue_b = [&](int kb, int bbuf, int sub) { issue_tile(rsrc_b, b_off, 2 + bbuf, kb, sub); };
 
   // ---- fragment addressing
   const int wn = wave & 1, wm = wave >> 1;
@@ -193,23 +263,35 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   const int a_frag_off = (wm * 64 + l16) * BK;               // + j * 16 rows
   const int b_frag_off = (wn * 128 + l16) * BK;               // + i * 16 rows, inside a b buffer
 
-  // ---- scales
-  int arow[4];
+  // ---- scales.  Raw values for one k-block are loaded at the top of the round before it and only
+  // combined (sa * sb) at its end, so nothing waits on global memory in between.
+  // Both scale arrays are read through buffer resources with 32-bit byte offsets (the host checks
+  // that they span less than 2 GiB): the row part of an offset is per tile, the k-block part a
+  // scalar, so a round spends no vector arithmetic on addresses.
+  const __amdgpu_buffer_rsrc_t rsrc_sa = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)p.sa, 0, MODE == kScaleTensor ? 4 : (int)((((int64_t)p.M - 1) * p.sa_sm + ((int64_t)kblocks - 1) * p.sa_sk + 1) * 4),
+      0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_sbb = __builtin_amdgcn_make_buffer_rsrc((void*)p.sb, 0, p.sb_bytes, 0x00020000);
+  uint32_t sa_voff[4];         // byte offset of this lane's four rows in sa
+  int sb_soff = 0;             // block form: byte offset of the b tile's scale row
+  const int sa_kstep = (int)p.sa_sk * 4, sb_kstep = (int)p.sb_sk * 4;
+  auto scale_target = [&](const TileInfo& ti) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    int r = row0 + wm * 64 + j * 16 + l16;
-    arow[j] = r < p.M ? r : p.M - 1;
-  }
-  const float* sbp = p.sb + (GROUPED ? (int64_t)expert * p.sb_se : 0);
-  int nblk_idx = (n0 + wn * 128) >> 7;
-  if (nblk_idx > (N >> 7) - 1) nblk_idx = (N >> 7) - 1;
-  // Raw scale values for one k-block: the loads are issued at the top of the round before it and
-  // only combined (sa * sb) at its end, so nothing waits on global memory in between.
+    for (int j = 0; j < 4; ++j) {
+      const int r = ti.row0 + wm * 64 + j * 16 + l16;
+      sa_voff[j] = (uint32_t)(r < p.M ? r : p.M - 1) * (uint32_t)((int)p.sa_sm * 4);
+    }
+    int nblk_idx = (ti.n0 + wn * 128) >> 7;
+    if (nblk_idx > (N >> 7) - 1) nblk_idx = (N >> 7) - 1;
+    sb_soff = ((GROUPED ? ti.expert * (int)p.sb_se : 0) + nblk_idx * (int)p.sb_sn) * 4;
+  };
   auto load_scales = [&](int kb, float raw[5]) {
-    if (MODE == kScaleBlock) raw[4] = sbp[(int64_t)nblk_idx * p.sb_sn + (int64_t)kb * p.sb_sk];
+    if (MODE == kScaleBlock)
+      raw[4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sbb, 0, sb_soff + kb * sb_kstep, 0));
     if (MODE != kScaleTensor) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) raw[j] = p.sa[(int64_t)arow[j] * p.sa_sm + (int64_t)kb * p.sa_sk];
+      for (int j = 0; j < 4; ++j)
+        raw[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, sa_voff[j], kb * sa_kstep, 0));
     }
   };
   auto combine_scales = [&](const float raw[5], float s[4]) {
@@ -217,68 +299,106 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     for (int j = 0; j < 4; ++j) s[j] = MODE == kScaleBlock ? raw[j] * raw[4] : raw[j];
   };
 
+  const v4f zero = {0.f, 0.f, 0.f, 0.f};
   v4f acc[8][4];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 4; ++j) acc[i][j] = zero;
 
-  // ---- prologue: k-block 0 of both operands (and k-block 1 of b where it has three buffers)
+  // ---- prologue: k-block 0 of both operands, k-block 1 of b where it has three buffers, and the
+  // first half of a's k-block 1
   float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_raw[5] = {1.f, 1.f, 1.f, 1.f, 1.f};
+  scale_target(T0);
   load_scales(0, s_raw);
   combine_scales(s_raw, s_cur);
+  {
+    const __amdgpu_buffer_rsrc_t ra = rsrc_a_of(T0), rb = rsrc_b_of(T0);
 #pragma unroll
-  for (int sub = 0; sub < 4; ++sub) issue_a(0, 0, sub);
+    for (int sub = 0; sub < 4; ++sub) issue_tile(ra, a_off, 0, 0, sub);
 #pragma unroll
-  for (int sub = 0; sub < 4; ++sub) issue_b(0, 0, sub);
-  if (kBAhead == 2) {
+    for (int sub = 0; sub < 4; ++sub) issue_tile(rb, b_off, 2, 0, sub);
+    int kb1;
+    const TileInfo t1 = pick_tile(tiles_ahead(0, 1, kblocks, kb1), T0, T1, T2);
+    if (kBAhead == 2) {
+      const __amdgpu_buffer_rsrc_t rb1 = rsrc_b_of(t1);
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) issue_b(1, 1, sub);
+      for (int sub = 0; sub < 4; ++sub) issue_tile(rb1, b_off, 3, kb1, sub);
+    }
+    issue_sb_load(T0, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    const __amdgpu_buffer_rsrc_t ra1 = rsrc_a_of(t1);
+    issue_tile(ra1, a_off, 1, kb1, 0);
+    issue_tile(ra1, a_off, 1, kb1, 1);
   }
-  issue_sb_load(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  __syncthreads();
 
   // The synchronisation point of a round sits before its last two n-subtiles, not at its end: what
   // follows the barrier (the weight fragments of the next round's first two subtiles, and the
   // activation fragments re-read one by one as the last subtile releases their registers) is then
   // covered by the matrix instructions still to be issued, and no round starts with every wave
   // waiting on LDS at once.  Fragments that cross the round boundary are carried in registers.
+  // Rounds follow each other without a gap across tiles: the last rounds of a tile already fetch
+  // the first k-blocks of the next one, and its stores drain while the next tile computes.
   v8i xf[4], wf_n0, wf_n1;
   wf_n0 = frag_read(lds + 2 * kTileBytes + b_frag_off, pc0);
 #pragma unroll
   for (int j = 0; j < 4; ++j) xf[j] = frag_read(lds + a_frag_off + j * 16 * BK, pc0);
   wf_n1 = frag_read(lds + 2 * kTileBytes + b_frag_off + 16 * BK, pc0);
-  // first two transfers of the next activation tile (normally issued after the previous barrier)
-  issue_a(1, 1, 0);
-  issue_a(1, 1, 1);
 
   constexpr bool kCarry = MODE == kScaleBlock;   // promote subtile 7 inside the next round's first group
-  const v4f zero = {0.f, 0.f, 0.f, 0.f};
   v4f part_c[4] = {zero, zero, zero, zero};
   float s_old[4] = {0.f, 0.f, 0.f, 0.f};
-  int bbuf = 0;                        // b buffer holding k-block kb
-  int sbuf = 0;                        // scale stage (wgrad form) holding k-block kb
+  int stage = 0;                       // a buffer holding the current k-block
+  int bbuf = 0;                        // b buffer holding the current k-block
+  int sbuf = 0;                        // scale stage (wgrad form) holding the current k-block
+  // transfer targets (ordinal in the tile list) and their buffer resources
+  int ord_1 = 0, ord_2 = 0, ord_b = 0;
+  TileInfo tile_1 = T0;
+  __amdgpu_buffer_rsrc_t rs_a1 = rsrc_a_of(T0), rs_a2 = rs_a1, rs_b = rsrc_b_of(T0);
 
+  for (int tile = 0; tile < my_tiles; ++tile) {
   for (int kb = 0; kb < kblocks; ++kb) {
-    const int stage = kb & 1;
-    // Transfers run past the last k-block too (into buffers nobody reads again; addresses past the
-    // tensor read as zero), which keeps the loop body free of branches.
-    load_scales(kb + 1 < kblocks ? kb + 1 : kb, s_raw);
+    // Where this round's transfers and scale loads go: one k-block ahead (scales, second half of
+    // that a tile), two ahead (first half of that a tile), kBAhead ahead (b tile).  Only in the last
+    // two rounds of a tile does a target move on to the next tile of the list; its resource is
+    // rebuilt then and stays valid when that tile becomes the current one.
+    int kb1 = kb + 1, kb2 = kb + 2, kbb = kb + kBAhead;
+    if (kb2 >= kblocks) {
+      const int o1 = tile + tiles_ahead(kb, 1, kblocks, kb1);
+      const int o2 = tile + tiles_ahead(kb, 2, kblocks, kb2);
+      const int ob = tile + tiles_ahead(kb, kBAhead, kblocks, kbb);
+      if (o1 != ord_1) {
+        ord_1 = o1;
+        tile_1 = pick_tile(o1 - tile, T0, T1, T2);
+        rs_a1 = rsrc_a_of(tile_1);
+        scale_target(tile_1);
+      }
+      if (o2 != ord_2) {
+        ord_2 = o2;
+        rs_a2 = rsrc_a_of(pick_tile(o2 - tile, T0, T1, T2));
+      }
+      if (ob != ord_b) {
+        ord_b = ob;
+        rs_b = rsrc_b_of(pick_tile(ob - tile, T0, T1, T2));
+      }
+    }
+    load_scales(kb1, s_raw);
     const uint8_t* bcur = lds + (2 + bbuf) * kTileBytes;
-    int bnext = bbuf + 1 == kBStages ? 0 : bbuf + 1;           // holds k-block kb + 1
-    int bbuf_issue = bbuf + kBAhead;                           // receives k-block kb + kBAhead
+    int bnext = bbuf + 1 == kBStages ? 0 : bbuf + 1;           // holds the next k-block
+    int bbuf_issue = bbuf + kBAhead;                           // receives the k-block kBAhead ahead
     if (bbuf_issue >= kBStages) bbuf_issue -= kBStages;
     const uint8_t* bnxt = lds + (2 + bnext) * kTileBytes;
     const uint8_t* anxt = lds + (stage ^ 1) * kTileBytes;
     int snext = sbuf + 1 == 3 ? 0 : sbuf + 1;
-    // Per round: the rest of a(kb+1) at subtiles 0,1; b(kb+kBAhead) at 2..5; after the barrier the
-    // first half of a(kb+2), into the buffer whose fragments every wave has just left behind.
-    // One transfer per subtile: a burst would queue up in the texture path ahead of the LDS reads.
+    // Per round: the rest of the next a tile at subtiles 0,1; the b tile at 2..5; after the barrier
+    // the first half of the a tile after next, into the buffer whose fragments every wave has just
+    // left behind.  One transfer per subtile: a burst would queue up in the texture path ahead of
+    // the LDS reads.
     auto issue_slot = [&](int i) {
-      if (i < 2) issue_a(kb + 1, stage ^ 1, i + 2);
-      else if (i < 6) issue_b(kb + kBAhead, bbuf_issue, i - 2);
-      else issue_a(kb + 2, stage, i - 6);
+      if (i < 2) issue_tile(rs_a1, a_off, stage ^ 1, kb1, i + 2);
+      else if (i < 6) issue_tile(rs_b, b_off, 2 + bbuf_issue, kbb, i - 2);
+      else issue_tile(rs_a2, a_off, stage, kb2, i - 6);
     };
     auto round_sync = [&]() {
       // Own transfers for the next round have landed and own LDS reads of this round's buffers are
@@ -307,7 +427,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       const float* sb_row = sb_lds + sbuf * BN + wn * 128 + g * 4;
       v4f sbv[2];
       if (MODE == kScaleRow) sbv[0] = *reinterpret_cast<const v4f*>(sb_row);
-      if (MODE == kScaleRow) issue_sb_load(kb + 1 < kblocks ? kb + 1 : kb, snext);
+      if (MODE == kScaleRow) issue_sb_load(tile_1, kb1, snext);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -371,64 +491,140 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
     for (int j = 0; j < 4; ++j) s_old[j] = s_cur[j];
     combine_scales(s_raw, s_cur);
+    stage ^= 1;
     bbuf = bnext;
     sbuf = snext;
   }
+  // ---- the tile is complete: last promotion, then its stores
   if (kCarry) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[7][j][r] = __builtin_fmaf(part_c[j][r], s_old[j], acc[7][j][r]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) part_c[j] = zero;
   }
-
-  // Transfers issued for rounds past the end still target this workgroup's LDS: drain them before
-  // the LDS can be handed to another workgroup.
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-
-  // ---- epilogue
+  // The wave's 64 x 128 results go out 16 rows at a time through its own 4 KB slice of the b buffer
+  // whose k-block was consumed last (nothing is in flight to that buffer, and this wave alone
+  // transfers into this slice later), so that a store instruction writes whole rows of 256 bytes
+  // instead of 16 pieces of 8 bytes.  The slice holds 16 rows x 256 B, 16-byte chunks XOR-ed with
+  // the row so that both the fragment-order writes and the row-order reads spread over all banks.
   float tensor_scale = 1.f;
   if (MODE == kScaleTensor) tensor_scale = p.sa[0] * p.sb[0];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int n = n0 + wn * 128 + i * 16 + g * 4;
-    if (n >= N) continue;
-    float bv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (p.bias) {
-      const uint2 braw = *reinterpret_cast<const uint2*>(p.bias + n);
-      bv[0] = bf16lo(braw.x); bv[1] = bf16hi(braw.x); bv[2] = bf16lo(braw.y); bv[3] = bf16hi(braw.y);
-    }
+  const int row0 = T0.row0, row_end = T0.row_end, n0 = T0.n0;
+  // Lane coordinates re-derived behind an opaque copy: store addresses built from them would
+  // otherwise be hoisted out of the tile loop and held in registers through the main loop.
+  int lane_e = lane;
+  asm volatile("" : "+v"(lane_e));
+  const int l16e = lane_e & 15, ge = lane_e >> 4;
+  uint8_t* stg = lds + (2 + (bbuf == 0 ? kBStages - 1 : bbuf - 1)) * kTileBytes + wave * 4096;
+  const int ncol = n0 + wn * 128;                 // first column of the wave tile
+  const bool cols_ok = ncol < N;
+  constexpr int kHalves = OUT_F32 ? 2 : 1;       // fp32 rows of 128 columns take two slices
+  constexpr int kPerHalf = 8 / kHalves;           // n-subtiles per slice
+  const uint32_t stg_w = (uint32_t)(uintptr_t)(lds_ptr_t)stg + l16e * 256;   // LDS byte address of this lane's row
+  auto store_tile = [&](auto with_bias, auto full_rows) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int m = row0 + wm * 64 + j * 16 + l16;
-      if (m >= row_end) continue;
-      float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        v[r] = acc[i][j][r];
-        if (MODE == kScaleTensor) v[r] *= tensor_scale;
-        v[r] += bv[r];
-      }
-      if (OUT_F32) {
-        float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.c) + (int64_t)m * p.ldc + n);
-        float4 o = make_float4(v[0], v[1], v[2], v[3]);
-        if (p.accumulate) {
-          float4 old = *dst;
-          o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
+      for (int h = 0; h < kHalves; ++h) {
+#pragma unroll
+        for (int ii = 0; ii < kPerHalf; ++ii) {
+          const int i = h * kPerHalf + ii;
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            v[r] = acc[i][j][r];
+            if (MODE == kScaleTensor) v[r] *= tensor_scale;
+          }
+          if (decltype(with_bias)::value) {
+            const uint2 braw = *reinterpret_cast<const uint2*>(p.bias + ncol + i * 16 + ge * 4);
+            v[0] += bf16lo(braw.x); v[1] += bf16hi(braw.x); v[2] += bf16lo(braw.y); v[3] += bf16hi(braw.y);
+          }
+          // The staging writes are issued as bare instructions: the compiler would otherwise make
+          // every LDS store wait for the tile transfers in flight (to other buffers) to land.
+          if (OUT_F32) {
+            const v4f o = {v[0], v[1], v[2], v[3]};
+            asm volatile("ds_write_b128 %0, %1" ::"v"(stg_w + (((ii * 4 + ge) ^ l16e) * 16)), "v"(o) : "memory");
+          } else {
+            u32x2 o;
+            o[0] = pack_bf16x2(v[0], v[1]);
+            o[1] = pack_bf16x2(v[2], v[3]);
+            asm volatile("ds_write_b64 %0, %1" ::"v"(stg_w + (((ii * 2 + (ge >> 1)) ^ l16e) * 16) + (ge & 1) * 8), "v"(o)
+                         : "memory");
+          }
+          acc[i][j] = zero;
         }
-        *dst = o;
-      } else {
-        uint2 o;
-        o.x = pack_bf16x2(v[0], v[1]);
-        o.y = pack_bf16x2(v[2], v[3]);
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + n) = o;
+#pragma unroll
+        for (int k2 = 0; k2 < 4; k2 += 2) {      // two rows per lane at a time (registers are scarce here)
+          v4i val[2];
+#pragma unroll
+          for (int k = 0; k < 2; ++k) {
+            const int row = 4 * (k2 + k) + ge;
+            val[k] = *reinterpret_cast<const v4i*>(stg + row * 256 + ((l16e ^ row) * 16));
+          }
+#pragma unroll
+          for (int k = 0; k < 2; ++k) {
+            const int m = row0 + wm * 64 + j * 16 + 4 * (k2 + k) + ge;
+            if (decltype(full_rows)::value || m < row_end) {
+              if (OUT_F32) {
+                float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.c) + (int64_t)m * p.ldc + ncol + h * 64 + l16e * 4);
+                const v4f fv = __builtin_bit_cast(v4f, val[k]);   // (a cast of the whole vector, not of its elements)
+                float4 o = make_float4(fv[0], fv[1], fv[2], fv[3]);
+                if (p.accumulate) {
+                  const float4 old = *dst;
+                  o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
+                }
+                *dst = o;
+              } else {
+                *reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + ncol + l16e * 8) = val[k];
+              }
+            }
+          }
+        }
       }
     }
+  };
+  if (cols_ok) {
+    // common case first: no bias, all 256 rows of the tile exist (no per-row predicate)
+    if (!p.bias && row0 + BM <= row_end) store_tile(std::false_type{}, std::true_type{});
+    else if (!p.bias) store_tile(std::false_type{}, std::false_type{});
+    else store_tile(std::true_type{}, std::false_type{});
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = zero;
   }
+  T0 = T1;
+  T1 = T2;
+  lookup(tile + 3, T2);
+  }
+
+  // Transfers issued past the end of the list (they fetch nothing) still target this workgroup's
+  // LDS: drain them before the LDS can be handed to another workgroup.
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+}
+
+// Workgroups to launch for `tiles` tiles: one per CU, a multiple of 8 (one share per XCD) unless
+// there are fewer than 8 tiles.
+static int persistent_grid(int64_t tiles) {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  int64_t g = tiles < cus ? tiles : cus;
+  if (g >= kXcds) g -= g % kXcds;
+  return (int)g;
 }
 
 template <int MODE, bool GROUPED>
 static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
-  dim3 grid((unsigned)tiles), block(kGemmThreads);
+  dim3 grid((unsigned)persistent_grid(tiles)), block(kGemmThreads);
   if (out_type == HPFP8_OUT_F32)
     gemm_kernel<MODE, GROUPED, true><<<grid, block, 0, stream>>>(p);
   else
@@ -449,7 +645,9 @@ static int check_common(const char* what, const void* a, int64_t lda, const void
                 "%s: lda=%lld and ldb=%lld must be multiples of 16 and at least K=%lld", what, (long long)lda,
                 (long long)ldb, (long long)K);
   HPFP8_REQUIRE(ldc >= N, HPFP8_ERR_SHAPE, "%s: ldc=%lld smaller than N=%lld", what, (long long)ldc, (long long)N);
-  HPFP8_REQUIRE(ldc % 4 == 0, HPFP8_ERR_ALIGN, "%s: ldc must be a multiple of 4", what);
+  // rows of c are written in 16-byte pieces
+  HPFP8_REQUIRE(ldc % (out_type == HPFP8_OUT_F32 ? 4 : 8) == 0, HPFP8_ERR_ALIGN,
+                "%s: ldc must be a multiple of %d", what, out_type == HPFP8_OUT_F32 ? 4 : 8);
   if (M == 0 || N == 0) return HPFP8_OK;
   HPFP8_REQUIRE(a && b && sa && sb && c, HPFP8_ERR_ARG, "%s: null buffer", what);
   HPFP8_REQUIRE(aligned16(a) && aligned16(b) && aligned16(c) && (!bias || aligned16(bias)), HPFP8_ERR_ALIGN,
@@ -457,6 +655,16 @@ static int check_common(const char* what, const void* a, int64_t lda, const void
   // 32-bit byte offsets inside the tile loader, including rows read past the end of a tile
   HPFP8_REQUIRE((M + BM) * lda < (int64_t)0x7FFFFFFF && (N + BN) * ldb < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
                 "%s: an operand exceeds 2 GiB", what);
+  return 1;
+}
+
+// Scale arrays are addressed with 32-bit byte offsets inside the kernels.
+static int check_scale_span(const char* what, int64_t rows, int64_t kblocks, int64_t stride_r, int64_t stride_k,
+                            const char* name) {
+  HPFP8_REQUIRE(stride_r >= 0 && stride_k >= 0, HPFP8_ERR_SHAPE, "%s: negative %s stride", what, name);
+  if (rows == 0) return 1;
+  HPFP8_REQUIRE(((rows - 1) * stride_r + (kblocks - 1) * stride_k + 1) * 4 < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
+                "%s: the %s array spans 2 GiB or more", what, name);
   return 1;
 }
 
@@ -476,9 +684,15 @@ int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa
   GemmParams p{};
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = ldb;
   p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k; p.sb_sn = sb_stride_n; p.sb_sk = sb_stride_k;
+  rc = check_scale_span("gemm_blockwise", M, K / BK, sa_stride_m, sa_stride_k, "sa");
+  if (rc <= 0) return rc;
+  rc = check_scale_span("gemm_blockwise", sb_gran == 128 ? N / kBlock : N, K / BK, sb_stride_n, sb_stride_k, "sb");
+  if (rc <= 0) return rc;
+  p.sb_bytes = (int)(((N / kBlock - 1) * sb_stride_n + (K / BK - 1) * sb_stride_k + 1) * 4);
   p.c = c; p.ldc = ldc; p.bias = (const uint16_t*)bias;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.accumulate = accumulate;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  p.tiles = (int)tiles;
   if (sb_gran == 128) return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
   // per-row b scales travel to LDS as one contiguous 1 KB piece per k-block
   HPFP8_REQUIRE(sb_stride_n == 1 && sb_stride_k >= N && sb_stride_k % 4 == 0 && aligned16(sb), HPFP8_ERR_SHAPE,
@@ -499,6 +713,7 @@ int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const
   p.c = c; p.ldc = ldc; p.bias = (const uint16_t*)bias;
   p.M = (int)M; p.N = (int)N; p.K = (int)K;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  p.tiles = (int)tiles;
   return launch<kScaleTensor, false>(p, out_type, tiles, (hipStream_t)stream);
 }
 
@@ -515,6 +730,10 @@ int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, in
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = K;
   p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k;
   p.sb_sn = K / BK; p.sb_sk = 1; p.sb_se = (N / kBlock) * (K / BK);
+  rc = check_scale_span("gemm_grouped", total_m, K / BK, sa_stride_m, sa_stride_k, "sa");
+  if (rc <= 0) return rc;
+  HPFP8_REQUIRE((int64_t)experts * p.sb_se * 4 < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE, "gemm_grouped: b scale array exceeds 2 GiB");
+  p.sb_bytes = (int)((int64_t)experts * p.sb_se * 4);
   p.c = c; p.ldc = ldc; p.offs = offs; p.experts = experts;
   p.M = (int)total_m; p.N = (int)N; p.K = (int)K;
   // upper bound on row tiles: every expert may add one partial tile
