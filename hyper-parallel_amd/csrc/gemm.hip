@@ -7,13 +7,16 @@
 //     one FMA per element (acc += partial * sa * sb).
 //   * The weight-like operand b feeds the MFMA "A" port and the activation-like operand a the
 //     "B" port: a lane then holds 4 consecutive n for one m, which makes the per-row scale
-//     sa(m,kb) a per-lane constant and the bf16 store 8 contiguous bytes.
+//     sa(m,kb) a per-lane constant.
 //   * Workgroup tile 256(m) x 256(n) x 128(k), 8 waves as 4(m) x 2(n), wave tile 64 x 128
 //     (128 fp32 accumulators per lane, 2 waves per SIMD so one wave's FMAs overlap the other's
-//     MFMAs).  Two LDS stages of 64 KB; tiles are DMA'd global -> LDS with 128-bit buffer loads
-//     (out-of-range rows read as zero), 16-byte chunks XOR-swizzled by row so that both the DMA
-//     writes and the ds_read_b128 fragment reads are bank-conflict free.
-//   * Workgroup ids are remapped so that each XCD (own L2) works on a contiguous run of tiles.
+//     MFMAs).  LDS holds two buffers for the a tile and three for the b tile (32 KB each); tiles
+//     are DMA'd global -> LDS with 128-bit buffer loads (out-of-range rows read as zero), 16-byte
+//     chunks XOR-swizzled by row so that both the DMA writes and the ds_read_b128 fragment reads
+//     are bank-conflict free.
+//   * The grid is persistent: one workgroup per CU walks a list of tiles, and the rounds of
+//     consecutive tiles follow each other without a gap.  Each XCD (own L2) owns a contiguous run
+//     of tile numbers.
 #include <type_traits>
 
 #include "hpfp8_device.h"

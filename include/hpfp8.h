@@ -123,7 +123,8 @@ int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t
  *        wgrad    a = grad_out^T codes (128x1 requant), b = x^T codes,    sb_gran = 1; the b scales must
  *                 then be k-block-major: sb_stride_n = 1, sb_stride_k >= N (what the *_kmajor quantizers write)
  * bias: bf16[N] or NULL.  out_type HPFP8_OUT_BF16 / HPFP8_OUT_F32; ldc = row stride of c in
- * elements.  accumulate != 0 (fp32 output only) adds into c instead of overwriting it, the fp32
+ * elements, a multiple of 8 (bf16) or 4 (fp32): rows are written in 16-byte pieces.  Scale strides are
+ * non-negative; each operand and each scale array must span less than 2 GiB (HPFP8_ERR_SHAPE otherwise).  accumulate != 0 (fp32 output only) adds into c instead of overwriting it, the fp32
  * main-grad bookkeeping of hyper_parallel/platform/torch/fully_shard/param.py:134-167. */
 int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                          const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
