@@ -310,7 +310,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     for (int j = 0; j < 4; ++j) acc[i][j] = zero;
 
   // ---- prologue: k-block 0 of both operands, k-block 1 of b where it has three buffers, and the
-  // first half of a's k-block 1
+  // first half of k-block 1 of a (and of b where it has two buffers)
   float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_raw[5] = {1.f, 1.f, 1.f, 1.f, 1.f};
   scale_target(T0);
   load_scales(0, s_raw);
@@ -334,6 +334,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     const __amdgpu_buffer_rsrc_t ra1 = rsrc_a_of(t1);
     issue_tile(ra1, a_off, 1, kb1, 0);
     issue_tile(ra1, a_off, 1, kb1, 1);
+    if (kBAhead == 1) {
+      const __amdgpu_buffer_rsrc_t rb1 = rsrc_b_of(t1);
+      issue_tile(rb1, b_off, 3, kb1, 0);
+      issue_tile(rb1, b_off, 3, kb1, 1);
+    }
   }
 
   // The synchronisation point of a round sits before its last two n-subtiles, not at its end: what
@@ -356,34 +361,33 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   int bbuf = 0;                        // b buffer holding the current k-block
   int sbuf = 0;                        // scale stage (wgrad form) holding the current k-block
   // transfer targets (ordinal in the tile list) and their buffer resources
-  int ord_1 = 0, ord_2 = 0, ord_b = 0;
+  int ord_1 = 0, ord_2 = 0;
   TileInfo tile_1 = T0;
-  __amdgpu_buffer_rsrc_t rs_a1 = rsrc_a_of(T0), rs_a2 = rs_a1, rs_b = rsrc_b_of(T0);
+  __amdgpu_buffer_rsrc_t rs_a1 = rsrc_a_of(T0), rs_a2 = rs_a1, rs_b1 = rsrc_b_of(T0), rs_b2 = rs_b1;
 
   for (int tile = 0; tile < my_tiles; ++tile) {
   for (int kb = 0; kb < kblocks; ++kb) {
     // Where this round's transfers and scale loads go: one k-block ahead (scales, second half of
-    // that a tile), two ahead (first half of that a tile), kBAhead ahead (b tile).  Only in the last
+    // those tiles), two ahead (first half of those tiles, or the whole b tile when it has three
+    // buffers).  Only in the last
     // two rounds of a tile does a target move on to the next tile of the list; its resource is
     // rebuilt then and stays valid when that tile becomes the current one.
-    int kb1 = kb + 1, kb2 = kb + 2, kbb = kb + kBAhead;
+    int kb1 = kb + 1, kb2 = kb + 2;
     if (kb2 >= kblocks) {
       const int o1 = tile + tiles_ahead(kb, 1, kblocks, kb1);
       const int o2 = tile + tiles_ahead(kb, 2, kblocks, kb2);
-      const int ob = tile + tiles_ahead(kb, kBAhead, kblocks, kbb);
       if (o1 != ord_1) {
         ord_1 = o1;
         tile_1 = pick_tile(o1 - tile, T0, T1, T2);
         rs_a1 = rsrc_a_of(tile_1);
+        if (kBAhead == 1) rs_b1 = rsrc_b_of(tile_1);
         scale_target(tile_1);
       }
       if (o2 != ord_2) {
         ord_2 = o2;
-        rs_a2 = rsrc_a_of(pick_tile(o2 - tile, T0, T1, T2));
-      }
-      if (ob != ord_b) {
-        ord_b = ob;
-        rs_b = rsrc_b_of(pick_tile(ob - tile, T0, T1, T2));
+        const TileInfo t2 = pick_tile(o2 - tile, T0, T1, T2);
+        rs_a2 = rsrc_a_of(t2);
+        rs_b2 = rsrc_b_of(t2);
       }
     }
     load_scales(kb1, s_raw);
@@ -394,14 +398,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     const uint8_t* bnxt = lds + (2 + bnext) * kTileBytes;
     const uint8_t* anxt = lds + (stage ^ 1) * kTileBytes;
     int snext = sbuf + 1 == 3 ? 0 : sbuf + 1;
-    // Per round: the rest of the next a tile at subtiles 0,1; the b tile at 2..5; after the barrier
-    // the first half of the a tile after next, into the buffer whose fragments every wave has just
-    // left behind.  One transfer per subtile: a burst would queue up in the texture path ahead of
-    // the LDS reads.
+    // Per round, with three b buffers: the rest of the next a tile at subtiles 0,1; the b tile two
+    // rounds ahead at 2..5; after the barrier the first half of the a tile after next, into the
+    // buffer whose fragments every wave has just left behind.  One transfer per subtile: a burst
+    // would queue up in the texture path ahead of the LDS reads.
+    // With two b buffers (wgrad form) the b tile has to land within one round like the a tile, so
+    // both go out in the four subtiles that follow the barrier, one transfer of each per subtile.
     auto issue_slot = [&](int i) {
-      if (i < 2) issue_tile(rs_a1, a_off, stage ^ 1, kb1, i + 2);
-      else if (i < 6) issue_tile(rs_b, b_off, 2 + bbuf_issue, kbb, i - 2);
-      else issue_tile(rs_a2, a_off, stage, kb2, i - 6);
+      if (kBAhead == 2) {
+        if (i < 2) issue_tile(rs_a1, a_off, stage ^ 1, kb1, i + 2);
+        else if (i < 6) issue_tile(rs_b2, b_off, 2 + bbuf_issue, kb2, i - 2);
+        else issue_tile(rs_a2, a_off, stage, kb2, i - 6);
+      } else if (i < 2) {
+        issue_tile(rs_a1, a_off, stage ^ 1, kb1, i + 2);
+        issue_tile(rs_b1, b_off, 2 + bnext, kb1, i + 2);
+      } else if (i >= 6) {
+        issue_tile(rs_a2, a_off, stage, kb2, i - 6);
+        issue_tile(rs_b2, b_off, 2 + bbuf, kb2, i - 6);
+      }
     };
     auto round_sync = [&]() {
       // Own transfers for the next round have landed and own LDS reads of this round's buffers are
@@ -521,11 +535,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   asm volatile("" : "+v"(lane_e));
   const int l16e = lane_e & 15, ge = lane_e >> 4;
   uint8_t* stg = lds + (2 + (bbuf == 0 ? kBStages - 1 : bbuf - 1)) * kTileBytes + wave * 4096;
+  // With two b buffers the lower half of that slice already receives the next transfers: rows 0..7
+  // then go to its upper half and rows 8..15 to the upper half of this wave's slice of the a buffer
+  // that is being refilled (its upper half is filled after these stores).
+  uint8_t* stg_hi = kBAhead == 1 ? lds + (stage ^ 1) * kTileBytes + wave * 4096 + 2048 : stg + 2048;
+  if (kBAhead == 1) stg += 2048;
+  auto stg_row = [&](int row) { return (row < 8 ? stg : stg_hi) + (row & 7) * 256; };
   const int ncol = n0 + wn * 128;                 // first column of the wave tile
   const bool cols_ok = ncol < N;
   constexpr int kHalves = OUT_F32 ? 2 : 1;       // fp32 rows of 128 columns take two slices
   constexpr int kPerHalf = 8 / kHalves;           // n-subtiles per slice
-  const uint32_t stg_w = (uint32_t)(uintptr_t)(lds_ptr_t)stg + l16e * 256;   // LDS byte address of this lane's row
+  const uint32_t stg_w = (uint32_t)(uintptr_t)(lds_ptr_t)stg_row(l16e);   // LDS byte address of this lane's row
   auto store_tile = [&](auto with_bias, auto full_rows) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -564,7 +584,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
             const int row = 4 * (k2 + k) + ge;
-            val[k] = *reinterpret_cast<const v4i*>(stg + row * 256 + ((l16e ^ row) * 16));
+            val[k] = *reinterpret_cast<const v4i*>(stg_row(row) + ((l16e ^ row) * 16));
           }
 #pragma unroll
           for (int k = 0; k < 2; ++k) {

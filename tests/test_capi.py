@@ -57,6 +57,15 @@ def test_argument_errors_are_reported_without_launching():
     # accumulate needs fp32 output
     rc = lib.hpfp8_gemm_blockwise(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 128, 128, 128, None, p, 128, 0, 1, None)
     assert rc == -1
+    # rows of c are written in 16-byte pieces: ldc a multiple of 8 for bf16, of 4 for fp32
+    rc = lib.hpfp8_gemm_blockwise(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 128, 128, 128, None, p, 132, 0, 0, None)
+    assert rc == -3 and b"ldc" in lib.hpfp8_last_error()
+    # negative scale stride
+    rc = lib.hpfp8_gemm_blockwise(p, 128, p, -1, 1, p, 128, p, 1, 1, 128, 128, 128, 128, None, p, 128, 0, 0, None)
+    assert rc == -2 and b"stride" in lib.hpfp8_last_error()
+    # a scale array spanning 2 GiB or more
+    rc = lib.hpfp8_gemm_blockwise(p, 128, p, 1 << 30, 1, p, 128, p, 1, 1, 128, 128, 128, 128, None, p, 128, 0, 0, None)
+    assert rc == -2 and b"2 GiB" in lib.hpfp8_last_error()
     # empty problems succeed without touching the device
     assert lib.hpfp8_quantize_1x128_bf16(None, 0, 128, None, None, None, None) == 0
     assert lib.hpfp8_gemm_per_tensor(None, 128, None, None, 128, None, 0, 128, 128, None, None, 128, 0, None) == 0

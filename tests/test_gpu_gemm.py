@@ -122,6 +122,25 @@ def test_cfg1_per_tensor_linear(gpu):
     assert rel(U.f32(y), exact.numpy()) < 0.05
 
 
+def test_output_row_stride_and_many_tiles_per_workgroup(gpu):
+    """c may be a column slice of a wider buffer (ldc > N), and the neighbouring columns must stay
+    untouched; 1200 tiles on a grid of one workgroup per CU gives every workgroup several tiles."""
+    import hpfp8
+    M, N, K = 5000, 15360, 256
+    x = U.randn_bf16((M, K), 11, 1.0, 0.001, 50.0).to(gpu)
+    w = U.randn_bf16((N, K), 12, 0.006).to(gpu)
+    xq, sxi = hpfp8.quantize_1x128(x, kmajor=True)
+    wq, swi = hpfp8.quantize_128x128(w)
+    ref = ref_f64_torch(xq, sxi, wq, swi.repeat_interleave(128, dim=0), gpu)
+    for dt, tol in ((torch.float32, TOL_F32), (torch.bfloat16, TOL_BF16)):
+        wide = torch.full((M, N + 24), 7.0, dtype=dt, device=gpu)
+        out = wide[:, 8:8 + N]
+        hpfp8.gemm_blockwise(xq, sxi, wq, swi, out=out)
+        assert rel(U.f32(out), ref.cpu().numpy()) < tol
+        assert bool((wide[:, :8] == 7.0).all()) and bool((wide[:, 8 + N:] == 7.0).all())
+        assert torch.equal(out, hpfp8.gemm_blockwise(xq, sxi, wq, swi, out_dtype=dt))
+
+
 @pytest.mark.parametrize("M,N,K,seed", [(256, 256, 128, 1), (512, 1024, 7168, 2), (1000, 384, 1024, 3),
                                          (8, 128, 256, 4), (4096, 512, 2048, 5)])
 def test_blockwise_forward_shapes(gpu, M, N, K, seed):
