@@ -137,6 +137,11 @@ def other_configs(dev):
         "requant_t_x": gb(m * k * 3 + k * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(x, kmajor=True))),
         "requant_t_grad_out": gb(m * n * 3 + n * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(go, kmajor=True))),
         "quantize_grad_out": gb(m * n * 3 + m * (n // 128) * 4, _time(lambda: hpfp8.quantize_1x128(go, kmajor=True))),
+        # both operand forms from one read (what fp8_linear uses in training): 2 + 1 + 1 bytes per element + scales
+        "quantize_both_forms_x": gb(m * k * 4 + 2 * m * (k // 128) * 4,
+                                    _time(lambda: hpfp8.quantize_1x128_and_128x1_t(x, kmajor=True))),
+        "quantize_both_forms_grad_out": gb(m * n * 4 + 2 * m * (n // 128) * 4,
+                                           _time(lambda: hpfp8.quantize_1x128_and_128x1_t(go, kmajor=True))),
         "dgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq, sgo, wqt, sw.t()))),
         "wgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1))),
     }

@@ -267,16 +267,22 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // ---------------------------------------------------------------------------------------------
 // 128x1 groups, transposed output (wgrad operands): x[M,K] -> qt[K,M], scales [K, M/128]
 // ---------------------------------------------------------------------------------------------
-template <bool KMAJOR>
+// With DUAL the same pass also writes the 1x128 quantization of x itself (codes q[M,K], one scale per
+// row and 128 columns: [M, K/128], or [K/128, M] with KMAJOR): forward / dgrad operand and wgrad
+// operand from one read of the bf16 source.
+template <bool KMAJOR, bool DUAL>
 __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int m, int k,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale_t,
-                                                            float* __restrict__ scale_inv_t) {
+                                                            float* __restrict__ scale_inv_t,
+                                                            uint8_t* __restrict__ q, float* __restrict__ scale_r,
+                                                            float* __restrict__ scale_inv_r) {
   const int kb = k >> 7, mb = m >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   const int wave = threadIdx.x >> 6;
   __shared__ uint32_t part[4][64];  // [wave][cg*4 + word]
   __shared__ float s_scale[128];
+  __shared__ float s_row[DUAL ? 256 : 2];   // scale, scale_inv of the tile's 128 rows
   __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
   // A workgroup walks kTilesPerBlock tiles down a tile column (tr fastest), loading tile t+1 before
   // the LDS phases of tile t.
@@ -313,7 +319,28 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
 #pragma unroll
       for (int i = 0; i < 4; ++i) part[wave][cg * 4 + i] = cm[i];
     }
+    if (DUAL) {
+      // the 16 threads of a row quad hold a whole 128-column group of each of their 8 rows
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const int row = tile_row(rq, p);
+        const uint32_t mr = row16_max_u32(mag8(v[p]));
+        float s, si;
+        scales_from_amax(__uint_as_float(mr << 16), s, si);
+        *reinterpret_cast<uint2*>(q + ((int64_t)tr * 128 + row) * k + tc * 128 + cg * 8) = cvt8<false>(v[p], s);
+        if (cg == 0) {
+          s_row[row] = s;
+          s_row[128 + row] = si;
+        }
+      }
+    }
     __syncthreads();
+    if (DUAL && threadIdx.x >= 128) {
+      const int row = threadIdx.x - 128;
+      const int64_t o = KMAJOR ? (int64_t)tc * m + tr * 128 + row : ((int64_t)tr * 128 + row) * kb + tc;
+      if (scale_r) scale_r[o] = s_row[row];
+      scale_inv_r[o] = s_row[128 + row];
+    }
     if (threadIdx.x < 128) {
       const int col = threadIdx.x, word = col >> 1;
       uint32_t mw = pk_max_u16(pk_max_u16(part[0][word], part[1][word]), pk_max_u16(part[2][word], part[3][word]));
@@ -531,8 +558,10 @@ int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void*
   return check_launch("quantize_128x128");
 }
 
+// q != nullptr: also the 1x128 quantization of x itself (codes q, scales scale / scale_inv).
 static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, int64_t m, int64_t k, void* q_t,
-                                 int64_t ld_t, float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
+                                 int64_t ld_t, float* scale_t, float* scale_inv_t, hpfp8_stream_t stream,
+                                 void* q = nullptr, float* scale = nullptr, float* scale_inv = nullptr) {
   HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)m, (long long)k);
@@ -544,13 +573,23 @@ static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, i
   HPFP8_REQUIRE(aligned16(x) && aligned16(q_t), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
   HPFP8_REQUIRE(ld_t >= m && ld_t % 16 == 0, HPFP8_ERR_SHAPE, "%s: ld_t=%lld must be a multiple of 16 and at least m",
                 what, (long long)ld_t);
+  HPFP8_REQUIRE(!q || (scale_inv && aligned16(q)), HPFP8_ERR_ARG, "%s: q needs scale_inv and 16-byte alignment", what);
   hipStream_t s = (hipStream_t)stream;
-  if (kmajor)
-    quant_128x1_t_kernel<true><<<(unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock), 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
-                                                                 ld_t, scale_t, scale_inv_t);
-  else
-    quant_128x1_t_kernel<false><<<(unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock), 256, 0, s>>>((const uint16_t*)x, (int)m, (int)k, (uint8_t*)q_t,
-                                                                  ld_t, scale_t, scale_inv_t);
+  const unsigned grid = (unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock);
+  const uint16_t* xs = (const uint16_t*)x;
+  uint8_t* qt8 = (uint8_t*)q_t;
+  uint8_t* q8 = (uint8_t*)q;
+  if (q) {
+    if (kmajor)
+      quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv);
+    else
+      quant_128x1_t_kernel<false, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv);
+  } else {
+    if (kmajor)
+      quant_128x1_t_kernel<true, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr);
+    else
+      quant_128x1_t_kernel<false, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr);
+  }
   return check_launch(what);
 }
 
@@ -562,6 +601,14 @@ int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, 
 int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t,
                                        float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
   return quantize_128x1_t_impl("quantize_128x1_t_kmajor", true, x, m, k, q_t, ld_t, scale_t, scale_inv_t, stream);
+}
+
+int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, int kmajor, void* q, float* scale,
+                                          float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
+                                          float* scale_inv_t, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(m == 0 || k == 0 || q != nullptr, HPFP8_ERR_ARG, "quantize_1x128_and_128x1_t: null buffer");
+  return quantize_128x1_t_impl("quantize_1x128_and_128x1_t", kmajor != 0, x, m, k, q_t, ld_t, scale_t, scale_inv_t,
+                               stream, q, scale, scale_inv);
 }
 
 int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,

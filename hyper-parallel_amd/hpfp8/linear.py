@@ -9,7 +9,8 @@ tensors it also fits `custom_shard(func, ...)` (hyper_parallel/core/shard/local_
 
 Recipes
   "blockwise"  : activations / output gradients 1x128, weights 128x128; wgrad operands are
-                 re-quantized 128x1 (transposed) from the bf16 sources.
+                 quantized 128x1 (transposed) from the bf16 sources, in the same pass that makes
+                 the 1x128 codes where both are needed.
   "per_tensor" : one scale per tensor (amax -> 448/amax); backward also per tensor.
 """
 from __future__ import annotations
@@ -32,41 +33,55 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias):
         x2 = _flatten(x)
-        xq, sx = ops.quantize_1x128(x2, kmajor=True)
-        need_wgrad_inputs = x.requires_grad or weight.requires_grad
+        m = x2.shape[0]
+        # With a weight gradient to come and a token count that allows it, x is read once: its 1x128
+        # codes for this GEMM and its transposed 128x1 codes for wgrad, which are what is kept for
+        # backward (1 byte per element instead of the bf16 source).
+        fused = weight.requires_grad and m % ops.BLOCK == 0 and m > 0
+        if fused:
+            xq, sx, xt, sxt = ops.quantize_1x128_and_128x1_t(x2.contiguous(), kmajor=True)
+        else:
+            xq, sx = ops.quantize_1x128(x2, kmajor=True)
+            xt = sxt = None
         if x.requires_grad:
             wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
         else:
             wq, sw = ops.quantize_128x128(weight)
             wqt = None
         y = ops.gemm_blockwise(xq, sx, wq, sw, bias=bias)
-        ctx.save_for_backward(x2 if weight.requires_grad else None, wqt, sw)
+        ctx.save_for_backward(x2 if (weight.requires_grad and not fused) else None, xt, sxt, wqt, sw)
         ctx.x_shape = x.shape
         ctx.has_bias = bias is not None
-        ctx.need = (x.requires_grad, weight.requires_grad, need_wgrad_inputs)
+        ctx.need = (x.requires_grad, weight.requires_grad)
         return y.reshape(x.shape[:-1] + (weight.shape[0],))
 
     @staticmethod
     def backward(ctx, grad_out):
-        x2, wqt, sw = ctx.saved_tensors
-        need_dx, need_dw, _ = ctx.need
+        x2, xt, sxt, wqt, sw = ctx.saved_tensors
+        need_dx, need_dw = ctx.need
         go = _flatten(grad_out)
         if go.dtype != torch.bfloat16:
             go = go.to(torch.bfloat16)
         go = go.contiguous()
+        m = go.shape[0]
+        if need_dw and m % ops.BLOCK:
+            raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
         dx = dw = db = None
+        goq = sgo = got = sgot = None
+        if need_dx and need_dw:
+            goq, sgo, got, sgot = ops.quantize_1x128_and_128x1_t(go, kmajor=True)   # one read of grad_out
+        elif need_dx:
+            goq, sgo = ops.quantize_1x128(go, kmajor=True)
+        elif need_dw:
+            got, sgot = ops.quantize_128x1_t(go, kmajor=True)
         if need_dx:
             # dx[M,K] = go[M,N] . W[N,K]: contraction over N, b operand = W^T codes [K,N] whose
             # 128x128 scales are W's with the two strides swapped.
-            goq, sgo = ops.quantize_1x128(go, kmajor=True)
             dx = ops.gemm_blockwise(goq, sgo, wqt, sw.t()).reshape(ctx.x_shape)
         if need_dw:
             # dW[N,K] = go^T[N,M] . x[M,K]: contraction over tokens, both operands 1x128 along M
-            m = go.shape[0]
-            if m % ops.BLOCK:
-                raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
-            got, sgot = ops.quantize_128x1_t(go, kmajor=True)
-            xt, sxt = ops.quantize_128x1_t(x2, kmajor=True)
+            if xt is None:
+                xt, sxt = ops.quantize_128x1_t(x2, kmajor=True)
             dw = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)

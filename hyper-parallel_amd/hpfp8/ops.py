@@ -191,6 +191,29 @@ def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = F
     return (qt, scale, scale_inv) if want_scale else (qt, scale_inv)
 
 
+def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True):
+    """Both operand forms of x[M, K] from one read of it.
+
+    Returns (codes[M, K], scale_inv[M, K/128], codes_t[K, M], scale_inv_t[K, M/128]), bit-identical to
+    ``quantize_1x128(x, kmajor=kmajor)`` and ``quantize_128x1_t(x, kmajor=kmajor)``.  M and K multiples of 128.
+    """
+    x = _check_bf16(x, "x")
+    if x.dim() != 2:
+        raise ValueError("x must be 2-D")
+    m, k = x.shape
+    if m % BLOCK or k % BLOCK:
+        raise ValueError(f"shape {tuple(x.shape)} is not a multiple of {BLOCK} in both dims")
+    q = torch.empty((m, k), dtype=FP8, device=x.device)
+    qt = _empty_codes_t(k, m, x.device)
+    s_inv = torch.empty((k // BLOCK, m) if kmajor else (m, k // BLOCK), dtype=torch.float32, device=x.device)
+    st_inv = torch.empty((m // BLOCK, k) if kmajor else (k, m // BLOCK), dtype=torch.float32, device=x.device)
+    _lib.call("hpfp8_quantize_1x128_and_128x1_t_bf16", _ptr(x), m, k, int(kmajor), _ptr(q), None, _ptr(s_inv),
+              _ptr(qt), _ld(qt), None, _ptr(st_inv), _stream())
+    if kmajor:
+        s_inv, st_inv = s_inv.t(), st_inv.t()
+    return q, s_inv, qt, st_inv
+
+
 def dequantize_1x128(q: torch.Tensor, scale_inv: torch.Tensor, grad_scale: float = 1.0) -> torch.Tensor:
     """codes[..., C] with scale_inv[..., C/128] -> bf16."""
     q = _check_fp8(q, "q")

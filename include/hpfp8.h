@@ -99,6 +99,17 @@ int hpfp8_quantize_128x1_t_bf16(const void* x, int64_t m, int64_t k, void* q_t, 
 int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t,
                                        float* scale_t, float* scale_inv_t, hpfp8_stream_t stream);
 
+/* Both quantizations of one bf16 matrix from one read of it: the 1x128 form (forward / dgrad
+ * operand: q[m, k], scales [m, k/128], or [k/128, m] when kmajor != 0) and the transposed 128x1 form
+ * (wgrad operand: q_t[k, m] with row stride ld_t, scales [k, m/128], or [m/128, k] when kmajor != 0).
+ * Codes and scales are bit-identical to hpfp8_quantize_1x128[_kmajor]_bf16 and
+ * hpfp8_quantize_128x1_t[_kmajor]_bf16 on the same input.  m and k multiples of 128.  Serves the same
+ * call site as those two (operand preparation for hyper_parallel/core/shard/_op_dispatch.py:277-283,
+ * forward and backward). */
+int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, int kmajor, void* q, float* scale,
+                                          float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
+                                          float* scale_inv_t, hpfp8_stream_t stream);
+
 /* ---- dequantizers ----------------------------------------------------------------------------
  * The cast-back site hyper_parallel/core/hsdp/hsdp_grad_buffer.py:116-125: out = bf16(decode(q)
  * * scale_inv); when grad_scale != 1 the bf16 result is multiplied by it and rounded again. */

@@ -94,6 +94,14 @@ def test_seeded_parity_all_quantizers(gpu, shape, seed, std, of, om):
     qt, s, si = hpfp8.quantize_128x1_t(xg, want_scale=True)
     rq, rs, rsi = C.quantize_128x1_t(xb)
     assert np.array_equal(U.codes(qt), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    # both forms from one read of x: same codes and scales as the two separate quantizers
+    rq1, _, rsi1 = C.quantize_1x128(xb)
+    for kmajor in (True, False):
+        q1, si1, qt2, sit2 = hpfp8.quantize_1x128_and_128x1_t(xg, kmajor=kmajor)
+        assert np.array_equal(U.codes(q1), rq1) and eq_f32(si1, rsi1)
+        assert np.array_equal(U.codes(qt2), rq) and eq_f32(sit2, rsi)
+        if min(si1.shape) > 1 and min(sit2.shape) > 1:      # (strides of a one-column tensor say nothing)
+            assert (si1.stride(0) == 1) == kmajor and (sit2.stride(0) == 1) == kmajor
 
 
 @pytest.mark.parametrize("shape", [(512, 7168), (100, 384), (16, 128), (33, 640)])
