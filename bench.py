@@ -181,6 +181,19 @@ def other_configs(dev):
         "quantize": gb(nbytes, _time(lambda: hpfp8.quantize_bucket(flat))),
         "dequantize": gb(nbytes, _time(lambda: hpfp8.dequantize_bucket(codes, si))),
     }
+    # the same 2^29 elements as 72 separate gradients (64 of 2048x4096 minus 8 of them split into
+    # bias-sized pieces): packing fused with the quantization, and the cast back fused with the unpacking
+    sizes = [2048 * 4096] * 56 + [7168] * 8 + [2048 * 4096 * 8 - 7168 * 8]
+    views, pos = [], 0
+    for n_ in sizes:
+        views.append(flat[pos:pos + n_])
+        pos += n_
+    bucket = hpfp8.Fp8GradBucket(sizes, shard_size=1, grad_scale=0.5)
+    q2, si2 = bucket.pack(views)
+    outs = [torch.empty(n_, dtype=torch.bfloat16, device=dev) for n_ in sizes]
+    res["cfg5_bucket"]["pack_and_quantize_72_grads"] = gb(nbytes, _time(lambda: bucket.pack(views)))
+    res["cfg5_bucket"]["dequantize_and_unpack_72_grads"] = gb(
+        nbytes, _time(lambda: bucket.unpack(q2[0], si2[0], outs)))
     return res
 
 

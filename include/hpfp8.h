@@ -118,6 +118,29 @@ int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t r
 int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
                                   void* out, hpfp8_stream_t stream);
 
+/* ---- gradient bucket: pack + quantize, dequantize + unpack -------------------------------------
+ * The FP8 form of HSDPGradBuffer._copy_grad_to_unsharded_buffer and ._set_grad_data
+ * (hyper_parallel/core/hsdp/hsdp_grad_buffer.py:95-108, :116-135).  The bucket is `shards` rows of
+ * row_elems elements (a multiple of 128); parameter e owns elements [offsets[e], offsets[e] +
+ * numels[e]) of every row, offsets ascending multiples of 128 starting at 0, the gap up to the next
+ * offset (or the end of the row) is padding.  grads, numels, offsets are HOST arrays of `entries`
+ * items; grads[e] is a device pointer to bf16 data.
+ *
+ * pack:   row s of the bucket = chunk s of every gradient (grads[e] holds shards * numels[e]
+ *         elements, chunk s = elements [s * numels[e], (s + 1) * numels[e])), quantized in 1x128
+ *         groups along the row: q[shards, row_elems] E4M3, scale / scale_inv [shards, row_elems / 128]
+ *         (scale may be NULL).  Padding is written as zero codes.  Same codes and scales as
+ *         hpfp8_quantize_1x128_bf16 on the packed bf16 rows.
+ * unpack: one (reduced) row q[row_elems], scale_inv[row_elems / 128] -> grads[e][0 .. numels[e]) =
+ *         bf16(decode * scale_inv), then, when grad_scale != 1, bf16(that * grad_scale): the order of
+ *         hsdp_grad_buffer.py:121-125.  Same values as hpfp8_dequantize_1x128_bf16 on the row. */
+int hpfp8_bucket_pack_quantize_bf16(const void* const* grads, const int64_t* numels, const int64_t* offsets,
+                                    int entries, int shards, int64_t row_elems, void* q, float* scale,
+                                    float* scale_inv, hpfp8_stream_t stream);
+int hpfp8_bucket_unpack_dequantize_bf16(void* const* grads, const int64_t* numels, const int64_t* offsets,
+                                        int entries, int64_t row_elems, const void* q, const float* scale_inv,
+                                        float grad_scale, hpfp8_stream_t stream);
+
 /* ---- scaled FP8 GEMMs -------------------------------------------------------------------------
  * Replace aten::linear (forward) and its autograd backward (dgrad, wgrad) as called from
  * hyper_parallel/core/shard/_op_dispatch.py:277-283.

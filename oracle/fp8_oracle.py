@@ -254,6 +254,41 @@ def dequantize_bucket(codes: np.ndarray, scale_inv: np.ndarray, grad_scale: floa
     return bits
 
 
+def bucket_offsets(numels):
+    """Start of every parameter in a bucket row and the row length: the running index of
+    hyper_parallel/core/hsdp/hsdp_grad_buffer.py:72-80, with every start rounded up to a multiple
+    of 128 (so that no scaling group straddles two parameters)."""
+    offsets, end = [], 0
+    for n in numels:
+        offsets.append(end)
+        end = -(-(end + int(n)) // BLOCK) * BLOCK
+    return offsets, end
+
+
+def pack_bucket(grad_bits, numels, shard_size: int = 1) -> np.ndarray:
+    """bf16 bit patterns of the packed bucket [shard_size, row_elems]: row s holds chunk s of every
+    gradient at that parameter's offset (`buffer[:, start:end] = grad.view(shard_size, -1)`,
+    hsdp_grad_buffer.py:95-108); padding is zero."""
+    offsets, row = bucket_offsets(numels)
+    out = np.zeros((shard_size, row), dtype=np.uint16)
+    for g, n, o in zip(grad_bits, numels, offsets):
+        g = np.asarray(g, dtype=np.uint16).reshape(-1)
+        if g.size != shard_size * n:
+            raise ValueError("gradient size does not match shard_size * numel")
+        out[:, o:o + n] = g.reshape(shard_size, n)
+    return out
+
+
+def unpack_bucket(row_bits: np.ndarray, numels):
+    """Pieces of one (reduced) bucket row, one per parameter (`buffer[:, start:end]`,
+    hsdp_grad_buffer.py:126-135)."""
+    offsets, row = bucket_offsets(numels)
+    row_bits = np.asarray(row_bits).reshape(-1)
+    if row_bits.size != row:
+        raise ValueError("row has the wrong length")
+    return [row_bits[o:o + n].copy() for n, o in zip(numels, offsets)]
+
+
 # --------------------------------------------------------------------------------------
 # GEMMs.  All return fp32 [M, N] before the final rounding plus the bf16 bit patterns.
 # a: codes [M, K]; b: codes [N, K]  (weight layout [out, in], contraction on the last dim of

@@ -191,3 +191,51 @@ def test_bucket_full_size_properties(gpu):
     c8 = codes.view(torch.uint8).view(-1, 128)
     assert not bool(((c8 & 0x7F) == 0x7F).any())
     assert bool((((c8 & 0x7F) == 0x7E).any(dim=1)).all())
+
+
+@pytest.mark.parametrize("shard_size,grad_scale", [(1, 1.0), (2, 0.125), (4, 0.3)])
+def test_fused_bucket_pack_and_unpack(gpu, shard_size, grad_scale):
+    """Fp8GradBucket.pack == quantize_1x128 of the oracle's packed rows; unpack == the oracle's cast
+    back of one row, sliced.  Sizes cover: multiples of 128, a ragged tail (zero-padded group), a
+    parameter smaller than one vector, odd chunk sizes (unaligned chunk starts for shard_size > 1),
+    more parameters than one launch carries, and one parameter spanning several workgroups."""
+    import hpfp8
+    numels = [384 * 256, 1000, 7, 128, 129, 4099, 20000] + [256 + 8 * i for i in range(60)]
+    rng = np.random.default_rng(13)
+    grads = []
+    for e, n in enumerate(numels):
+        g = U.randn_bf16((shard_size * n,), 100 + e, 1e-3 * (1 + e % 5), 0.002, 200.0)
+        grads.append(g)
+    bucket = hpfp8.Fp8GradBucket(numels, shard_size=shard_size, grad_scale=grad_scale)
+    offsets, row = O.bucket_offsets(numels)
+    assert bucket.offsets == offsets and bucket.row_elems == row
+    q, si = bucket.pack([g.to(gpu) for g in grads])
+    packed = O.pack_bucket([U.bits(g) for g in grads], numels, shard_size)
+    rq, _, rsi = O.quantize_1x128(packed)
+    assert np.array_equal(U.codes(q), rq)
+    assert np.array_equal(U.f32_bits(U.f32(si)), U.f32_bits(rsi))
+    # the reduced row: take row (shard_size - 1) as it is (a real reduction would produce another row of codes)
+    r = shard_size - 1
+    outs = [torch.full((n,), 7.0, dtype=torch.bfloat16, device=gpu) for n in numels]
+    bucket.unpack(q[r].contiguous(), si[r].contiguous(), outs)
+    back = O.dequantize_bucket(rq[r], rsi[r], grad_scale)
+    for e, piece in enumerate(O.unpack_bucket(back, numels)):
+        assert np.array_equal(U.bits(outs[e]), piece), e
+    # same values as the unfused path on the packed bf16 row
+    flat = torch.from_numpy(packed[r].astype(np.int16)).view(torch.bfloat16).to(gpu)
+    c2, s2 = hpfp8.quantize_bucket(flat)
+    assert torch.equal(c2.view(torch.uint8), q[r].view(torch.uint8)) and torch.equal(s2, si[r])
+
+
+def test_bucket_argument_checks(gpu):
+    import hpfp8
+    b = hpfp8.Fp8GradBucket([256, 100], shard_size=2)
+    good = [torch.zeros(512, dtype=torch.bfloat16, device=gpu), torch.zeros(200, dtype=torch.bfloat16, device=gpu)]
+    with pytest.raises(ValueError):
+        b.pack(good[:1])
+    with pytest.raises(ValueError):
+        b.pack([good[0], torch.zeros(100, dtype=torch.bfloat16, device=gpu)])
+    with pytest.raises(TypeError):
+        b.pack([good[0], torch.zeros(200, dtype=torch.float32, device=gpu)])
+    q, si = b.pack(good)
+    assert q.shape == (2, 384) and si.shape == (2, 3) and not bool(q.view(torch.uint8).any())

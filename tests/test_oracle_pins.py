@@ -334,3 +334,28 @@ def test_grouped_equals_loop_of_dense_with_empty_experts():
             ye, _ = O.gemm_blockwise(xq[start:start + cnt], sxi[start:start + cnt], wq3[e], swi3[e])
             assert np.array_equal(y[start:start + cnt], ye)
         start += cnt
+
+
+def test_bucket_packing_against_an_element_loop():
+    """pack_bucket / unpack_bucket restate slicing assignments; pinned by the index arithmetic written
+    out element by element on a small case, by the zero padding, and by unpack(pack(x)) == x."""
+    rng = np.random.default_rng(9)
+    numels, S = [130, 128, 5, 300], 3
+    grads = [rng.integers(1, 65535, size=S * n).astype(np.uint16) for n in numels]
+    offsets, row = O.bucket_offsets(numels)
+    assert offsets == [0, 256, 384, 512] and row == 896
+    packed = O.pack_bucket(grads, numels, S)
+    want = np.zeros((S, row), dtype=np.uint16)
+    for e, n in enumerate(numels):
+        for s_ in range(S):
+            for i in range(n):
+                want[s_, offsets[e] + i] = grads[e][s_ * n + i]
+    assert np.array_equal(packed, want)
+    covered = np.zeros(row, dtype=bool)
+    for e, n in enumerate(numels):
+        covered[offsets[e]:offsets[e] + n] = True
+    assert not packed[:, ~covered].any()
+    for s_ in range(S):
+        pieces = O.unpack_bucket(packed[s_], numels)
+        for e, n in enumerate(numels):
+            assert np.array_equal(pieces[e], grads[e][s_ * n:(s_ + 1) * n])
