@@ -10,8 +10,14 @@ weight dims and along the contraction dim must be multiples of 128, so that no 1
 This module imports hyper_parallel and is only loaded by hyper_parallel's own dispatcher; the hpfp8
 package never imports it.
 """
+import os
+import sys
+
 from hyper_parallel.core.layout import Layout
 from hyper_parallel.core.shard.ops.parallel_ops import DistributedOp
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+from layout_rule import bias_divisor, infer_fp8_linear_map  # noqa: E402  (same directory, loaded by file path)
 
 
 class Fp8LinearDistributedOp(DistributedOp):
@@ -27,27 +33,20 @@ class Fp8LinearDistributedOp(DistributedOp):
             raise ValueError("fp8_linear inputs must have same mesh_shape")
         if bias_layout and bias_layout.mesh_shape != x_layout.mesh_shape:
             raise ValueError("fp8_linear bias and x must have same mesh_shape")
-        x_map, w_map = x_layout.alias_tensor_map, w_layout.alias_tensor_map
-        if x_map[-1] != w_map[-1]:
-            raise ValueError(f"Contracting dimensions must have same layout. Got {x_map[-1]} and {w_map[-1]}")
-        if bias_layout and bias_layout.alias_tensor_map[0] != w_map[0]:
-            raise ValueError("Output dimensions of weight and bias must have same sharding")
+        out_map, partial_axes = infer_fp8_linear_map(
+            x_layout.alias_tensor_map, w_layout.alias_tensor_map,
+            bias_layout.alias_tensor_map if bias_layout else None)
         out = Layout(mesh_shape=x_layout.mesh_shape, alias_name=x_layout.alias_name, rank_list=x_layout.rank_list)
-        out = out(*(x_map[:-1] + (w_map[0],)))
-        contract = x_map[-1]
-        if contract != "None":
-            for axis in (contract if isinstance(contract, tuple) else (contract,)):
-                out.set_partial_by_dev_axis(axis, "sum")
+        out = out(*out_map)
+        for axis in partial_axes:
+            out.set_partial_by_dev_axis(axis, "sum")
         return out
 
     def get_expand_impl(self, func, output_layout, layouts, extra_args):
-        x_map = layouts[0].alias_tensor_map
-        contract = x_map[-1]
-        if contract == "None" or not layouts[2]:
+        x_layout = layouts[0]
+        factor = bias_divisor(x_layout.alias_tensor_map, x_layout.mesh_shape, x_layout.alias_name)
+        if factor == 1 or not layouts[2]:
             return None
-        factor = 1
-        for axis in (contract if isinstance(contract, tuple) else (contract,)):
-            factor *= output_layout.mesh.get_device_num_along_axis(axis)
 
         def expand_impl(x, w, bias):
             return func(x, w, bias / factor)
