@@ -380,6 +380,27 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
 }
 
 // ---------------------------------------------------------------------------------------------
+// byte transpose of a code matrix: q[rows, cols] -> qt[cols, rows]
+// ---------------------------------------------------------------------------------------------
+// 128x128 blocks are symmetric, so the transposed codes of a weight (dgrad operand) can be made
+// from its codes alone, e.g. after the codes of all shards were gathered; no requantization.
+__global__ __launch_bounds__(256) void transpose_codes_kernel(const uint8_t* __restrict__ q, int rows, int cols,
+                                                              int64_t ld, uint8_t* __restrict__ qt, int64_t ld_t) {
+  const int rb = rows >> 7;
+  const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
+  __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
+  const int bc = blockIdx.x / rb, br = blockIdx.x % rb;
+  const uint8_t* src = q + (int64_t)br * 128 * ld + bc * 128 + cg * 8;
+  uint2 c[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + (int64_t)tile_row(rq, p) * ld));
+    c[p] = make_uint2(t.x, t.y);
+  }
+  store_tile_transposed(tile, c, cg, rq, qt + (int64_t)bc * 128 * ld_t + br * 128, ld_t);
+}
+
+// ---------------------------------------------------------------------------------------------
 // dequantize 1x128 groups back to bf16 (gradient bucket round trip)
 // ---------------------------------------------------------------------------------------------
 // out = bf16(decode(q) * scale_inv); if grad_scale != 1 the bf16 value is multiplied by it and
@@ -609,6 +630,25 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
   HPFP8_REQUIRE(m == 0 || k == 0 || q != nullptr, HPFP8_ERR_ARG, "quantize_1x128_and_128x1_t: null buffer");
   return quantize_128x1_t_impl("quantize_1x128_and_128x1_t", kmajor != 0, x, m, k, q_t, ld_t, scale_t, scale_inv_t,
                                stream, q, scale, scale_inv);
+}
+
+int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld, void* q_t, int64_t ld_t,
+                          hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "transpose_codes: negative shape");
+  HPFP8_REQUIRE(rows % kBlock == 0 && cols % kBlock == 0, HPFP8_ERR_SHAPE,
+                "transpose_codes: shape [%lld, %lld] is not a multiple of 128", (long long)rows, (long long)cols);
+  HPFP8_REQUIRE(rows < (1 << 30) && cols < (1 << 30), HPFP8_ERR_SHAPE, "transpose_codes: dimension too large");
+  const int64_t blocks = (rows / kBlock) * (cols / kBlock);
+  if (blocks == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "transpose_codes: tensor too large");
+  HPFP8_REQUIRE(q && q_t, HPFP8_ERR_ARG, "transpose_codes: null buffer");
+  HPFP8_REQUIRE(aligned16(q) && aligned16(q_t), HPFP8_ERR_ALIGN, "transpose_codes: buffers must be 16-byte aligned");
+  HPFP8_REQUIRE(ld >= cols && ld % 16 == 0 && ld_t >= rows && ld_t % 16 == 0, HPFP8_ERR_SHAPE,
+                "transpose_codes: ld=%lld / ld_t=%lld must be multiples of 16 and at least cols / rows", (long long)ld,
+                (long long)ld_t);
+  transpose_codes_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, (int)rows, (int)cols, ld,
+                                                                           (uint8_t*)q_t, ld_t);
+  return check_launch("transpose_codes");
 }
 
 int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,

@@ -15,7 +15,7 @@ Recipes
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import NamedTuple, Optional
 
 import torch
 from torch import nn
@@ -25,13 +25,30 @@ from . import ops
 RECIPES = ("blockwise", "per_tensor")
 
 
+class Fp8Weight(NamedTuple):
+    """A weight [N, K] already in its blockwise FP8 form: what `fp8_linear` would otherwise make from
+    the bf16 weight on every call."""
+    codes: torch.Tensor                 # e4m3 [N, K]
+    scale_inv: torch.Tensor             # fp32 [N/128, K/128]
+    codes_t: Optional[torch.Tensor]     # e4m3 [K, N] (dgrad operand) or None
+
+
+def quantize_weight(weight: torch.Tensor, with_transpose: bool = True) -> Fp8Weight:
+    """128x128-block quantization of a bf16 weight (and its transposed codes for dgrad)."""
+    if with_transpose:
+        wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
+        return Fp8Weight(wq, sw, wqt)
+    wq, sw = ops.quantize_128x128(weight)
+    return Fp8Weight(wq, sw, None)
+
+
 def _flatten(x: torch.Tensor):
     return x.reshape(-1, x.shape[-1])
 
 
 class _Fp8LinearBlockwise(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias):
+    def forward(ctx, x, weight, bias, wq=None, sw=None, wqt=None):
         x2 = _flatten(x)
         m = x2.shape[0]
         # With a weight gradient to come and a token count that allows it, x is read once: its 1x128
@@ -43,13 +60,16 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
         else:
             xq, sx = ops.quantize_1x128(x2, kmajor=True)
             xt = sxt = None
-        if x.requires_grad:
-            wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
-        else:
-            wq, sw = ops.quantize_128x128(weight)
-            wqt = None
+        if wq is None:                          # no prequantized form of the weight was passed in
+            if x.requires_grad:
+                wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
+            else:
+                wq, sw = ops.quantize_128x128(weight)
+        elif x.requires_grad and wqt is None:
+            wqt = ops.transpose_codes(wq)
         y = ops.gemm_blockwise(xq, sx, wq, sw, bias=bias)
-        ctx.save_for_backward(x2 if (weight.requires_grad and not fused) else None, xt, sxt, wqt, sw)
+        ctx.save_for_backward(x2 if (weight.requires_grad and not fused) else None, xt, sxt,
+                              wqt if x.requires_grad else None, sw)
         ctx.x_shape = x.shape
         ctx.has_bias = bias is not None
         ctx.need = (x.requires_grad, weight.requires_grad)
@@ -85,7 +105,7 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
             dw = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
-        return dx, dw, db
+        return dx, dw, db, None, None, None
 
 
 class _Fp8LinearPerTensor(torch.autograd.Function):
@@ -124,12 +144,16 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
 
 
 def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
-               recipe: str = "blockwise") -> torch.Tensor:
+               recipe: str = "blockwise", weight_fp8: Optional[Fp8Weight] = None) -> torch.Tensor:
     """y = input @ weight.T + bias computed through E4M3 operands with fp32 accumulation.
 
     input [..., in_features] bf16, weight [out_features, in_features] bf16, bias [out_features] bf16
     or None; returns bf16 [..., out_features].  in_features and out_features must be multiples of
     128 (ragged tails are rejected, not padded).
+
+    `weight_fp8` (blockwise recipe) is the weight's FP8 form made earlier -- by `quantize_weight`, or
+    from all-gathered FP8 shards (`hpfp8.fsdp`) -- and saves its quantization in this call; `weight`
+    is still the tensor that receives the gradient.
     """
     if recipe not in RECIPES:
         raise ValueError(f"recipe must be one of {RECIPES}, got {recipe!r}")
@@ -140,6 +164,13 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     for name, t in (("input", input), ("weight", weight), ("bias", bias)):
         if t is not None and t.dtype != torch.bfloat16:
             raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+    if weight_fp8 is not None:
+        if recipe != "blockwise":
+            raise ValueError("weight_fp8 is only used by the blockwise recipe")
+        if tuple(weight_fp8.codes.shape) != tuple(weight.shape):
+            raise ValueError("weight_fp8 does not have the weight's shape")
+        return _Fp8LinearBlockwise.apply(input, weight, bias, weight_fp8.codes, weight_fp8.scale_inv,
+                                         weight_fp8.codes_t)
     fn = _Fp8LinearBlockwise if recipe == "blockwise" else _Fp8LinearPerTensor
     return fn.apply(input, weight, bias)
 
@@ -148,8 +179,11 @@ class Fp8Linear(nn.Module):
     """Drop-in for torch.nn.Linear (bf16 parameters) whose matmuls run through fp8_linear."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, *, recipe: str = "blockwise",
-                 device=None, dtype=torch.bfloat16):
+                 cache_weight: bool = True, device=None, dtype=torch.bfloat16):
         super().__init__()
+        self.cache_weight = cache_weight
+        self._fp8: Optional[Fp8Weight] = None
+        self._fp8_key = None
         if recipe not in RECIPES:
             raise ValueError(f"recipe must be one of {RECIPES}, got {recipe!r}")
         if in_features % ops.BLOCK or out_features % ops.BLOCK:
@@ -167,7 +201,16 @@ class Fp8Linear(nn.Module):
                 self.bias.copy_(ref.bias)
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return fp8_linear(input, self.weight, self.bias, recipe=self.recipe)
+        if self.recipe != "blockwise" or not self.cache_weight:
+            return fp8_linear(input, self.weight, self.bias, recipe=self.recipe)
+        # The FP8 form of the weight is kept until the parameter is written again (optimizer step,
+        # load_state_dict, ...): micro-batches of one step and inference calls quantize it once.
+        key = (self.weight._version, self.weight.data_ptr())
+        if self._fp8_key != key:
+            with torch.no_grad():
+                self._fp8 = quantize_weight(self.weight.detach(), with_transpose=True)
+            self._fp8_key = key
+        return fp8_linear(input, self.weight, self.bias, recipe=self.recipe, weight_fp8=self._fp8)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

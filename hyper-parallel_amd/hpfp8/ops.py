@@ -167,6 +167,18 @@ def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: 
     return out
 
 
+def transpose_codes(q: torch.Tensor) -> torch.Tensor:
+    """codes[R, C] -> codes_t[C, R] (byte transpose; R, C multiples of 128).  With 128x128 scaling blocks
+    the transposed codes of a weight are its dgrad operand, scales reused with swapped strides."""
+    q = _check_codes_2d(q, "q")
+    r, c = q.shape
+    if r % BLOCK or c % BLOCK:
+        raise ValueError(f"shape {tuple(q.shape)} is not a multiple of {BLOCK} in both dims")
+    qt = _empty_codes_t(c, r, q.device)
+    _lib.call("hpfp8_transpose_codes", _ptr(q), r, c, _ld(q), _ptr(qt), _ld(qt), _stream())
+    return qt
+
+
 def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = False):
     """Transposed re-quantization for wgrad from the bf16 source.
 

@@ -110,6 +110,14 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
                                           float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
                                           float* scale_inv_t, hpfp8_stream_t stream);
 
+/* Byte transpose of a code matrix: q[rows, cols] (row stride ld) -> q_t[cols, rows] (row stride ld_t);
+ * rows, cols multiples of 128.  128x128 scaling blocks are symmetric, so this turns the codes of a
+ * weight into its dgrad operand without requantizing, e.g. after FP8 shards were all-gathered: the
+ * float8 all-gather extension point the reference leaves as a stub
+ * (hyper_parallel/platform/torch/fully_shard/param.py:299-310). */
+int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld, void* q_t, int64_t ld_t,
+                          hpfp8_stream_t stream);
+
 /* ---- dequantizers ----------------------------------------------------------------------------
  * The cast-back site hyper_parallel/core/hsdp/hsdp_grad_buffer.py:116-125: out = bf16(decode(q)
  * * scale_inv); when grad_scale != 1 the bf16 result is multiplied by it and rounded again. */

@@ -87,3 +87,51 @@ def test_grouped_linear_forward(gpu):
             ref = F.linear(x[start:start + c].float(), w[e].float())
             assert rel(y[start:start + c], ref) < 0.06
         start += c
+
+
+def test_prequantized_weight_and_module_cache(gpu):
+    """fp8_linear with a weight quantized beforehand gives bit-identical outputs and gradients to the
+    call that quantizes it itself; the module's cache is refreshed when the parameter is written."""
+    import hpfp8
+    x = U.randn_bf16((256, 384), 31).to(gpu).requires_grad_(True)
+    w = U.randn_bf16((256, 384), 32, 0.02).to(gpu).requires_grad_(True)
+    go = U.randn_bf16((256, 256), 33, 1e-3).to(gpu)
+    y0 = hpfp8.fp8_linear(x, w)
+    y0.backward(go)
+    gx0, gw0 = x.grad.clone(), w.grad.clone()
+    x.grad = w.grad = None
+    for with_t in (True, False):              # without transposed codes they are made from the codes
+        wf = hpfp8.quantize_weight(w.detach(), with_transpose=with_t)
+        y1 = hpfp8.fp8_linear(x, w, weight_fp8=wf)
+        y1.backward(go)
+        assert torch.equal(y1, y0) and torch.equal(x.grad, gx0) and torch.equal(w.grad, gw0)
+        x.grad = w.grad = None
+    mod = hpfp8.Fp8Linear(384, 256, bias=False, device=gpu)
+    with torch.no_grad():
+        mod.weight.copy_(w)
+    a = mod(x.detach())
+    key = mod._fp8_key
+    assert torch.equal(a, y0.detach()) and torch.equal(mod(x.detach()), a) and mod._fp8_key == key
+    with torch.no_grad():
+        mod.weight.mul_(2.0)                  # an in-place update, as an optimizer step is
+    b = mod(x.detach())
+    assert mod._fp8_key != key and torch.equal(b, hpfp8.fp8_linear(x.detach(), mod.weight.detach()))
+
+
+def test_fp8_all_gather_hooks_rebuild_the_full_weight(gpu):
+    """Per-shard quantization + concatenation (what an all-gather of the hook outputs produces) equals
+    quantizing the whole weight, transposed codes included; transpose_codes is a byte transpose."""
+    import hpfp8
+    w = U.randn_bf16((512, 384), 41, 0.02).to(gpu)
+    shards = w.chunk(4, dim=0)                # FSDP shards dim 0; 128 rows each
+    outs, metas = zip(*(hpfp8.fsdp.fsdp_pre_all_gather(s) for s in shards))
+    assert outs[0][0].dtype == torch.uint8 and outs[0][0].shape == (128, 384)
+    gathered = (torch.cat([o[0].reshape(-1) for o in outs]), torch.cat([o[1].reshape(-1) for o in outs]))
+    wf = hpfp8.fsdp.fsdp_post_all_gather(gathered, metas[0])
+    ref = hpfp8.quantize_weight(w, with_transpose=True)
+    assert torch.equal(wf.codes.view(torch.uint8), ref.codes.view(torch.uint8))
+    assert torch.equal(wf.scale_inv, ref.scale_inv)
+    assert torch.equal(wf.codes_t.view(torch.uint8), ref.codes_t.view(torch.uint8))
+    assert np.array_equal(U.codes(wf.codes_t), U.codes(wf.codes).T)
+    x = U.randn_bf16((128, 384), 42).to(gpu)
+    assert torch.equal(hpfp8.fp8_linear(x, w, weight_fp8=wf), hpfp8.fp8_linear(x, w))
