@@ -120,6 +120,12 @@ def other_configs(dev):
         "quantize_x": gb(x.numel() * 5, _time(lambda: hpfp8.quantize_per_tensor(x))),
         "gemm": tf(2.0 * 2048 * 1024 * 1024, _time(lambda: hpfp8.gemm_per_tensor(xq, sx, wq, sw))),
     }
+    # the step after cfg 2 in the MLP: SwiGLU of the gate/up output fused with the 1x128 quantization for the
+    # down projection (read 2 x 2 bytes, write 1 byte + scales per activation)
+    hgu = torch.randn((4096, 36864), generator=g, device=dev).to(torch.bfloat16)
+    res["cfg2_swiglu_quantize"] = gb(4096 * 18432 * 5 + 4096 * (18432 // 128) * 4,
+                                     _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True)))
+    del hgu
     # cfg 3: o_proj backward
     m, n, k = 4096, 7168, 16384
     x = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)

@@ -144,6 +144,93 @@ __global__ __launch_bounds__(256) void quant_1x128_kmajor_kernel(const uint16_t*
 }
 
 // ---------------------------------------------------------------------------------------------
+// SwiGLU fused with the 1x128 quantization of its result (input of the down projection)
+// ---------------------------------------------------------------------------------------------
+// exp(t), t clamped to [-86, 89], from IEEE fp32 operations only (no fused multiply-add, no hardware
+// exp), so that the CPU restatement reproduces it bit for bit: k = rint(t * log2 e),
+// r = t - k * ln2 (two constants), degree-6 Taylor polynomial in Horner form, times 2^(k-1), times 2
+// (two steps so that results up to the largest float come out finite and larger ones as +inf).
+__device__ __forceinline__ float exp_spec(float t) {
+  t = fminf(fmaxf(t, -86.0f), 89.0f);
+  const float k = __builtin_rintf(t * 1.44269504f);
+  float r = t - k * 0.693359375f;
+  r = r - k * -2.12194440e-4f;
+  float p = 1.0f / 720.0f;
+  p = p * r + 1.0f / 120.0f;
+  p = p * r + 1.0f / 24.0f;
+  p = p * r + 1.0f / 6.0f;
+  p = p * r + 0.5f;
+  p = p * r + 1.0f;
+  p = p * r + 1.0f;
+  return (p * __uint_as_float((uint32_t)((int)k + 126) << 23)) * 2.0f;
+}
+
+// bf16(bf16(silu(g)) * u) for two (g, u) pairs packed like their sources: the two roundings of the
+// unfused bf16 graph (silu, then the product).
+__device__ __forceinline__ uint32_t swiglu2(uint32_t gw, uint32_t uw) {
+  const float g0 = bf16lo(gw), g1 = bf16hi(gw);
+  const __bf16 s0 = (__bf16)(g0 / (1.0f + exp_spec(-g0)));
+  const __bf16 s1 = (__bf16)(g1 / (1.0f + exp_spec(-g1)));
+  const __bf16 a0 = (__bf16)((float)s0 * bf16lo(uw));
+  const __bf16 a1 = (__bf16)((float)s1 * bf16hi(uw));
+  return (uint32_t)__builtin_bit_cast(uint16_t, a0) | ((uint32_t)__builtin_bit_cast(uint16_t, a1) << 16);
+}
+
+// h[rows, 2 * inter] (row stride ld elements): gate = columns [0, inter), up = [inter, 2 inter).
+// q[rows, inter] = codes of act = silu(gate) * up in 1x128 groups; scales [rows, inter/128], or
+// [inter/128, rows] with KMAJOR.  Work split as in quant_1x128_kmajor_kernel.
+template <bool KMAJOR>
+__global__ __launch_bounds__(256) void swiglu_quant_1x128_kernel(const uint16_t* __restrict__ h, int64_t ld,
+                                                                 uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                                 float* __restrict__ scale_inv,
+                                                                 uint16_t* __restrict__ act, int rows, int inter) {
+  const int groups = inter >> 7;
+  const int gtiles = (groups + 3) >> 2;
+  const int g0 = (blockIdx.x % gtiles) * 4, row0 = (blockIdx.x / gtiles) * 16;
+  const int r = threadIdx.x >> 4, l16 = threadIdx.x & 15;
+  const int row = row0 + r;
+  __shared__ float s_s[4][16], s_si[4][16];
+  uint4 vg[4], vu[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const bool ok = row < rows && g0 + u < groups;
+    const uint16_t* src = h + (int64_t)row * ld + (g0 + u) * 128 + l16 * 8;
+    vg[u] = ok ? nt_load16(src) : make_uint4(0, 0, 0, 0);
+    vu[u] = ok ? nt_load16(src + inter) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const bool ok = row < rows && g0 + u < groups;
+    uint4 a;
+    a.x = swiglu2(vg[u].x, vu[u].x);
+    a.y = swiglu2(vg[u].y, vu[u].y);
+    a.z = swiglu2(vg[u].z, vu[u].z);
+    a.w = swiglu2(vg[u].w, vu[u].w);
+    const uint32_t m = row16_max_u32(mag8(a));
+    float s, si;
+    scales_from_amax(__uint_as_float(m << 16), s, si);
+    if (ok) {
+      const int64_t o = (int64_t)row * inter + (g0 + u) * 128 + l16 * 8;
+      nt_store8(q + o, cvt8<false>(a, s));
+      if (act) nt_store16(act + o, a);
+    }
+    if (l16 == 0) {
+      s_s[u][r] = s;
+      s_si[u][r] = si;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const int u = KMAJOR ? threadIdx.x >> 4 : threadIdx.x & 3, rr = KMAJOR ? threadIdx.x & 15 : threadIdx.x >> 2;
+    if (row0 + rr < rows && g0 + u < groups) {
+      const int64_t o = KMAJOR ? (int64_t)(g0 + u) * rows + row0 + rr : (int64_t)(row0 + rr) * groups + g0 + u;
+      if (scale) scale[o] = s_s[u][rr];
+      scale_inv[o] = s_si[u][rr];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // shared by the two tile kernels below: 128x128 tile, 256 threads
 // ---------------------------------------------------------------------------------------------
 // Thread t owns column group cg = t%16 (8 columns) and row quad rq = t/16: tile rows
@@ -630,6 +717,31 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
   HPFP8_REQUIRE(m == 0 || k == 0 || q != nullptr, HPFP8_ERR_ARG, "quantize_1x128_and_128x1_t: null buffer");
   return quantize_128x1_t_impl("quantize_1x128_and_128x1_t", kmajor != 0, x, m, k, q_t, ld_t, scale_t, scale_inv_t,
                                stream, q, scale, scale_inv);
+}
+
+int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
+                                     float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: negative shape");
+  HPFP8_REQUIRE(inter % kBlock == 0, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: width %lld is not a multiple of 128",
+                (long long)inter);
+  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 30), HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: dimension too large");
+  if (rows == 0 || inter == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(ld_h >= 2 * inter && ld_h % 8 == 0, HPFP8_ERR_SHAPE,
+                "swiglu_quantize_1x128: ld_h=%lld must be a multiple of 8 and at least twice the width", (long long)ld_h);
+  HPFP8_REQUIRE(h && q && scale_inv, HPFP8_ERR_ARG, "swiglu_quantize_1x128: null buffer");
+  HPFP8_REQUIRE(aligned16(h) && aligned16(q) && (!act || aligned16(act)), HPFP8_ERR_ALIGN,
+                "swiglu_quantize_1x128: buffers must be 16-byte aligned");
+  const int64_t groups = inter / kBlock;
+  const int64_t blocks = ((groups + 3) / 4) * ((rows + 15) / 16);
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: tensor too large");
+  hipStream_t s = (hipStream_t)stream;
+  if (kmajor)
+    swiglu_quant_1x128_kernel<true><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)h, ld_h, (uint8_t*)q, scale, scale_inv,
+                                                                     (uint16_t*)act, (int)rows, (int)inter);
+  else
+    swiglu_quant_1x128_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)h, ld_h, (uint8_t*)q, scale, scale_inv,
+                                                                      (uint16_t*)act, (int)rows, (int)inter);
+  return check_launch("swiglu_quantize_1x128");
 }
 
 int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld, void* q_t, int64_t ld_t,

@@ -26,13 +26,15 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
-def _check_bf16(x: torch.Tensor, name: str) -> torch.Tensor:
+def _check_bf16(x: torch.Tensor, name: str, contiguous: bool = True) -> torch.Tensor:
     if not isinstance(x, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor")
     if not x.is_cuda:
         raise ValueError(f"{name} must live on the GPU (got device {x.device}); this path has no CPU fallback")
     if x.dtype != torch.bfloat16:
         raise TypeError(f"{name} must be bfloat16, got {x.dtype}")
+    if not contiguous:
+        return x
     return x if x.is_contiguous() else x.contiguous()
 
 
@@ -165,6 +167,25 @@ def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: 
     if want_scale:
         out += (scale,)
     return out
+
+
+def swiglu_quantize_1x128(h: torch.Tensor, kmajor: bool = True, want_act: bool = False):
+    """h[M, 2I] bf16 (gate | up halves; any row stride that is a multiple of 8) ->
+    (codes[M, I], scale_inv[M, I/128]) of act = silu(gate) * up, plus act itself (bf16) if asked for."""
+    h = _check_bf16(h, "h", contiguous=False)
+    if h.dim() != 2 or h.shape[1] % (2 * BLOCK):
+        raise ValueError("h must be 2-D with a width that is a multiple of 256")
+    if h.stride(1) != 1 or h.stride(0) % 8 or h.data_ptr() % 16:
+        h = h.contiguous()
+    m, inter = h.shape[0], h.shape[1] // 2
+    q = torch.empty((m, inter), dtype=FP8, device=h.device)
+    s_inv = torch.empty((inter // BLOCK, m) if kmajor else (m, inter // BLOCK), dtype=torch.float32, device=h.device)
+    act = torch.empty((m, inter), dtype=torch.bfloat16, device=h.device) if want_act else None
+    _lib.call("hpfp8_swiglu_quantize_1x128_bf16", _ptr(h), m, inter, h.stride(0) if m > 1 else 2 * inter, int(kmajor),
+              _ptr(q), None, _ptr(s_inv), _ptr(act), _stream())
+    if kmajor:
+        s_inv = s_inv.t()
+    return (q, s_inv, act) if want_act else (q, s_inv)
 
 
 def transpose_codes(q: torch.Tensor) -> torch.Tensor:

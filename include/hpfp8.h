@@ -110,6 +110,18 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
                                           float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
                                           float* scale_inv_t, hpfp8_stream_t stream);
 
+/* SwiGLU fused with the 1x128 quantization of its result, the activations of the down projection
+ * (the step after the gate/up linear of a DeepSeekV3 MLP; in the reference this is eager
+ * F.silu(gate) * up between two aten::linear calls dispatched at
+ * hyper_parallel/core/shard/_op_dispatch.py:277-283).  h[rows, 2 * inter] bf16 with row stride ld_h
+ * elements: gate = columns [0, inter), up = columns [inter, 2 * inter).
+ *   act = bf16( bf16(silu(gate)) * up ),  silu(g) = g / (1 + exp(-g)) in fp32 with the exponential
+ *   defined operation by operation in csrc/quantize.hip (exp_spec) and restated in the oracle,
+ * quantized like hpfp8_quantize_1x128[_kmajor]_bf16: q[rows, inter], scales [rows, inter/128] or
+ * (kmajor != 0) [inter/128, rows].  act (bf16 [rows, inter]) is also written when not NULL. */
+int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
+                                     float* scale, float* scale_inv, void* act, hpfp8_stream_t stream);
+
 /* Byte transpose of a code matrix: q[rows, cols] (row stride ld) -> q_t[cols, rows] (row stride ld_t);
  * rows, cols multiples of 128.  128x128 scaling blocks are symmetric, so this turns the codes of a
  * weight into its dgrad operand without requantizing, e.g. after FP8 shards were all-gathered: the

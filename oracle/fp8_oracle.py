@@ -254,6 +254,43 @@ def dequantize_bucket(codes: np.ndarray, scale_inv: np.ndarray, grad_scale: floa
     return bits
 
 
+def exp_spec(t: np.ndarray) -> np.ndarray:
+    """The exponential the SwiGLU kernel defines, operation by operation in IEEE fp32 (no fused
+    multiply-add): clamp to [-86, 89], k = rint(t * log2 e), r = t - k * ln2 in two steps, degree-6
+    Taylor polynomial in Horner form, times 2^(k-1), times 2 (+inf beyond the largest float).  Not taken
+    from the reference (which has no such kernel); pinned against numpy's exp in the tests."""
+    f = np.float32
+    t = np.minimum(np.maximum(np.asarray(t, f), f(-86.0)), f(89.0))
+    k = np.rint(t * f(1.44269504))
+    r = t - k * f(0.693359375)
+    r = r - k * f(-2.12194440e-4)
+    p = np.full_like(r, f(1.0) / f(720.0))
+    for c in (f(1.0) / f(120.0), f(1.0) / f(24.0), f(1.0) / f(6.0), f(0.5), f(1.0), f(1.0)):
+        p = p * r + c
+    half = ((k.astype(np.int32) + 126).astype(np.uint32) << np.uint32(23)).view(f)
+    with np.errstate(over="ignore"):
+        return ((p * half).astype(f) * f(2.0)).astype(f)
+
+
+def swiglu(h_bits: np.ndarray) -> np.ndarray:
+    """bf16 bits of act = bf16(bf16(silu(gate)) * up) for h = [gate | up] (bf16 bits, [M, 2I]): the
+    eager bf16 graph F.silu(gate) * up with its two roundings, silu(g) = g / (1 + exp(-g)) in fp32."""
+    h_bits = np.asarray(h_bits, dtype=np.uint16)
+    inter = h_bits.shape[-1] // 2
+    g = bf16_bits_to_f32(h_bits[..., :inter])
+    u = bf16_bits_to_f32(h_bits[..., inter:])
+    s = (g / (np.float32(1.0) + exp_spec(-g))).astype(np.float32)
+    s = bf16_bits_to_f32(f32_to_bf16_bits(s))
+    return f32_to_bf16_bits((s * u).astype(np.float32))
+
+
+def swiglu_quantize_1x128(h_bits: np.ndarray):
+    """(codes, scale, scale_inv, act bits) of the SwiGLU result quantized in 1x128 groups."""
+    act = swiglu(h_bits)
+    codes, scale, scale_inv = quantize_1x128(act)
+    return codes, scale, scale_inv, act
+
+
 def bucket_offsets(numels):
     """Start of every parameter in a bucket row and the row length: the running index of
     hyper_parallel/core/hsdp/hsdp_grad_buffer.py:72-80, with every start rounded up to a multiple

@@ -359,3 +359,27 @@ def test_bucket_packing_against_an_element_loop():
         pieces = O.unpack_bucket(packed[s_], numels)
         for e, n in enumerate(numels):
             assert np.array_equal(pieces[e], grads[e][s_ * n:(s_ + 1) * n])
+
+
+def test_swiglu_restatement_against_numpy_and_torch():
+    """exp_spec within a few fp32 ulp of numpy's exp over its whole clamped range; swiglu equal to
+    torch's eager bf16 graph F.silu(gate) * up except where a last-place difference of the fp32
+    sigmoid crosses a bf16 rounding boundary (then one bf16 ulp)."""
+    import torch
+    import torch.nn.functional as F
+    t = np.concatenate([np.linspace(-86, 88.7, 200001), np.random.default_rng(0).normal(0, 3, 100000)]).astype(np.float32)
+    got = O.exp_spec(t).astype(np.float64)
+    want = np.exp(t.astype(np.float64))
+    assert np.max(np.abs(got - want) / want) < 4e-7
+    assert O.exp_spec(np.float32([0.0]))[0] == 1.0 and O.exp_spec(np.float32([-1000.0]))[0] == O.exp_spec(np.float32([-86.0]))[0] \
+        and np.isinf(O.exp_spec(np.float32([89.0, 1000.0]))).all()
+    g = torch.randn(64, 512, generator=torch.Generator().manual_seed(1)) * 3
+    g[0, :8] = torch.tensor([0.0, -0.0, 50.0, -50.0, 1e-3, -1e-3, 200.0, -200.0])
+    u = torch.randn(64, 512, generator=torch.Generator().manual_seed(2))
+    h = torch.cat([g, u], dim=1).to(torch.bfloat16)
+    ref = (F.silu(h[:, :512]) * h[:, 512:])
+    mine = O.swiglu(h.view(torch.int16).numpy().view(np.uint16))
+    ref_bits = ref.view(torch.int16).numpy().view(np.uint16)
+    diff = np.abs(mine.astype(np.int32) - ref_bits.astype(np.int32))
+    same_sign_zero = (mine & 0x7FFF) + (ref_bits & 0x7FFF) == 0
+    assert ((diff <= 1) | same_sign_zero).all() and (diff != 0).mean() < 2e-3
