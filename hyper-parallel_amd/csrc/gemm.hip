@@ -125,6 +125,13 @@ __device__ __forceinline__ TileInfo pick_tile(int q, TileInfo t0, TileInfo t1, T
   return r;
 }
 
+// End row of an expert as the kernel uses it: offsets that decrease or run past the row count (a
+// malformed table) are clamped, so that every address derived from them stays inside a.
+__device__ __forceinline__ int expert_end(int off, int prev, int total_rows) {
+  const int lo = off > prev ? off : prev;
+  return lo < total_rows ? lo : total_rows;
+}
+
 template <int MODE, bool GROUPED, bool OUT_F32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
   constexpr int kBStages = b_stages(MODE);
@@ -149,7 +156,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     // tiles are numbered expert by expert; an expert with no rows has none
     int prev = 0, mt = 0;
     for (int e = 0; e < p.experts; ++e) {
-      const int end = p.offs[e];
+      const int end = expert_end(p.offs[e], prev, p.M);
       mt += (end - prev + BM - 1) / BM;
       prev = end;
     }
@@ -178,7 +185,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       if (GROUPED) {
         int end = 0, cnt = 0;
         while (g_e < p.experts) {
-          end = p.offs[g_e];
+          end = expert_end(p.offs[g_e], g_prev, p.M);
           cnt = (end - g_prev + BM - 1) / BM;
           if (t < g_first + cnt * tiles_n) break;
           g_first += cnt * tiles_n;

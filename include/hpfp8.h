@@ -194,7 +194,8 @@ int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const
 /* MoE grouped form (one rank's local experts; no counterpart in the reference, whose expert
  * parallelism is unimplemented): rows of a[total_m, K] (row stride lda) are sorted by expert; offs[e] (int32,
  * device) is the inclusive prefix sum of per-expert row counts, a count may be 0, rows past
- * offs[experts-1] are left untouched; b[experts, N, K]; sb[experts, N/128, K/128];
+ * offs[experts-1] are left untouched (an offset below its predecessor or above total_m is read as clamped
+ * to that range); b[experts, N, K]; sb[experts, N/128, K/128];
  * sa(m, kb) = sa[m * sa_stride_m + kb * sa_stride_k]; c[total_m, N] bf16 or fp32. */
 int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                                  const void* b, const float* sb, const int32_t* offs, int experts,

@@ -271,3 +271,27 @@ def test_grouped_leaves_rows_past_the_last_offset_alone(gpu):
               wq.data_ptr(), swi.data_ptr(), offs.data_ptr(), 2, 300, N, K, out.data_ptr(), N, _lib.OUT_F32,
               ops._stream())
     assert bool((out[260:] == 7.0).all()) and not bool((out[:260] == 7.0).any())
+
+
+def test_grouped_clamps_a_malformed_offset_table(gpu):
+    """Offsets that decrease or run past the row count are read as clamped (an expert's end is at least
+    the previous end and at most total_m): the result is that of the clamped table and no row outside
+    a or c is touched."""
+    import hpfp8
+    from hpfp8 import _lib, ops
+    K, N, total = 256, 256, 700
+    x = U.randn_bf16((total, K), 50).to(gpu)
+    w = U.randn_bf16((4 * N, K), 51, 0.01).to(gpu)
+    xq, sxi = hpfp8.quantize_1x128(x)
+    wq, swi = hpfp8.quantize_128x128(w)
+    bad = torch.tensor([300, 200, 650, 900], dtype=torch.int32, device=gpu)      # clamps to 300, 300, 650, 700
+    good = torch.tensor([300, 300, 650, 700], dtype=torch.int32, device=gpu)
+    outs = []
+    for offs in (bad, good):
+        out = torch.full((total + 8, N), 7.0, dtype=torch.float32, device=gpu)
+        _lib.call("hpfp8_gemm_grouped_blockwise", xq.data_ptr(), K, sxi.data_ptr(), sxi.stride(0), sxi.stride(1),
+                  wq.data_ptr(), swi.data_ptr(), offs.data_ptr(), 4, total, N, K, out.data_ptr(), N, _lib.OUT_F32,
+                  ops._stream())
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1]) and bool((outs[0][total:] == 7.0).all())
+    assert not bool((outs[0][:total] == 7.0).any())
