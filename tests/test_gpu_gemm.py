@@ -295,3 +295,44 @@ def test_grouped_clamps_a_malformed_offset_table(gpu):
         outs.append(out)
     assert torch.equal(outs[0], outs[1]) and bool((outs[0][total:] == 7.0).all())
     assert not bool((outs[0][:total] == 7.0).any())
+
+
+def test_cfg4_moe_grouped_full_size(gpu):
+    """The grouped configuration at its real size (32 experts, 16384 tokens routed top-8 with Zipf
+    popularity = 131072 rows, fused gate/up [4096, 7168] per expert): every expert's rows equal the
+    dense kernel on that expert bit for bit (the grouped form only changes which tile goes where),
+    and 256-row samples of three experts agree with the dequantize-then-float64 product."""
+    import hpfp8
+    experts, total, N, K = 32, 131072, 4096, 7168
+    counts = _zipf_counts(total, experts, 7)
+    assert int(counts.sum()) == total and int((counts == 0).sum()) >= 2
+    offs = counts.cumsum(0).to(torch.int32).to(gpu)
+    g = torch.Generator(device=gpu).manual_seed(3)
+    xq = torch.empty((total, K), dtype=torch.float8_e4m3fn, device=gpu)
+    sxi = torch.empty((K // 128, total), dtype=torch.float32, device=gpu).t()
+    for r0 in range(0, total, 16384):
+        xc = torch.randn((16384, K), generator=g, device=gpu).to(torch.bfloat16)
+        q_, s_ = hpfp8.quantize_1x128(xc, kmajor=True)
+        xq[r0:r0 + 16384] = q_
+        sxi[r0:r0 + 16384] = s_
+    wq = torch.empty((experts, N, K), dtype=torch.float8_e4m3fn, device=gpu)
+    swi = torch.empty((experts, N // 128, K // 128), dtype=torch.float32, device=gpu)
+    for e in range(experts):
+        wc = (torch.randn((N, K), generator=g, device=gpu) * 0.006).to(torch.bfloat16)
+        wq[e], swi[e] = hpfp8.quantize_128x128(wc)
+    del xc, wc
+    y = hpfp8.gemm_grouped_blockwise(xq, sxi, wq, swi, offs)
+    assert y.shape == (total, N) and y.dtype == torch.bfloat16
+    start, checked = 0, 0
+    for e in range(experts):
+        cnt = int(counts[e])
+        if cnt:
+            dense = hpfp8.gemm_blockwise(xq[start:start + cnt], sxi[start:start + cnt], wq[e], swi[e])
+            assert torch.equal(y[start:start + cnt], dense), f"expert {e}"
+            if checked < 3 and cnt >= 256:
+                r0 = start + (cnt - 256) // 2
+                ref = ref_f64_torch(xq[r0:r0 + 256], sxi[r0:r0 + 256], wq[e], swi[e].repeat_interleave(128, dim=0), gpu)
+                assert rel(U.f32(y[r0:r0 + 256]), ref.cpu().numpy()) < TOL_BF16
+                checked += 1
+        start += cnt
+    assert checked == 3
