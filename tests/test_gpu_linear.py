@@ -135,3 +135,30 @@ def test_fp8_all_gather_hooks_rebuild_the_full_weight(gpu):
     assert np.array_equal(U.codes(wf.codes_t), U.codes(wf.codes).T)
     x = U.randn_bf16((128, 384), 42).to(gpu)
     assert torch.equal(hpfp8.fp8_linear(x, w, weight_fp8=wf), hpfp8.fp8_linear(x, w))
+
+
+def test_fp8_checkpoint_round_trip(gpu, tmp_path):
+    """Weights written as `weight` (float8_e4m3fn) + `weight_scale_inv` (the DeepSeek-V3 convention)
+    and read back: the loaded module computes with the stored codes, so its output equals the
+    saving module's bit for bit; the stored pair dequantizes to within the block's step."""
+    import hpfp8
+    from safetensors.torch import load_file
+    torch.manual_seed(1)
+    model = torch.nn.Sequential(hpfp8.Fp8Linear(256, 384, bias=True, device=gpu),
+                                torch.nn.GELU(),
+                                hpfp8.Fp8Linear(384, 128, bias=False, device=gpu))
+    x = U.randn_bf16((128, 256), 61).to(gpu)
+    y = model(x)
+    path = str(tmp_path / "model.safetensors")
+    hpfp8.checkpoint.save_fp8_checkpoint(hpfp8.checkpoint.fp8_state_dict(model), path)
+    raw = load_file(path)
+    assert raw["0.weight"].dtype == torch.float8_e4m3fn and raw["0.weight_scale_inv"].shape == (3, 2)
+    assert raw["0.bias"].dtype == torch.bfloat16 and "2.weight_scale_inv" in raw
+    clone = torch.nn.Sequential(hpfp8.Fp8Linear(256, 384, bias=True, device=gpu),
+                                torch.nn.GELU(),
+                                hpfp8.Fp8Linear(384, 128, bias=False, device=gpu))
+    hpfp8.checkpoint.load_into(clone, hpfp8.checkpoint.load_fp8_checkpoint(path, device=gpu))
+    assert torch.equal(clone(x), y)
+    w, wd = model[0].weight.detach().float(), clone[0].weight.detach().float()
+    amax = w.view(3, 128, 2, 128).abs().amax(dim=(1, 3), keepdim=True)
+    assert bool(((w - wd).view(3, 128, 2, 128).abs() <= amax / 28 + amax / 256).all())
