@@ -25,11 +25,14 @@ __global__ __launch_bounds__(256) void amax_bf16_kernel(const uint16_t* __restri
   uint32_t m = 0;
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * 256;
-  for (; i + 3 * stride < nvec; i += 4 * stride) {
-    uint4 a = xv[i], b = xv[i + stride], c = xv[i + 2 * stride], d = xv[i + 3 * stride];
-    m = umax(m, umax(umax(mag8(a), mag8(b)), umax(mag8(c), mag8(d))));
+  for (; i + 7 * stride < nvec; i += 8 * stride) {     // eight 128-bit loads in flight per thread
+    uint4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = nt_load16(&xv[i + u * stride]);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) m = umax(m, mag8(v[u]));
   }
-  for (; i < nvec; i += stride) m = umax(m, mag8(xv[i]));
+  for (; i < nvec; i += stride) m = umax(m, mag8(nt_load16(&xv[i])));
   if (blockIdx.x == 0 && threadIdx.x < (n & 7)) m = umax(m, x[(nvec << 3) + threadIdx.x] & 0x7FFFu);
   m = row16_max_u32(m);
   __shared__ uint32_t part[16];
@@ -37,7 +40,11 @@ __global__ __launch_bounds__(256) void amax_bf16_kernel(const uint16_t* __restri
   __syncthreads();
   if (threadIdx.x < 16) {
     m = row16_max_u32(part[threadIdx.x]);
-    if (threadIdx.x == 0) atomicMax(amax_bits, m << 16);
+    // The result only grows, so a block whose maximum does not exceed a (possibly stale) reading of
+    // it has nothing to add; this keeps most of the same-address atomics out of the L2.
+    if (threadIdx.x == 0 &&
+        (m << 16) > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+      atomicMax(amax_bits, m << 16);
   }
 }
 
@@ -57,8 +64,15 @@ __global__ __launch_bounds__(256) void cast_per_tensor_kernel(const uint16_t* __
   uint2* qv = reinterpret_cast<uint2*>(q);
   const int64_t nvec = n >> 3;
   const int64_t stride = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += stride)
-    qv[i] = cvt8<true>(xv[i], scale);
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {     // four 128-bit loads in flight per thread
+    uint4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = nt_load16(&xv[i + u * stride]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) nt_store8(&qv[i + u * stride], cvt8<true>(v[u], scale));
+  }
+  for (; i < nvec; i += stride) nt_store8(&qv[i], cvt8<true>(nt_load16(&xv[i]), scale));
   if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {
     int64_t j = (nvec << 3) + threadIdx.x;
     uint32_t r = cvt2<false, true>(0u, x[j], scale);
@@ -577,10 +591,10 @@ int hpfp8_amax_bf16(const void* x, int64_t n, float* amax_out, hpfp8_stream_t st
   fill_u32_kernel<<<1, 64, 0, s>>>(reinterpret_cast<uint32_t*>(amax_out), 0u, 1);
   if (n > 0) {
     int64_t nvec = n >> 3;
-    int blocks = (int)((nvec + 256 * 8 - 1) / (256 * 8));
+    int64_t blocks = (nvec + 256 * 8 - 1) / (256 * 8);
     if (blocks < 1) blocks = 1;
-    if (blocks > 4096) blocks = 4096;
-    amax_bf16_kernel<<<blocks, 256, 0, s>>>((const uint16_t*)x, n, reinterpret_cast<uint32_t*>(amax_out));
+    if (blocks > 2048) blocks = 2048;    // 8 resident workgroups per CU on 256 CUs; the rest is the grid-stride loop
+    amax_bf16_kernel<<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)x, n, reinterpret_cast<uint32_t*>(amax_out));
   }
   return check_launch("amax");
 }
