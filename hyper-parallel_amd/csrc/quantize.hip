@@ -548,6 +548,28 @@ __global__ __launch_bounds__(256) void dequant_1x128_kernel(const uint2* __restr
   }
 }
 
+// main[i] += (decode(q[i]) * scale_inv) * grad_scale in fp32: a reduced FP8 gradient added onto an
+// fp32 main gradient in one pass (the `main_grad += reduced_grad` of
+// hyper_parallel/platform/torch/fully_shard/param.py:160-167 for an FP8 reduce dtype).
+__global__ __launch_bounds__(256) void dequant_1x128_accumulate_kernel(const uint2* __restrict__ q,
+                                                                       const float* __restrict__ scale_inv,
+                                                                       float4* __restrict__ main_grad, int64_t nvec,
+                                                                       float grad_scale) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const u32x2 c = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(&q[i]));
+  const float si = scale_inv[i >> 4];
+  float4 m0 = main_grad[2 * i], m1 = main_grad[2 * i + 1];
+  const v2f a = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.x, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.x, true);
+  const v2f d = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.y, false), e = __builtin_amdgcn_cvt_pk_f32_fp8((int)c.y, true);
+  m0.x += (a.x * si) * grad_scale; m0.y += (a.y * si) * grad_scale;
+  m0.z += (b.x * si) * grad_scale; m0.w += (b.y * si) * grad_scale;
+  m1.x += (d.x * si) * grad_scale; m1.y += (d.y * si) * grad_scale;
+  m1.z += (e.x * si) * grad_scale; m1.w += (e.y * si) * grad_scale;
+  main_grad[2 * i] = m0;
+  main_grad[2 * i + 1] = m1;
+}
+
 // codes with one scale per 128x128 block (weights) -> bf16
 __global__ __launch_bounds__(256) void dequant_128x128_kernel(const uint8_t* __restrict__ q,
                                                               const float* __restrict__ scale_inv,
@@ -792,6 +814,23 @@ int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t r
   dequant_1x128_kernel<UNROLL><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
       (const uint2*)q, scale_inv, (uint4*)out, nvec, grad_scale, grad_scale != 1.0f ? 1 : 0);
   return check_launch("dequantize_1x128");
+}
+
+int hpfp8_dequantize_1x128_accumulate_f32(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
+                                          float* main_grad, float grad_scale, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "dequantize_1x128_accumulate: negative shape");
+  HPFP8_REQUIRE(cols % kBlock == 0, HPFP8_ERR_SHAPE,
+                "dequantize_1x128_accumulate: last dim %lld is not a multiple of 128", (long long)cols);
+  const int64_t nvec = rows * cols / 8;
+  if (nvec == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(q && scale_inv && main_grad, HPFP8_ERR_ARG, "dequantize_1x128_accumulate: null buffer");
+  HPFP8_REQUIRE(aligned16(q) && aligned16(main_grad), HPFP8_ERR_ALIGN,
+                "dequantize_1x128_accumulate: buffers must be 16-byte aligned");
+  const int64_t blocks = (nvec + 255) / 256;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "dequantize_1x128_accumulate: tensor too large");
+  dequant_1x128_accumulate_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+      (const uint2*)q, scale_inv, (float4*)main_grad, nvec, grad_scale);
+  return check_launch("dequantize_1x128_accumulate");
 }
 
 int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,

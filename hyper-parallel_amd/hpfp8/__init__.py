@@ -8,7 +8,7 @@ _lib.load()
 
 from .ops import (amax, quantize_per_tensor, quantize_1x128, quantize_128x128, quantize_128x1_t,  # noqa: E402
                   quantize_1x128_and_128x1_t, transpose_codes, swiglu_quantize_1x128,
-                  dequantize_1x128, dequantize_128x128, gemm_blockwise, gemm_per_tensor,
+                  dequantize_1x128, dequantize_1x128_accumulate, dequantize_128x128, gemm_blockwise, gemm_per_tensor,
                   gemm_grouped_blockwise)
 from .linear import fp8_linear, Fp8Linear, fp8_grouped_linear, Fp8Weight, quantize_weight  # noqa: E402
 from . import fsdp, checkpoint  # noqa: E402
@@ -17,7 +17,7 @@ from .bucket import quantize_bucket, dequantize_bucket, Fp8GradBucket  # noqa: E
 __all__ = [
     "amax", "quantize_per_tensor", "quantize_1x128", "quantize_128x128", "quantize_128x1_t",
     "quantize_1x128_and_128x1_t", "transpose_codes", "swiglu_quantize_1x128", "Fp8Weight", "quantize_weight", "fsdp", "checkpoint",
-    "dequantize_1x128", "dequantize_128x128", "gemm_blockwise", "gemm_per_tensor",
+    "dequantize_1x128", "dequantize_1x128_accumulate", "dequantize_128x128", "gemm_blockwise", "gemm_per_tensor",
     "gemm_grouped_blockwise", "fp8_linear", "Fp8Linear", "fp8_grouped_linear",
     "quantize_bucket", "dequantize_bucket", "Fp8GradBucket",
 ]

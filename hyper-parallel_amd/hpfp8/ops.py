@@ -10,6 +10,8 @@ from __future__ import annotations
 
 from typing import Optional, Tuple
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -261,6 +263,25 @@ def dequantize_1x128(q: torch.Tensor, scale_inv: torch.Tensor, grad_scale: float
     _lib.call("hpfp8_dequantize_1x128_bf16", _ptr(q), _ptr(scale_inv), rows, cols, _ptr(out), float(grad_scale),
               _stream())
     return out
+
+
+def dequantize_1x128_accumulate(q: torch.Tensor, scale_inv: torch.Tensor, main_grad: torch.Tensor,
+                                grad_scale: float = 1.0) -> torch.Tensor:
+    """main_grad (fp32, same shape as q, contiguous) += decode(q) * scale_inv * grad_scale, in place."""
+    q = _check_fp8(q, "q")
+    scale_inv = _check_f32(scale_inv, "scale_inv")
+    cols = q.shape[-1]
+    if cols % BLOCK:
+        raise ValueError(f"last dim {cols} is not a multiple of {BLOCK}")
+    rows = q.numel() // cols if cols else 0
+    if scale_inv.numel() != rows * (cols // BLOCK) or not scale_inv.is_contiguous() or not q.is_contiguous():
+        raise ValueError("q must be contiguous and scale_inv contiguous with one entry per 128 codes")
+    if main_grad.dtype != torch.float32 or not main_grad.is_cuda or not main_grad.is_contiguous() or \
+            main_grad.numel() != q.numel():
+        raise ValueError("main_grad must be a contiguous float32 GPU tensor with as many elements as q")
+    _lib.call("hpfp8_dequantize_1x128_accumulate_f32", _ptr(q), _ptr(scale_inv), rows, cols, _ptr(main_grad),
+              ctypes.c_float(grad_scale), _stream())
+    return main_grad
 
 
 def dequantize_128x128(q: torch.Tensor, scale_inv: torch.Tensor) -> torch.Tensor:

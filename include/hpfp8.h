@@ -137,6 +137,12 @@ int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t r
                                 void* out, float grad_scale, hpfp8_stream_t stream);
 int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
                                   void* out, hpfp8_stream_t stream);
+/* main_grad[i] += (decode(q[i]) * scale_inv) * grad_scale, all in fp32 (two multiplications, then the
+ * addition): a reduced FP8 gradient added onto the fp32 main gradient in one pass, the
+ * `main_grad += reduced_grad` of hyper_parallel/platform/torch/fully_shard/param.py:160-167 under
+ * MixedPrecisionPolicy.apply_grad_on_fp32_main_grad (platform/torch/fully_shard/utils.py:24). */
+int hpfp8_dequantize_1x128_accumulate_f32(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
+                                          float* main_grad, float grad_scale, hpfp8_stream_t stream);
 
 /* ---- gradient bucket: pack + quantize, dequantize + unpack -------------------------------------
  * The FP8 form of HSDPGradBuffer._copy_grad_to_unsharded_buffer and ._set_grad_data

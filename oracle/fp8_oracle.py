@@ -291,6 +291,18 @@ def swiglu_quantize_1x128(h_bits: np.ndarray):
     return codes, scale, scale_inv, act
 
 
+def dequantize_1x128_accumulate(codes: np.ndarray, scale_inv: np.ndarray, main_grad: np.ndarray,
+                                grad_scale: float = 1.0) -> np.ndarray:
+    """main_grad + (decode(codes) * scale_inv) * grad_scale in fp32, operation by operation: the
+    `main_grad += reduced_grad` of hyper_parallel/platform/torch/fully_shard/param.py:160-167 with the
+    reduced gradient held as E4M3 codes and 1x128 scales."""
+    f = np.float32
+    v = e4m3_decode(codes).astype(f).reshape(-1, BLOCK)
+    v = (v * np.asarray(scale_inv, f).reshape(-1, 1)).astype(f)
+    v = (v * f(grad_scale)).astype(f)
+    return (np.asarray(main_grad, f).reshape(-1, BLOCK) + v).astype(f).reshape(np.shape(main_grad))
+
+
 def bucket_offsets(numels):
     """Start of every parameter in a bucket row and the row length: the running index of
     hyper_parallel/core/hsdp/hsdp_grad_buffer.py:72-80, with every start rounded up to a multiple

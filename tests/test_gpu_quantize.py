@@ -266,3 +266,17 @@ def test_swiglu_fused_with_quantize(gpu, shape, kmajor):
     wide[:, :w2] = hg
     q2, si2 = hpfp8.swiglu_quantize_1x128(wide[:, :w2], kmajor=kmajor)
     assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(si2, si)
+
+
+def test_dequantize_accumulate_into_fp32_main_grad(gpu):
+    import hpfp8
+    g = U.randn_bf16((300, 640), 71, 1e-3, 0.002, 100.0)
+    q, si = hpfp8.quantize_1x128(g.to(gpu))
+    main = torch.randn((300, 640), generator=torch.Generator().manual_seed(3)) * 1e-3
+    got = hpfp8.dequantize_1x128_accumulate(q, si, main.to(gpu).clone(), grad_scale=0.25)
+    want = O.dequantize_1x128_accumulate(U.codes(q), U.f32(si), main.numpy(), 0.25)
+    assert np.array_equal(U.f32_bits(U.f32(got)), U.f32_bits(want))
+    # twice the same gradient with grad_scale 1 == adding the bf16-free dequantized values twice
+    again = hpfp8.dequantize_1x128_accumulate(q, si, got, grad_scale=1.0)
+    want2 = O.dequantize_1x128_accumulate(U.codes(q), U.f32(si), want, 1.0)
+    assert np.array_equal(U.f32_bits(U.f32(again)), U.f32_bits(want2))
