@@ -218,7 +218,7 @@ def main():
 
     import torch
     import hpfp8
-    from hpfp8 import _lib, ops
+    from hpfp8 import _lib
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     lib = _lib.load()
