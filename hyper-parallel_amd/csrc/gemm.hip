@@ -229,7 +229,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
                                              (int)((int64_t)(ti.row_end - ti.row0) * p.lda), 0x00020000);
   };
   auto rsrc_b_of = [&](const TileInfo& ti) {
-    const int rows = N - ti.n0 > 0 ? N - ti.n0 : 0;
+    int rows = N - ti.n0 > 0 ? N - ti.n0 : 0;
+    if (rows > BN) rows = BN;
     const uint8_t* base = p.b + (GROUPED ? (int64_t)ti.expert * N * p.ldb : 0) + (int64_t)(rows ? ti.n0 : 0) * p.ldb;
     return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)((int64_t)rows * p.ldb), 0x00020000);
   };
@@ -682,9 +683,11 @@ static int check_common(const char* what, const void* a, int64_t lda, const void
   HPFP8_REQUIRE(a && b && sa && sb && c, HPFP8_ERR_ARG, "%s: null buffer", what);
   HPFP8_REQUIRE(aligned16(a) && aligned16(b) && aligned16(c) && (!bias || aligned16(bias)), HPFP8_ERR_ALIGN,
                 "%s: buffers must be 16-byte aligned", what);
-  // 32-bit byte offsets inside the tile loader, including rows read past the end of a tile
-  HPFP8_REQUIRE((M + BM) * lda < (int64_t)0x7FFFFFFF && (N + BN) * ldb < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
-                "%s: an operand exceeds 2 GiB", what);
+  // 32-bit byte offsets inside one tile's buffer resource (256 rows); the operands themselves may be
+  // of any size
+  HPFP8_REQUIRE(BM * lda < (int64_t)0x7FFFFFFF && BN * ldb < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
+                "%s: a row stride of 8 MiB or more is not supported", what);
+  HPFP8_REQUIRE(M < (int64_t)0x7FFFFF00 && N < (int64_t)0x7FFFFF00, HPFP8_ERR_SHAPE, "%s: M or N too large", what);
   return 1;
 }
 

@@ -336,3 +336,24 @@ def test_cfg4_moe_grouped_full_size(gpu):
                 checked += 1
         start += cnt
     assert checked == 3
+
+
+def test_activation_matrix_larger_than_2_gib(gpu):
+    """Tiles are addressed relative to their own first row, so the code matrix as a whole may exceed
+    what a 32-bit byte offset spans: rows beyond byte 2^31 give the same bits as the same rows
+    passed on their own."""
+    import hpfp8
+    M, N, K = 327680, 256, 7168                      # a is 2.19 GiB
+    g = torch.Generator(device=gpu).manual_seed(9)
+    a = torch.randint(0, 0x7F, (M, K), generator=g, device=gpu, dtype=torch.uint8)
+    a |= torch.randint(0, 2, (M, K), generator=g, device=gpu, dtype=torch.uint8) << 7
+    a = a.view(torch.float8_e4m3fn)
+    sa = (torch.rand((K // 128, M), generator=g, device=gpu) + 0.5).t()
+    w = (torch.randn((N, K), generator=g, device=gpu) * 0.01).to(torch.bfloat16)
+    wq, sw = hpfp8.quantize_128x128(w)
+    y = hpfp8.gemm_blockwise(a, sa, wq, sw)
+    for r0 in (0, 299520, M - 256):                  # 299520 * 7168 is just below 2^31, the tile crosses it
+        part = hpfp8.gemm_blockwise(a[r0:r0 + 256], sa[r0:r0 + 256], wq, sw)
+        assert torch.equal(y[r0:r0 + 256], part), r0
+    ref = ref_f64_torch(a[M - 256:], sa[M - 256:], wq, sw.repeat_interleave(128, dim=0), gpu)
+    assert rel(U.f32(y[M - 256:]), ref.cpu().numpy()) < TOL_BF16
