@@ -32,7 +32,7 @@ constexpr int kTileBytes = 256 * BK;          // one operand tile in LDS (32 KB)
 // third buffer and its transfers run two k-blocks ahead; a's re-reads come from the Infinity Cache.
 __host__ __device__ constexpr int b_stages(int mode) { return mode == 2 /* kScaleRow: LDS also holds scales */ ? 2 : 3; }
 constexpr int kXcds = 8;
-constexpr int kGroupM = 8, kGroupN = 4;   // tile rectangle one XCD works on at a time
+constexpr int kRectTiles = 32;              // tiles of the rectangle one XCD (32 CUs) works on at a time
 
 enum ScaleMode { kScaleTensor = 0, kScaleBlock = 1, kScaleRow = 2 };
 
@@ -86,16 +86,21 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 }
 
 // Tile number -> (m tile, n tile).  Consecutive numbers (one XCD's CUs at any moment) cover
-// kGroupM x kGroupN rectangles of tiles, n fastest inside a rectangle, so the L2 of that XCD serves
-// each activation / weight panel to several CUs.  Rectangles at the right and bottom edges shrink.
+// gm x gn rectangles of tiles (gm * gn = 32), n fastest inside a rectangle, so the L2 of that XCD
+// serves each activation / weight panel to several CUs.  A panel of a is fetched once per column
+// of rectangles (tiles_n / gn times in all) and a panel of b once per row of rectangles: the longer
+// side of the rectangle goes along the shorter side of the tile grid, so that the larger operand,
+// the one the Infinity Cache cannot hold, is the one fetched fewer times.  Rectangles at the right
+// and bottom edges shrink.
 __device__ __forceinline__ void rect_map(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int per_ngroup = kGroupN * tiles_m;
+  const int gm = tiles_m > tiles_n ? 4 : 8, gn_full = kRectTiles / gm;
+  const int per_ngroup = gn_full * tiles_m;
   const int ng = t / per_ngroup, rest = t % per_ngroup;
-  const int gn = (tiles_n - ng * kGroupN) < kGroupN ? (tiles_n - ng * kGroupN) : kGroupN;
-  const int mg = rest / (kGroupM * gn);
-  const int r3 = rest - mg * kGroupM * gn;
-  tm = mg * kGroupM + r3 / gn;
-  tn = ng * kGroupN + r3 % gn;
+  const int gn = (tiles_n - ng * gn_full) < gn_full ? (tiles_n - ng * gn_full) : gn_full;
+  const int mg = rest / (gm * gn);
+  const int r3 = rest - mg * gm * gn;
+  tm = mg * gm + r3 / gn;
+  tn = ng * gn_full + r3 % gn;
 }
 
 // One output tile of a workgroup's list.  A tile with no rows (row0 == row_end, n0 >= N) stands for
@@ -148,7 +153,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   const int tiles_n = (N + BN - 1) / BN;
 
   // ---- the tile list of this workgroup.  The grid is persistent (one workgroup per CU); tiles are
-  // numbered so that consecutive numbers cover kGroupM x kGroupN rectangles, each XCD (workgroup ids
+  // numbered so that consecutive numbers cover rectangles of 32 tiles (rect_map), each XCD (workgroup ids
   // congruent mod 8, own L2) owns a contiguous run of numbers, and the workgroups of an XCD walk
   // through that run side by side, so at any moment they work on one rectangle.
   int total_tiles = p.tiles;
@@ -222,17 +227,24 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   lookup(2, T2);
   // ---- global -> LDS tile DMA.  One wave instruction moves 8 rows x 128 B (lane i -> LDS slot
   // i); the lane picks the 16-byte global chunk whose swizzled home is its slot.  The buffer
-  // resource of a transfer starts at the tile's first row and ends with the tensor (or the expert),
-  // so lane offsets do not depend on the tile and rows past the end read as zero.
+  // resource of a transfer starts at the tile's first row and ends with the tensor, so lane
+  // offsets do not depend on the tile and rows past the end of the tensor read as zero.
+  // (The resource runs on to the end of the tensor rather than to the end of the tile: transfers
+  // through a resource that only just covers the rows they touch were measured markedly slower.  Rows
+  // of a between the end of a ragged tile and the end of the tensor are read but never stored.)
+  auto span_bytes = [](int64_t rows, int64_t ld) {
+    const int64_t bytes = rows * ld;
+    return (int)(bytes < (int64_t)0x7FFFF000 ? bytes : (int64_t)0x7FFFF000);   // 256 rows always fit (host check)
+  };
   auto rsrc_a_of = [&](const TileInfo& ti) {
-    return __builtin_amdgcn_make_buffer_rsrc((void*)(p.a + (int64_t)ti.row0 * p.lda), 0,
-                                             (int)((int64_t)(ti.row_end - ti.row0) * p.lda), 0x00020000);
+    const int rows = ti.row_end > ti.row0 ? p.M - ti.row0 : 0;
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(p.a + (int64_t)ti.row0 * p.lda), 0, span_bytes(rows, p.lda),
+                                             0x00020000);
   };
   auto rsrc_b_of = [&](const TileInfo& ti) {
-    int rows = N - ti.n0 > 0 ? N - ti.n0 : 0;
-    if (rows > BN) rows = BN;
+    const int rows = N - ti.n0 > 0 ? N - ti.n0 : 0;
     const uint8_t* base = p.b + (GROUPED ? (int64_t)ti.expert * N * p.ldb : 0) + (int64_t)(rows ? ti.n0 : 0) * p.ldb;
-    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)((int64_t)rows * p.ldb), 0x00020000);
+    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, span_bytes(rows, p.ldb), 0x00020000);
   };
   uint32_t a_off[4], b_off[4];
 #pragma unroll
