@@ -151,6 +151,11 @@ def other_configs(dev):
         "dgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq, sgo, wqt, sw.t()))),
         "wgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1))),
     }
+    # the same weight gradient added onto an fp32 main gradient (apply_grad_on_fp32_main_grad)
+    main_grad = torch.zeros((n, k), dtype=torch.float32, device=dev)
+    res["cfg3_backward"]["wgrad_gemm_into_fp32_main_grad"] = tf(
+        fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=main_grad, accumulate=True)))
+    del main_grad
     del x, go, w, wq, wqt, goq, got, xt
     torch.cuda.empty_cache()
     # cfg 4: MoE grouped, 32 experts, 131072 routed rows, Zipf(1.1) counts, two empty experts

@@ -618,9 +618,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
                   const float4 old = *dst;
                   o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
                 }
-                *dst = o;
+                // streaming stores: the output is not read again here, and as ordinary stores a tile's
+                // 128-256 KB would push operand panels out of the L2
+                __builtin_nontemporal_store(v4f{o.x, o.y, o.z, o.w}, reinterpret_cast<v4f*>(dst));
               } else {
-                *reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + ncol + l16e * 8) = val[k];
+                __builtin_nontemporal_store(
+                    val[k], reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + ncol + l16e * 8));
               }
             }
           }
