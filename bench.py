@@ -84,7 +84,7 @@ def cpu_baseline(x_bits, w_bits, target_seconds=15.0):
     }
 
 
-def _time(fn, iters=20, warm=20):
+def _time(fn, iters=30, warm=40):
     import torch
     for _ in range(warm):
         fn()
@@ -126,6 +126,26 @@ def other_configs(dev):
     res["cfg2_swiglu_quantize"] = gb(4096 * 18432 * 5 + 4096 * (18432 // 128) * 4,
                                      _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True)))
     del hgu
+    # cfg 2 as a training step of the module: forward + backward through fp8_linear (the weight's FP8 form
+    # made beforehand, as Fp8Linear's cache does), beside torch's bf16 F.linear on the same tensors
+    import torch.nn.functional as F
+    xt_ = torch.randn((4096, 7168), generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+    wt_ = (torch.randn((36864, 7168), generator=g, device=dev) * 0.006).to(torch.bfloat16).requires_grad_(True)
+    got_ = (torch.randn((4096, 36864), generator=g, device=dev) * 1e-3).to(torch.bfloat16)
+    wf_ = hpfp8.quantize_weight(wt_.detach())
+
+    def _step(fn):
+        y_ = fn()
+        y_.backward(got_)
+        xt_.grad = None
+        wt_.grad = None
+
+    ms_fp8 = _time(lambda: _step(lambda: hpfp8.fp8_linear(xt_, wt_, weight_fp8=wf_)), iters=20, warm=30)
+    ms_bf16 = _time(lambda: _step(lambda: F.linear(xt_, wt_)), iters=20, warm=30)
+    res["cfg2_training_step"] = {"fp8_linear_fwd_bwd_ms": ms_fp8, "torch_bf16_linear_fwd_bwd_ms": ms_bf16,
+                                 "TFLOP/s": 3 * 2.0 * 4096 * 36864 * 7168 / ms_fp8 / 1e9}
+    del xt_, wt_, got_, wf_
+    torch.cuda.empty_cache()
     # cfg 3: o_proj backward
     m, n, k = 4096, 7168, 16384
     x = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
