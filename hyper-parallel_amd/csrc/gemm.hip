@@ -137,14 +137,18 @@ __device__ __forceinline__ int expert_end(int off, int prev, int total_rows) {
   return lo < total_rows ? lo : total_rows;
 }
 
-template <int MODE, bool GROUPED, bool OUT_F32>
+template <int MODE, bool GROUPED, bool OUT_F32, bool ACC>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
+  static_assert(!ACC || (OUT_F32 && MODE != kScaleTensor), "accumulating onto c: fp32 output, promoted sums");
   constexpr int kBStages = b_stages(MODE);
   constexpr int kBAhead = kBStages - 1;     // k-blocks between issuing a b transfer and using it
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[(2 + kBStages) * kTileBytes];
+  // One LDS object for everything.  (With a second __shared__ array the compiler tells the two apart
+  // with alias scopes, and from then on makes every LDS read wait for all transfers into the array it
+  // reads, those to other buffers included: the transfers' latency would be paid in every round.)
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[(2 + kBStages) * kTileBytes + (MODE == kScaleRow ? 3 * BN * 4 : 0)];
   // per-row scales of the b operand for one k-block (wgrad form), three stages of 256 floats: the
   // stage of k-block kb+1 is filled while slower waves may still read that of kb-1
-  __shared__ __attribute__((aligned(16))) float sb_lds[MODE == kScaleRow ? 3 * BN : 4];
+  float* const sb_lds = reinterpret_cast<float*>(lds + (2 + kBStages) * kTileBytes);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -322,8 +326,36 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     for (int j = 0; j < 4; ++j) s[j] = MODE == kScaleBlock ? raw[j] * raw[4] : raw[j];
   };
 
+  // ---- accumulators.  When the result is added onto c (ACC), a tile's accumulators do not start from
+  // zero but from the tile's old values, loaded right before its first round in the order in which
+  // that round touches them: they cost no registers and only the first of them is waited for.  A
+  // lane's four sums of one 16 x 16 subtile are four consecutive columns of one row: one 16-byte
+  // load.  The resource ends with the tensor: rows past it (and the tiles past the end of the list)
+  // read as zero.
+  auto rsrc_c_of = [&](const TileInfo& ti) {
+    const int ncol = ti.n0 + wn * 128;
+    const bool ok = ti.row_end > ti.row0 && ncol < N;
+    int64_t bytes = ok ? (((int64_t)p.M - ti.row0 - 1) * p.ldc + N - ncol) * 4 : 0;
+    if (bytes > (int64_t)0x7FFFF000) bytes = 0x7FFFF000;       // 256 rows always fit (host check)
+    const float* base = reinterpret_cast<const float*>(p.c) + (ok ? (int64_t)ti.row0 * p.ldc + ncol : 0);
+    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
+  };
+  const int c_jstep = 16 * (int)p.ldc * 4;                     // bytes between the rows of subtiles j and j + 1
+  auto old_values = [&](const __amdgpu_buffer_rsrc_t& rs, uint32_t lane_off, int i, int j) {
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off + i * 64, j * c_jstep, 0));
+  };
   const v4f zero = {0.f, 0.f, 0.f, 0.f};
   v4f acc[8][4];
+  auto load_old_values = [&](const TileInfo& ti) {
+    int lane_c = lane;
+    asm volatile("" : "+v"(lane_c));    // (keeps the lane offset out of the registers held through the rounds)
+    const __amdgpu_buffer_rsrc_t rc = rsrc_c_of(ti);
+    const uint32_t c_lane = ((uint32_t)(wm * 64 + (lane_c & 15)) * (uint32_t)p.ldc + (lane_c >> 4) * 4) * 4u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = old_values(rc, c_lane, i, j);
+  };
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
@@ -386,6 +418,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   __amdgpu_buffer_rsrc_t rs_a1 = rsrc_a_of(T0), rs_a2 = rs_a1, rs_b1 = rsrc_b_of(T0), rs_b2 = rs_b1;
 
   for (int tile = 0; tile < my_tiles; ++tile) {
+  if (ACC) load_old_values(T0);
   for (int kb = 0; kb < kblocks; ++kb) {
     // Where this round's transfers and scale loads go: one k-block ahead (scales, second half of
     // those tiles), two ahead (first half of those tiles, or the whole b tile when it has three
@@ -613,14 +646,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
               if (OUT_F32) {
                 float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.c) + (int64_t)m * p.ldc + ncol + h * 64 + l16e * 4);
                 const v4f fv = __builtin_bit_cast(v4f, val[k]);   // (a cast of the whole vector, not of its elements)
-                float4 o = make_float4(fv[0], fv[1], fv[2], fv[3]);
-                if (p.accumulate) {
-                  const float4 old = *dst;
-                  o.x += old.x; o.y += old.y; o.z += old.z; o.w += old.w;
-                }
                 // streaming stores: the output is not read again here, and as ordinary stores a tile's
                 // 128-256 KB would push operand panels out of the L2
-                __builtin_nontemporal_store(v4f{o.x, o.y, o.z, o.w}, reinterpret_cast<v4f*>(dst));
+                __builtin_nontemporal_store(fv, reinterpret_cast<v4f*>(dst));
               } else {
                 __builtin_nontemporal_store(
                     val[k], reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + ncol + l16e * 8));
@@ -638,9 +666,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     else store_tile(std::true_type{}, std::false_type{});
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = zero;
+      for (int i = 0; i < 8; ++i) acc[i][j] = zero;
   }
   T0 = T1;
   T1 = T2;
@@ -671,10 +699,17 @@ static int persistent_grid(int64_t tiles) {
 template <int MODE, bool GROUPED>
 static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
   dim3 grid((unsigned)persistent_grid(tiles)), block(kGemmThreads);
-  if (out_type == HPFP8_OUT_F32)
-    gemm_kernel<MODE, GROUPED, true><<<grid, block, 0, stream>>>(p);
-  else
-    gemm_kernel<MODE, GROUPED, false><<<grid, block, 0, stream>>>(p);
+  if (out_type == HPFP8_OUT_F32) {
+    if constexpr (MODE != kScaleTensor && !GROUPED) {   // (the per-tensor and grouped entry points have no accumulate)
+      if (p.accumulate) {
+        gemm_kernel<MODE, GROUPED, true, true><<<grid, block, 0, stream>>>(p);
+        return check_launch("gemm");
+      }
+    }
+    gemm_kernel<MODE, GROUPED, true, false><<<grid, block, 0, stream>>>(p);
+  } else {
+    gemm_kernel<MODE, GROUPED, false, false><<<grid, block, 0, stream>>>(p);
+  }
   return check_launch("gemm");
 }
 
@@ -703,6 +738,9 @@ static int check_common(const char* what, const void* a, int64_t lda, const void
   HPFP8_REQUIRE(BM * lda < (int64_t)0x7FFFFFFF && BN * ldb < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
                 "%s: a row stride of 8 MiB or more is not supported", what);
   HPFP8_REQUIRE(M < (int64_t)0x7FFFFF00 && N < (int64_t)0x7FFFFF00, HPFP8_ERR_SHAPE, "%s: M or N too large", what);
+  // the old values of a tile are read with 32-bit byte offsets (256 rows of c)
+  HPFP8_REQUIRE(!accumulate || BM * ldc * 4 < (int64_t)0x7FFFF000, HPFP8_ERR_SHAPE,
+                "%s: accumulate needs a row stride of c below 8 MiB", what);
   return 1;
 }
 
@@ -743,6 +781,8 @@ int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa
   p.tiles = (int)tiles;
   if (sb_gran == 128) return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
   // per-row b scales travel to LDS as one contiguous 1 KB piece per k-block
+  if (K == BK) sb_stride_k = N;     // a single k-block: the stride between k-blocks is never used
+  p.sb_sk = sb_stride_k;
   HPFP8_REQUIRE(sb_stride_n == 1 && sb_stride_k >= N && sb_stride_k % 4 == 0 && aligned16(sb), HPFP8_ERR_SHAPE,
                 "gemm_blockwise: with sb_gran=1 the b scales must be k-block-major (sb_stride_n = 1, sb_stride_k >= N, "
                 "16-byte aligned rows)");

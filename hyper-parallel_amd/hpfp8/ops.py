@@ -333,7 +333,7 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
     want_sb = (n // BLOCK, kb) if sb_gran == 128 else (n, kb)
     if sb_gran not in (1, 128) or tuple(sb.shape) != want_sb:
         raise ValueError(f"sb must be {list(want_sb)} for sb_gran={sb_gran}, got {tuple(sb.shape)}")
-    if sb_gran == 1 and (sb.stride(0) != 1 or sb.stride(1) < n or sb.stride(1) % 4 or sb.data_ptr() % 16):
+    if sb_gran == 1 and (sb.stride(0) != 1 or (kb > 1 and (sb.stride(1) < n or sb.stride(1) % 4)) or sb.data_ptr() % 16):
         sb = sb.t().contiguous().t()        # the kernel wants per-row b scales k-block-major
     if bias is not None:
         bias = _check_bf16(bias, "bias")

@@ -141,6 +141,38 @@ def test_output_row_stride_and_many_tiles_per_workgroup(gpu):
         assert torch.equal(out, hpfp8.gemm_blockwise(xq, sxi, wq, swi, out_dtype=dt))
 
 
+@pytest.mark.parametrize("M,N,K", [(320, 384, 512), (2500, 7808, 128), (3000, 5248, 256)])
+def test_accumulate_onto_fp32_is_exact_on_integer_inputs(gpu, M, N, K):
+    """accumulate adds the product onto what c holds.  With integer-valued operands, power-of-two scales
+    and an integer-valued c every sum is exact in fp32, so the result must equal old + product whatever
+    the order of summation; the larger cases give every workgroup several tiles (also with a single
+    k-block per tile), a ragged last row tile, a half-used last column tile and ldc > N, and the
+    columns of the wider buffer next to c must stay untouched."""
+    import hpfp8
+    rng = np.random.default_rng(M + N + K)
+    ai = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    bi = rng.integers(-8, 9, size=(N, K)).astype(np.float32)
+    a, b = O.e4m3_encode(ai), O.e4m3_encode(bi)
+    sa = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
+    sb = (2.0 ** rng.integers(-3, 4, size=(N // 128, K // 128))).astype(np.float32)
+    sbr = (2.0 ** rng.integers(-3, 4, size=(N, K // 128))).astype(np.float32)
+    old = rng.integers(-1000, 1001, size=(M, N)).astype(np.float32)
+    aq, bq = fp8(a, gpu), fp8(b, gpu)
+    for gran, sb_np in ((128, sb), (1, sbr)):
+        prod = hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, out_dtype=torch.float32)
+        if M * N * K <= 64 * 1024 * 1024:
+            want, _ = (O.gemm_blockwise if gran == 128 else O.gemm_rowwise_both)(a, sa, b, sb_np)
+            assert np.array_equal(U.f32(prod), want)
+        wide = torch.full((M, N + 12), 7.0, dtype=torch.float32, device=gpu)
+        c = wide[:, 4:4 + N]
+        c.copy_(torch.from_numpy(old))
+        hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, out=c, accumulate=True)
+        assert torch.equal(c, torch.from_numpy(old).to(gpu) + prod)
+        hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, out=c, accumulate=True)
+        assert torch.equal(c, torch.from_numpy(old).to(gpu) + 2 * prod)
+        assert bool((wide[:, :4] == 7.0).all()) and bool((wide[:, 4 + N:] == 7.0).all())
+
+
 @pytest.mark.parametrize("M,N,K,seed", [(256, 256, 128, 1), (512, 1024, 7168, 2), (1000, 384, 1024, 3),
                                          (8, 128, 256, 4), (4096, 512, 2048, 5)])
 def test_blockwise_forward_shapes(gpu, M, N, K, seed):
