@@ -48,7 +48,8 @@ def _flatten(x: torch.Tensor):
 
 class _Fp8LinearBlockwise(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, wq=None, sw=None, wqt=None):
+    def forward(ctx, x, weight, bias, wq=None, sw=None, wqt=None, on_main_grad=False):
+        ctx.main_grad_of = weight if on_main_grad else None
         x2 = _flatten(x)
         m = x2.shape[0]
         # With a weight gradient to come and a token count that allows it, x is read once: its 1x128
@@ -102,10 +103,19 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
             # dW[N,K] = go^T[N,M] . x[M,K]: contraction over tokens, both operands 1x128 along M
             if xt is None:
                 xt, sxt = ops.quantize_128x1_t(x2, kmajor=True)
-            dw = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1)
+            param = ctx.main_grad_of
+            if param is None:
+                dw = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1)
+            elif getattr(param, "main_grad", None) is None:
+                # the fp32 main gradient of hyper_parallel/platform/torch/fully_shard/param.py:134-167: the
+                # first weight gradient creates it, later ones are added onto it by the GEMM itself, and
+                # .grad stays empty
+                param.main_grad = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out_dtype=torch.float32)
+            else:
+                ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=param.main_grad, accumulate=True)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
-        return dx, dw, db, None, None, None
+        return dx, dw, db, None, None, None, None
 
 
 class _Fp8LinearPerTensor(torch.autograd.Function):
@@ -144,7 +154,8 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
 
 
 def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
-               recipe: str = "blockwise", weight_fp8: Optional[Fp8Weight] = None) -> torch.Tensor:
+               recipe: str = "blockwise", weight_fp8: Optional[Fp8Weight] = None,
+               apply_grad_on_fp32_main_grad: bool = False) -> torch.Tensor:
     """y = input @ weight.T + bias computed through E4M3 operands with fp32 accumulation.
 
     input [..., in_features] bf16, weight [out_features, in_features] bf16, bias [out_features] bf16
@@ -154,6 +165,11 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     `weight_fp8` (blockwise recipe) is the weight's FP8 form made earlier -- by `quantize_weight`, or
     from all-gathered FP8 shards (`hpfp8.fsdp`) -- and saves its quantization in this call; `weight`
     is still the tensor that receives the gradient.
+
+    `apply_grad_on_fp32_main_grad` (blockwise recipe; the flag of the reference's mixed-precision
+    policy, hyper_parallel/platform/torch/fully_shard/param.py:134-167) sends the weight gradient to
+    `weight.main_grad` instead of `weight.grad`: a float32 [out_features, in_features] tensor that the
+    first backward creates and every later one adds onto, inside the wgrad GEMM.
     """
     if recipe not in RECIPES:
         raise ValueError(f"recipe must be one of {RECIPES}, got {recipe!r}")
@@ -164,24 +180,34 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     for name, t in (("input", input), ("weight", weight), ("bias", bias)):
         if t is not None and t.dtype != torch.bfloat16:
             raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+    if apply_grad_on_fp32_main_grad:
+        if recipe != "blockwise":
+            raise ValueError("apply_grad_on_fp32_main_grad is only implemented for the blockwise recipe")
+        mg = getattr(weight, "main_grad", None)
+        if mg is not None and (mg.dtype != torch.float32 or tuple(mg.shape) != tuple(weight.shape) or
+                               not mg.is_contiguous()):
+            raise ValueError("weight.main_grad must be a contiguous float32 tensor of the weight's shape")
     if weight_fp8 is not None:
         if recipe != "blockwise":
             raise ValueError("weight_fp8 is only used by the blockwise recipe")
         if tuple(weight_fp8.codes.shape) != tuple(weight.shape):
             raise ValueError("weight_fp8 does not have the weight's shape")
         return _Fp8LinearBlockwise.apply(input, weight, bias, weight_fp8.codes, weight_fp8.scale_inv,
-                                         weight_fp8.codes_t)
-    fn = _Fp8LinearBlockwise if recipe == "blockwise" else _Fp8LinearPerTensor
-    return fn.apply(input, weight, bias)
+                                         weight_fp8.codes_t, apply_grad_on_fp32_main_grad)
+    if recipe == "blockwise":
+        return _Fp8LinearBlockwise.apply(input, weight, bias, None, None, None, apply_grad_on_fp32_main_grad)
+    return _Fp8LinearPerTensor.apply(input, weight, bias)
 
 
 class Fp8Linear(nn.Module):
     """Drop-in for torch.nn.Linear (bf16 parameters) whose matmuls run through fp8_linear."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, *, recipe: str = "blockwise",
-                 cache_weight: bool = True, device=None, dtype=torch.bfloat16):
+                 cache_weight: bool = True, apply_grad_on_fp32_main_grad: bool = False, device=None,
+                 dtype=torch.bfloat16):
         super().__init__()
         self.cache_weight = cache_weight
+        self.apply_grad_on_fp32_main_grad = apply_grad_on_fp32_main_grad
         self._fp8: Optional[Fp8Weight] = None
         self._fp8_key = None
         if recipe not in RECIPES:
@@ -202,7 +228,8 @@ class Fp8Linear(nn.Module):
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         if self.recipe != "blockwise" or not self.cache_weight:
-            return fp8_linear(input, self.weight, self.bias, recipe=self.recipe)
+            return fp8_linear(input, self.weight, self.bias, recipe=self.recipe,
+                              apply_grad_on_fp32_main_grad=self.apply_grad_on_fp32_main_grad)
         # The FP8 form of the weight is kept until the parameter is written again (optimizer step,
         # load_state_dict, ...): micro-batches of one step and inference calls quantize it once.
         key = (self.weight._version, self.weight.data_ptr())
@@ -210,7 +237,8 @@ class Fp8Linear(nn.Module):
             with torch.no_grad():
                 self._fp8 = quantize_weight(self.weight.detach(), with_transpose=True)
             self._fp8_key = key
-        return fp8_linear(input, self.weight, self.bias, recipe=self.recipe, weight_fp8=self._fp8)
+        return fp8_linear(input, self.weight, self.bias, recipe=self.recipe, weight_fp8=self._fp8,
+                          apply_grad_on_fp32_main_grad=self.apply_grad_on_fp32_main_grad)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "

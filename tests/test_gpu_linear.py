@@ -67,7 +67,7 @@ def test_module_is_a_drop_in_for_nn_linear(gpu):
         loss = (mod(x).float() ** 2).mean()
         loss.backward()
         opt.step()
-        loss0 = loss0 if loss0 is not None else float(loss)
+        loss0 = loss0 if loss0 is not None else float(loss.detach())
     assert float(loss) < loss0
     nob = hpfp8.Fp8Linear(256, 128, bias=False, device=gpu)
     assert nob(x).shape == (128, 128)
@@ -116,6 +116,43 @@ def test_prequantized_weight_and_module_cache(gpu):
         mod.weight.mul_(2.0)                  # an in-place update, as an optimizer step is
     b = mod(x.detach())
     assert mod._fp8_key != key and torch.equal(b, hpfp8.fp8_linear(x.detach(), mod.weight.detach()))
+
+
+def test_weight_gradient_onto_fp32_main_grad(gpu):
+    """apply_grad_on_fp32_main_grad: the first backward creates weight.main_grad as the fp32 weight
+    gradient, later ones are added onto it by the wgrad GEMM, weight.grad stays empty and the other
+    gradients are those of the ordinary call."""
+    import hpfp8
+    x = U.randn_bf16((512, 384), 51).to(gpu).requires_grad_(True)
+    w = U.randn_bf16((256, 384), 52, 0.02).to(gpu).requires_grad_(True)
+    go1 = U.randn_bf16((512, 256), 53, 1e-3).to(gpu)
+    go2 = U.randn_bf16((512, 256), 54, 2e-3).to(gpu)
+    grads = []
+    for go in (go1, go2):
+        hpfp8.fp8_linear(x, w).backward(go)
+        grads.append((x.grad.clone(), w.grad.float().clone()))
+        x.grad = w.grad = None
+    hpfp8.fp8_linear(x, w, apply_grad_on_fp32_main_grad=True).backward(go1)
+    assert w.grad is None and w.main_grad.dtype == torch.float32 and torch.equal(x.grad, grads[0][0])
+    first = w.main_grad.clone()
+    assert torch.equal(first.to(torch.bfloat16).float(), grads[0][1])      # the same sums before the bf16 rounding
+    x.grad = None
+    hpfp8.fp8_linear(x, w, apply_grad_on_fp32_main_grad=True).backward(go2)
+    assert w.grad is None and torch.equal(x.grad, grads[1][0])
+    want = first.double() + grads[1][1].double()
+    assert rel(w.main_grad, want) < 3e-3                                   # (grads[1] went through bf16)
+    second_alone = w.main_grad.double() - first.double()
+    assert rel(second_alone, grads[1][1]) < 5e-3
+    mod = hpfp8.Fp8Linear(384, 256, bias=True, apply_grad_on_fp32_main_grad=True, device=gpu)
+    mod(x.detach()).backward(go1)
+    mod(x.detach()).backward(go1)
+    assert mod.weight.grad is None and mod.bias.grad is not None
+    ref_mod = hpfp8.Fp8Linear(384, 256, bias=True, device=gpu)
+    ref_mod.load_state_dict(mod.state_dict())
+    ref_mod(x.detach()).backward(go1)
+    assert rel(mod.weight.main_grad, 2 * ref_mod.weight.grad.double()) < 3e-3
+    with pytest.raises(ValueError):
+        hpfp8.fp8_linear(x, w, recipe="per_tensor", apply_grad_on_fp32_main_grad=True)
 
 
 def test_fp8_all_gather_hooks_rebuild_the_full_weight(gpu):
