@@ -200,6 +200,39 @@ def test_blockwise_forward_shapes(gpu, M, N, K, seed):
     assert rel(U.f32(acc), (ref + 1.5).cpu().numpy()) < TOL_F32
 
 
+def test_repeated_launches_give_identical_bits(gpu):
+    """The kernels synchronise their LDS buffers by hand (counted waits and one barrier per k-block); a
+    missing wait would show as launches of the same problem that differ now and then.  Every form,
+    several tiles per workgroup, 40 launches each."""
+    import hpfp8
+    T, A, B = 512, 2560, 7808
+    ga = U.randn_bf16((T, A), 61, 1e-3).to(gpu)
+    gb = U.randn_bf16((T, B), 62).to(gpu)
+    at, sat = hpfp8.quantize_128x1_t(ga, kmajor=True)
+    bt, sbt = hpfp8.quantize_128x1_t(gb, kmajor=True)
+    aq, sa = hpfp8.quantize_1x128(ga.t().contiguous(), kmajor=True)
+    bq, sb = hpfp8.quantize_128x128(gb.t().contiguous())
+    one = torch.ones(1, device=gpu)
+    old = torch.from_numpy(np.random.default_rng(0).standard_normal((A, B)).astype(np.float32)).to(gpu)
+    acc = torch.empty_like(old)
+
+    def accumulate():
+        acc.copy_(old)
+        return hpfp8.gemm_blockwise(at, sat, bt, sbt, sb_gran=1, out=acc, accumulate=True)
+
+    forms = {
+        "row scales": lambda: hpfp8.gemm_blockwise(at, sat, bt, sbt, sb_gran=1),
+        "row scales, fp32": lambda: hpfp8.gemm_blockwise(at, sat, bt, sbt, sb_gran=1, out_dtype=torch.float32),
+        "row scales, accumulate": accumulate,
+        "block scales": lambda: hpfp8.gemm_blockwise(aq, sa, bq, sb),
+        "per tensor": lambda: hpfp8.gemm_per_tensor(aq, one, bq, one),
+    }
+    for name, fn in forms.items():
+        first = fn().clone()
+        for _ in range(40):
+            assert torch.equal(fn(), first), name
+
+
 def test_cfg2_dense_mlp_forward_slice_and_full_properties(gpu):
     """Config 2: x[4096,7168] with 0.1% x50 outliers, W[36864,7168] ~ N(0,0.006).  Full size on the
     GPU; checked against a float64 dequantized matmul on a slice of output columns plus linearity
