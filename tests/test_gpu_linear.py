@@ -68,7 +68,7 @@ def test_module_is_a_drop_in_for_nn_linear(gpu):
         loss.backward()
         opt.step()
         loss0 = loss0 if loss0 is not None else float(loss.detach())
-    assert float(loss) < loss0
+    assert float(loss.detach()) < loss0
     nob = hpfp8.Fp8Linear(256, 128, bias=False, device=gpu)
     assert nob(x).shape == (128, 128)
 
@@ -153,6 +153,35 @@ def test_weight_gradient_onto_fp32_main_grad(gpu):
     assert rel(mod.weight.main_grad, 2 * ref_mod.weight.grad.double()) < 3e-3
     with pytest.raises(ValueError):
         hpfp8.fp8_linear(x, w, recipe="per_tensor", apply_grad_on_fp32_main_grad=True)
+
+
+@pytest.mark.parametrize("recipe", ["blockwise", "per_tensor"])
+def test_forward_replays_from_a_captured_graph(gpu, recipe):
+    """Every entry point only enqueues kernels on the stream it is given (no allocation, no
+    synchronisation, no memset), so a forward pass can be captured into a graph; each replay, with
+    eager work and synchronisations in between, must give the eager result for the input of the moment."""
+    import hpfp8
+    w = U.randn_bf16((384, 512), 71, 0.02).to(gpu)
+    b = U.randn_bf16((384,), 72, 0.1).to(gpu)
+    xs = [U.randn_bf16((256, 512), 73 + i, 1.0 + i).to(gpu) for i in range(4)]
+    x_static = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        for _ in range(3):
+            hpfp8.fp8_linear(x_static, w, b, recipe=recipe)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), torch.no_grad():
+        y_static = hpfp8.fp8_linear(x_static, w, b, recipe=recipe)
+    for x in xs[1:] + xs[:2]:
+        x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            want = hpfp8.fp8_linear(x, w, b, recipe=recipe)
+        assert torch.equal(y_static, want)
 
 
 def test_fp8_all_gather_hooks_rebuild_the_full_weight(gpu):
