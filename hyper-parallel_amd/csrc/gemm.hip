@@ -30,11 +30,15 @@ constexpr int kTileBytes = 256 * BK;          // one operand tile in LDS (32 KB)
 // LDS: two buffers for the a tile, then kBStages buffers for the b tile.  The b operand is the one
 // that streams from HBM (each weight panel is used by one XCD only), so where LDS allows it gets a
 // third buffer and its transfers run two k-blocks ahead; a's re-reads come from the Infinity Cache.
-__host__ __device__ constexpr int b_stages(int mode) { return mode == 2 /* kScaleRow: LDS also holds scales */ ? 2 : 3; }
+__host__ __device__ constexpr int b_stages(int mode) { return (mode == 2 || mode == 4) /* per-row b scales: LDS also holds them */ ? 2 : 3; }
 constexpr int kXcds = 8;
 constexpr int kRectTiles = 32;              // tiles of the rectangle one XCD (32 CUs) works on at a time
 
-enum ScaleMode { kScaleTensor = 0, kScaleBlock = 1, kScaleRow = 2 };
+// kScalePow2: scales laid out as for kScaleBlock but every one a power of two; the matrix instruction
+// applies them itself (its E8M0 block-scale operands) and accumulates across k-blocks, so there is no
+// promotion arithmetic at all.
+// kScalePow2Row: the same with the scales laid out as for kScaleRow.
+enum ScaleMode { kScaleTensor = 0, kScaleBlock = 1, kScaleRow = 2, kScalePow2 = 3, kScalePow2Row = 4 };
 
 struct GemmParams {
   const uint8_t* a;
@@ -139,13 +143,16 @@ __device__ __forceinline__ int expert_end(int off, int prev, int total_rows) {
 
 template <int MODE, bool GROUPED, bool OUT_F32, bool ACC>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
-  static_assert(!ACC || (OUT_F32 && MODE != kScaleTensor), "accumulating onto c: fp32 output, promoted sums");
+  static_assert(!ACC || (OUT_F32 && (MODE == kScaleBlock || MODE == kScaleRow)), "accumulating onto c: fp32 output, promoted sums");
   constexpr int kBStages = b_stages(MODE);
+  constexpr bool kRowScales = MODE == kScaleRow || MODE == kScalePow2Row;   // per-row b scales, staged in LDS
+  constexpr bool kPromote = MODE == kScaleBlock || MODE == kScaleRow;       // partial sums scaled by FMAs
+  constexpr bool kHwScale = MODE == kScalePow2 || MODE == kScalePow2Row;    // scales applied by the MFMA
   constexpr int kBAhead = kBStages - 1;     // k-blocks between issuing a b transfer and using it
   // One LDS object for everything.  (With a second __shared__ array the compiler tells the two apart
   // with alias scopes, and from then on makes every LDS read wait for all transfers into the array it
   // reads, those to other buffers included: the transfers' latency would be paid in every round.)
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[(2 + kBStages) * kTileBytes + (MODE == kScaleRow ? 3 * BN * 4 : 0)];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[(2 + kBStages) * kTileBytes + (kRowScales ? 3 * BN * 4 : 0)];
   // per-row scales of the b operand for one k-block (wgrad form), three stages of 256 floats: the
   // stage of k-block kb+1 is filled while slower waves may still read that of kb-1
   float* const sb_lds = reinterpret_cast<float*>(lds + (2 + kBStages) * kTileBytes);
@@ -262,9 +269,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // wgrad form: the 256 per-row scales of the b tile for one k-block are one more 1 KB transfer
   // (wave 0), possible because that scale array is k-block-major (unit stride over rows).
   const __amdgpu_buffer_rsrc_t rsrc_sb = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)p.sb, 0, MODE == kScaleRow ? (int)((((int64_t)kblocks - 1) * p.sb_sk + N) * 4) : 0, 0x00020000);
+      (void*)p.sb, 0, kRowScales ? (int)((((int64_t)kblocks - 1) * p.sb_sk + N) * 4) : 0, 0x00020000);
   auto issue_sb_load = [&](const TileInfo& ti, int kb, int stage) {
-    if (MODE == kScaleRow && wave == 0)
+    if (kRowScales && wave == 0)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sb, (lds_ptr_t)(sb_lds + stage * BN), 16,
                                                (uint32_t)(ti.n0 + lane * 4) * 4u, (int)(kb * p.sb_sk * 4), 0, 0);
   };
@@ -313,7 +320,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     sb_soff = ((GROUPED ? ti.expert * (int)p.sb_se : 0) + nblk_idx * (int)p.sb_sn) * 4;
   };
   auto load_scales = [&](int kb, float raw[5]) {
-    if (MODE == kScaleBlock)
+    if (MODE == kScaleBlock || MODE == kScalePow2)
       raw[4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sbb, 0, sb_soff + kb * sb_kstep, 0));
     if (MODE != kScaleTensor) {
 #pragma unroll
@@ -321,9 +328,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
         raw[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, sa_voff[j], kb * sa_kstep, 0));
     }
   };
+  // kScalePow2: the exponent fields of the scales of the current k-block, which are their E8M0 codes:
+  // e_a[j] for the activation rows j * 16 + l16 of this lane, e_b for the weight block
+  int e_a[4] = {127, 127, 127, 127}, e_b = 127;
   auto combine_scales = [&](const float raw[5], float s[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) s[j] = MODE == kScaleBlock ? raw[j] * raw[4] : raw[j];
+    if (kHwScale) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) e_a[j] = (int)(__builtin_bit_cast(uint32_t, raw[j]) >> 23);
+      if (MODE == kScalePow2) e_b = (int)(__builtin_bit_cast(uint32_t, raw[4]) >> 23);
+    }
   };
 
   // ---- accumulators.  When the result is added onto c (ACC), a tile's accumulators do not start from
@@ -483,7 +498,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       return i + 2 < 8 ? frag_read(bcur + b_frag_off + (i + 2) * 16 * BK, pc0)
                        : frag_read(bnxt + b_frag_off + (i + 2 - 8) * 16 * BK, pc0);
     };
-    if (MODE != kScaleTensor) {
+    if (kPromote) {
       // Software pipeline over the 8 n-subtiles: the matrix instructions of subtile i are issued
       // interleaved with the promotion FMAs of subtile i-1, whose partial sums left the matrix
       // pipe four instructions earlier, so neither pipe waits for the other.
@@ -541,15 +556,27 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       v8i wf[3];
       wf[0] = wf_n0;
       wf[1] = wf_n1;
+      // per-row b scales: this lane's row of subtile i is row i * 16 + l16 of the wave's 128
+      const float* sb_lane = sb_lds + sbuf * BN + wn * 128 + l16;
+      int e_bi[2] = {127, 127};
+      if (MODE == kScalePow2Row) e_bi[0] = (int)(__builtin_bit_cast(uint32_t, sb_lane[0]) >> 23);
+      if (MODE == kScalePow2Row) issue_sb_load(tile_1, kb1, snext);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if (i == 6) round_sync();
         wf[(i + 2) % 3] = read_ahead(i);
+        if (MODE == kScalePow2Row && i < 7) e_bi[(i + 1) & 1] = (int)(__builtin_bit_cast(uint32_t, sb_lane[(i + 1) * 16]) >> 23);
         issue_slot(i);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i % 3], xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+          // (weights on the A port, activations on the B port: a lane's own row is the one it supplies
+          // the scale of)
+          if (kHwScale)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i % 3], xf[j], acc[i][j], 0, 0, 0,
+                                                                        MODE == kScalePow2 ? e_b : e_bi[i & 1], 0, e_a[j]);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i % 3], xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
           if (i == 7) xf[j] = frag_read(anxt + a_frag_off + j * 16 * BK, pc0);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -700,7 +727,7 @@ template <int MODE, bool GROUPED>
 static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
   dim3 grid((unsigned)persistent_grid(tiles)), block(kGemmThreads);
   if (out_type == HPFP8_OUT_F32) {
-    if constexpr (MODE != kScaleTensor && !GROUPED) {   // (the per-tensor and grouped entry points have no accumulate)
+    if constexpr ((MODE == kScaleBlock || MODE == kScaleRow) && !GROUPED) {   // (the per-tensor and grouped entry points have no accumulate)
       if (p.accumulate) {
         gemm_kernel<MODE, GROUPED, true, true><<<grid, block, 0, stream>>>(p);
         return check_launch("gemm");
@@ -760,10 +787,10 @@ using namespace hpfp8;
 
 extern "C" {
 
-int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
-                         const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
-                         int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
-                         int64_t ldc, int out_type, int accumulate, hpfp8_stream_t stream) {
+static int gemm_blockwise_impl(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                               const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+                               int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
+                               int64_t ldc, int out_type, int accumulate, bool pow2, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(sb_gran == 1 || sb_gran == 128, HPFP8_ERR_ARG, "gemm_blockwise: sb_gran must be 1 or 128");
   int rc = check_common("gemm_blockwise", a, lda, b, ldb, sa, sb, M, N, K, bias, c, ldc, out_type, accumulate);
   if (rc <= 0) return rc;
@@ -779,7 +806,11 @@ int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.accumulate = accumulate;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   p.tiles = (int)tiles;
-  if (sb_gran == 128) return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
+  HPFP8_REQUIRE(!pow2 || !accumulate, HPFP8_ERR_ARG, "gemm_blockwise_pow2: no accumulate form");
+  if (sb_gran == 128) {
+    if (pow2) return launch<kScalePow2, false>(p, out_type, tiles, (hipStream_t)stream);
+    return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
+  }
   // per-row b scales travel to LDS as one contiguous 1 KB piece per k-block
   if (K == BK) sb_stride_k = N;     // a single k-block: the stride between k-blocks is never used
   p.sb_sk = sb_stride_k;
@@ -788,7 +819,24 @@ int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa
                 "16-byte aligned rows)");
   HPFP8_REQUIRE(((K / BK - 1) * sb_stride_k + N) * 4 < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
                 "gemm_blockwise: b scale array too large");
+  if (pow2) return launch<kScalePow2Row, false>(p, out_type, tiles, (hipStream_t)stream);
   return launch<kScaleRow, false>(p, out_type, tiles, (hipStream_t)stream);
+}
+
+int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                         const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+                         int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
+                         int64_t ldc, int out_type, int accumulate, hpfp8_stream_t stream) {
+  return gemm_blockwise_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, ldb, sb, sb_stride_n, sb_stride_k, sb_gran, M, N, K,
+                             bias, c, ldc, out_type, accumulate, false, stream);
+}
+
+int hpfp8_gemm_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                              const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+                              int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
+                              int out_type, hpfp8_stream_t stream) {
+  return gemm_blockwise_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, ldb, sb, sb_stride_n, sb_stride_k, sb_gran, M, N, K,
+                             bias, c, ldc, out_type, 0, true, stream);
 }
 
 int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,

@@ -71,10 +71,18 @@ __device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w <
 __device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
 
 // amax -> quantize multiplier and its inverse: two IEEE fp32 divisions, never rcp * x.
-__device__ __forceinline__ void scales_from_amax(float amax, float& scale, float& scale_inv) {
+// pow2: the inverse is rounded up to the next power of two (its exponent field is then its E8M0 code,
+// which the matrix instruction can apply by itself) and the multiplier is its exact reciprocal.
+__device__ __forceinline__ void scales_from_amax(float amax, float& scale, float& scale_inv, int pow2 = 0) {
   float amc = fmaxf(amax, kAmaxEps);
   scale = kFp8Max / amc;
   scale_inv = amc / kFp8Max;
+  if (pow2) {
+    uint32_t u = __float_as_uint(scale_inv);
+    if (u & 0x007FFFFFu) u = (u & 0xFF800000u) + 0x00800000u;
+    scale_inv = __uint_as_float(u);
+    scale = 1.0f / scale_inv;
+  }
 }
 
 __device__ __forceinline__ float clamp448(float y) {

@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kmajor_kernel(const uint16_t*
                                                                  uint8_t* __restrict__ q,
                                                                  float* __restrict__ scale,
                                                                  float* __restrict__ scale_inv, int rows,
-                                                                 int cols) {
+                                                                 int cols, int pow2) {
   const int groups = cols >> 7;
   const int gtiles = (groups + 3) >> 2;
   const int g0 = (blockIdx.x % gtiles) * 4, row0 = (blockIdx.x / gtiles) * 16;
@@ -139,7 +139,7 @@ __global__ __launch_bounds__(256) void quant_1x128_kmajor_kernel(const uint16_t*
     const bool ok = row < rows && g0 + u < groups;
     uint32_t m = row16_max_u32(mag8(v[u]));
     float s, si;
-    scales_from_amax(__uint_as_float(m << 16), s, si);
+    scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
     if (ok) nt_store8(q + (int64_t)row * cols + (g0 + u) * 128 + l16 * 8, cvt8<false>(v[u], s));
     if (l16 == 0) {
       s_s[u][r] = s;
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
                                                             int cols, uint8_t* __restrict__ q,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale,
-                                                            float* __restrict__ scale_inv) {
+                                                            float* __restrict__ scale_inv, int pow2) {
   const int cb = cols >> 7, rb = rows >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   __shared__ uint32_t part[16];
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
       m = row16_max_u32(part[threadIdx.x]);
       if (threadIdx.x == 0) {
         float s, si;
-        scales_from_amax(__uint_as_float(m << 16), s, si);
+        scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
         s_scale = s;
         if (scale) scale[sidx] = s;
         scale_inv[sidx] = si;
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
                                                             float* __restrict__ scale_t,
                                                             float* __restrict__ scale_inv_t,
                                                             uint8_t* __restrict__ q, float* __restrict__ scale_r,
-                                                            float* __restrict__ scale_inv_r) {
+                                                            float* __restrict__ scale_inv_r, int pow2) {
   const int kb = k >> 7, mb = m >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   const int wave = threadIdx.x >> 6;
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
         const int row = tile_row(rq, p);
         const uint32_t mr = row16_max_u32(mag8(v[p]));
         float s, si;
-        scales_from_amax(__uint_as_float(mr << 16), s, si);
+        scales_from_amax(__uint_as_float(mr << 16), s, si, pow2);
         *reinterpret_cast<uint2*>(q + ((int64_t)tr * 128 + row) * k + tc * 128 + cg * 8) = cvt8<false>(v[p], s);
         if (cg == 0) {
           s_row[row] = s;
@@ -447,7 +447,7 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
       uint32_t mw = pk_max_u16(pk_max_u16(part[0][word], part[1][word]), pk_max_u16(part[2][word], part[3][word]));
       uint32_t mag = (col & 1) ? (mw >> 16) : (mw & 0xFFFFu);
       float s, si;
-      scales_from_amax(__uint_as_float(mag << 16), s, si);
+      scales_from_amax(__uint_as_float(mag << 16), s, si, pow2);
       s_scale[col] = s;
       // row-major [k, m/128], or block-major [m/128, k] (unit stride over the output rows)
       int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
@@ -660,8 +660,8 @@ int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q
   return check_launch("quantize_1x128");
 }
 
-int hpfp8_quantize_1x128_kmajor_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
-                                     float* scale_inv, hpfp8_stream_t stream) {
+static int quantize_1x128_kmajor_impl(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                                      float* scale_inv, int pow2, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_1x128_kmajor: negative shape");
   HPFP8_REQUIRE(cols % kBlock == 0, HPFP8_ERR_SHAPE,
                 "quantize_1x128_kmajor: last dim %lld is not a multiple of 128", (long long)cols);
@@ -674,12 +674,22 @@ int hpfp8_quantize_1x128_kmajor_bf16(const void* x, int64_t rows, int64_t cols, 
   const int64_t blocks = ((groups + 3) / 4) * ((rows + 15) / 16);
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "quantize_1x128_kmajor: tensor too large");
   quant_1x128_kmajor_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
-      (const uint16_t*)x, (uint8_t*)q, scale, scale_inv, (int)rows, (int)cols);
+      (const uint16_t*)x, (uint8_t*)q, scale, scale_inv, (int)rows, (int)cols, pow2);
   return check_launch("quantize_1x128_kmajor");
 }
 
-int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
-                                float* scale, float* scale_inv, hpfp8_stream_t stream) {
+int hpfp8_quantize_1x128_kmajor_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                                     float* scale_inv, hpfp8_stream_t stream) {
+  return quantize_1x128_kmajor_impl(x, rows, cols, q, scale, scale_inv, 0, stream);
+}
+
+int hpfp8_quantize_1x128_kmajor_pow2_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                                          float* scale_inv, hpfp8_stream_t stream) {
+  return quantize_1x128_kmajor_impl(x, rows, cols, q, scale, scale_inv, 1, stream);
+}
+
+static int quantize_128x128_impl(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
+                                 float* scale, float* scale_inv, int pow2, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_128x128: negative shape");
   HPFP8_REQUIRE(rows % kBlock == 0 && cols % kBlock == 0, HPFP8_ERR_SHAPE,
                 "quantize_128x128: shape [%lld, %lld] is not a multiple of 128", (long long)rows, (long long)cols);
@@ -695,17 +705,27 @@ int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void*
   hipStream_t s = (hipStream_t)stream;
   if (q_t)
     quant_128x128_kernel<true><<<(unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock), 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
-                                                                (uint8_t*)q, (uint8_t*)q_t, ld_t, scale, scale_inv);
+                                                                (uint8_t*)q, (uint8_t*)q_t, ld_t, scale, scale_inv, pow2);
   else
     quant_128x128_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
-                                                                 (uint8_t*)q, nullptr, 0, scale, scale_inv);
+                                                                 (uint8_t*)q, nullptr, 0, scale, scale_inv, pow2);
   return check_launch("quantize_128x128");
+}
+
+int hpfp8_quantize_128x128_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
+                                float* scale, float* scale_inv, hpfp8_stream_t stream) {
+  return quantize_128x128_impl(w, rows, cols, q, q_t, ld_t, scale, scale_inv, 0, stream);
+}
+
+int hpfp8_quantize_128x128_pow2_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
+                                     float* scale, float* scale_inv, hpfp8_stream_t stream) {
+  return quantize_128x128_impl(w, rows, cols, q, q_t, ld_t, scale, scale_inv, 1, stream);
 }
 
 // q != nullptr: also the 1x128 quantization of x itself (codes q, scales scale / scale_inv).
 static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, int64_t m, int64_t k, void* q_t,
                                  int64_t ld_t, float* scale_t, float* scale_inv_t, hpfp8_stream_t stream,
-                                 void* q = nullptr, float* scale = nullptr, float* scale_inv = nullptr) {
+                                 void* q = nullptr, float* scale = nullptr, float* scale_inv = nullptr, int pow2 = 0) {
   HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)m, (long long)k);
@@ -725,14 +745,14 @@ static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, i
   uint8_t* q8 = (uint8_t*)q;
   if (q) {
     if (kmajor)
-      quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv);
+      quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
     else
-      quant_128x1_t_kernel<false, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv);
+      quant_128x1_t_kernel<false, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
   } else {
     if (kmajor)
-      quant_128x1_t_kernel<true, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr);
+      quant_128x1_t_kernel<true, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
     else
-      quant_128x1_t_kernel<false, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr);
+      quant_128x1_t_kernel<false, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
   }
   return check_launch(what);
 }
@@ -753,6 +773,20 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
   HPFP8_REQUIRE(m == 0 || k == 0 || q != nullptr, HPFP8_ERR_ARG, "quantize_1x128_and_128x1_t: null buffer");
   return quantize_128x1_t_impl("quantize_1x128_and_128x1_t", kmajor != 0, x, m, k, q_t, ld_t, scale_t, scale_inv_t,
                                stream, q, scale, scale_inv);
+}
+
+int hpfp8_quantize_128x1_t_kmajor_pow2_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t,
+                                            float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
+  return quantize_128x1_t_impl("quantize_128x1_t_kmajor_pow2", true, x, m, k, q_t, ld_t, scale_t, scale_inv_t, stream,
+                               nullptr, nullptr, nullptr, 1);
+}
+
+int hpfp8_quantize_1x128_and_128x1_t_pow2_bf16(const void* x, int64_t m, int64_t k, int kmajor, void* q, float* scale,
+                                               float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
+                                               float* scale_inv_t, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(m == 0 || k == 0 || q != nullptr, HPFP8_ERR_ARG, "quantize_1x128_and_128x1_t_pow2: null buffer");
+  return quantize_128x1_t_impl("quantize_1x128_and_128x1_t_pow2", kmajor != 0, x, m, k, q_t, ld_t, scale_t, scale_inv_t,
+                               stream, q, scale, scale_inv, 1);
 }
 
 int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,

@@ -33,11 +33,17 @@ SIGNATURES = {
     "hpfp8_bucket_unpack_dequantize_bf16": [_vp, _vp, _vp, ctypes.c_int, _i64, _vp, _vp, ctypes.c_float, _vp],
     "hpfp8_quantize_1x128_and_128x1_t_bf16": [_vp, _i64, _i64, ctypes.c_int, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_quantize_128x128_bf16": [_vp, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
+    "hpfp8_quantize_1x128_kmajor_pow2_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
+    "hpfp8_quantize_128x128_pow2_bf16": [_vp, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
+    "hpfp8_quantize_128x1_t_kmajor_pow2_bf16": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp],
+    "hpfp8_quantize_1x128_and_128x1_t_pow2_bf16": [_vp, _i64, _i64, ctypes.c_int, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_quantize_128x1_t_bf16": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_dequantize_1x128_bf16": [_vp, _vp, _i64, _i64, _vp, _f32, _vp],
     "hpfp8_dequantize_128x128_bf16": [_vp, _vp, _i64, _i64, _vp, _vp],
     "hpfp8_gemm_blockwise": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp,
                              _vp, _i64, _int, _int, _vp],
+    "hpfp8_gemm_blockwise_pow2": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp,
+                                  _vp, _i64, _int, _vp],
     "hpfp8_gemm_per_tensor": [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _int, _vp],
     "hpfp8_gemm_grouped_blockwise": [_vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _i64,
                                      _int, _vp],

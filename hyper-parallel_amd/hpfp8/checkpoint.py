@@ -24,9 +24,9 @@ def fp8_state_dict(module: torch.nn.Module) -> Dict[str, torch.Tensor]:
     `<name>.weight_scale_inv` entry; everything else (biases, other layers) unchanged."""
     out = dict(module.state_dict())
     for name, sub in module.named_modules():
-        if isinstance(sub, Fp8Linear) and sub.recipe == "blockwise":
+        if isinstance(sub, Fp8Linear) and sub.recipe != "per_tensor":
             key = f"{name}.weight" if name else "weight"
-            wf = quantize_weight(sub.weight.detach(), with_transpose=False)
+            wf = quantize_weight(sub.weight.detach(), with_transpose=False, pow2=sub.recipe == "blockwise_pow2")
             out[key] = wf.codes
             out[key + SCALE_SUFFIX] = wf.scale_inv
     return out
@@ -62,9 +62,12 @@ def load_into(module: torch.nn.Module, state: Mapping[str, torch.Tensor]) -> Non
     module.load_state_dict(plain)
     for name, sub in module.named_modules():
         key = f"{name}.weight" if name else "weight"
-        if isinstance(sub, Fp8Linear) and key in fp8 and sub.recipe == "blockwise":
+        if isinstance(sub, Fp8Linear) and key in fp8 and sub.recipe != "per_tensor":
             codes, scale_inv = fp8[key]
             codes = codes.to(sub.weight.device).contiguous()
             scale_inv = scale_inv.to(sub.weight.device).float().contiguous()
-            sub._fp8 = Fp8Weight(codes, scale_inv, ops.transpose_codes(codes))
+            pow2 = sub.recipe == "blockwise_pow2"
+            if pow2 and bool((scale_inv.view(torch.int32) & 0x007FFFFF).any()):
+                continue        # plain fp32 scales: this module quantizes the dequantized weight itself
+            sub._fp8 = Fp8Weight(codes, scale_inv, ops.transpose_codes(codes), pow2)
             sub._fp8_key = (sub.weight._version, sub.weight.data_ptr())

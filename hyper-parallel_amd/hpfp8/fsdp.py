@@ -20,15 +20,15 @@ from . import ops
 from .linear import Fp8Weight
 
 
-def fsdp_pre_all_gather(weight_shard: torch.Tensor) -> Tuple[Tuple[torch.Tensor, torch.Tensor], Any]:
+def fsdp_pre_all_gather(weight_shard: torch.Tensor, pow2: bool = False) -> Tuple[Tuple[torch.Tensor, torch.Tensor], Any]:
     """bf16 shard [N/S, K] -> ((codes as uint8 [N/S, K], scale_inv fp32 [N/S/128, K/128]), metadata).
 
     The two tensors are the all-gather inputs (uint8 rather than float8 so that any collective
     backend accepts them); metadata carries what the post hook needs to rebuild the shapes."""
     if weight_shard.dim() != 2:
         raise ValueError("weight shard must be 2-D")
-    codes, scale_inv = ops.quantize_128x128(weight_shard.contiguous())
-    return (codes.view(torch.uint8), scale_inv), {"k": weight_shard.shape[1]}
+    codes, scale_inv = ops.quantize_128x128(weight_shard.contiguous(), pow2=pow2)
+    return (codes.view(torch.uint8), scale_inv), {"k": weight_shard.shape[1], "pow2": bool(pow2)}
 
 
 def fsdp_post_all_gather(all_gather_outputs: Sequence[torch.Tensor], metadata: Any, *,
@@ -43,4 +43,4 @@ def fsdp_post_all_gather(all_gather_outputs: Sequence[torch.Tensor], metadata: A
     if codes.shape[0] != scale_inv.shape[0] * ops.BLOCK:
         raise ValueError("gathered codes and scales do not belong together")
     codes_t = ops.transpose_codes(codes) if with_transpose else None
-    return Fp8Weight(codes, scale_inv, codes_t)
+    return Fp8Weight(codes, scale_inv, codes_t, bool(metadata.get("pow2", False)))

@@ -115,12 +115,15 @@ def quantize_per_tensor(x: torch.Tensor, amax_in: Optional[torch.Tensor] = None
     return q, scale, scale_inv
 
 
-def quantize_1x128(x: torch.Tensor, want_scale: bool = False, kmajor: bool = False):
+def quantize_1x128(x: torch.Tensor, want_scale: bool = False, kmajor: bool = False, pow2: bool = False):
     """x[..., C] -> (codes, scale_inv[..., C/128]) (plus scale when ``want_scale``).
 
     With ``kmajor`` the scales are STORED k-block-major ([C/128, rows] in memory) and returned as the
     transposed view, so they index exactly like the row-major result but the GEMM reads them with
     unit stride across rows.  Values are identical in both layouts.
+
+    ``pow2`` (k-block-major layout only; also on the other blockwise quantizers): scale_inv rounded up
+    to a power of two, the optional recipe whose GEMMs are ``gemm_blockwise(..., pow2_scales=True)``.
     """
     x = _check_bf16(x, "x")
     if x.dim() < 1:
@@ -131,12 +134,14 @@ def quantize_1x128(x: torch.Tensor, want_scale: bool = False, kmajor: bool = Fal
     rows = x.numel() // cols if cols else 0
     q = torch.empty(x.shape, dtype=FP8, device=x.device)
     sshape = x.shape[:-1] + (cols // BLOCK,)
+    if pow2 and not kmajor:
+        raise ValueError("pow2 scales are written in the k-block-major layout only (kmajor=True)")
     if kmajor:
         store = (cols // BLOCK, rows)
         scale_inv = torch.empty(store, dtype=torch.float32, device=x.device)
         scale = torch.empty(store, dtype=torch.float32, device=x.device) if want_scale else None
-        _lib.call("hpfp8_quantize_1x128_kmajor_bf16", _ptr(x), rows, cols, _ptr(q), _ptr(scale), _ptr(scale_inv),
-                  _stream())
+        _lib.call("hpfp8_quantize_1x128_kmajor_pow2_bf16" if pow2 else "hpfp8_quantize_1x128_kmajor_bf16", _ptr(x), rows,
+                  cols, _ptr(q), _ptr(scale), _ptr(scale_inv), _stream())
         scale_inv = scale_inv.t()
         scale = scale.t() if want_scale else None
         if x.dim() != 2:
@@ -149,7 +154,7 @@ def quantize_1x128(x: torch.Tensor, want_scale: bool = False, kmajor: bool = Fal
     return (q, scale, scale_inv) if want_scale else (q, scale_inv)
 
 
-def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: bool = False):
+def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: bool = False, pow2: bool = False):
     """w[R, C] -> (codes[R, C], scale_inv[R/128, C/128]) (+ codes_t[C, R]) (+ scale)."""
     w = _check_bf16(w, "w")
     if w.dim() != 2:
@@ -161,8 +166,8 @@ def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: 
     qt = _empty_codes_t(c, r, w.device) if with_transpose else None     # row stride padded, see _padded_ld
     scale_inv = torch.empty((r // BLOCK, c // BLOCK), dtype=torch.float32, device=w.device)
     scale = torch.empty_like(scale_inv) if want_scale else None
-    _lib.call("hpfp8_quantize_128x128_bf16", _ptr(w), r, c, _ptr(q), _ptr(qt), _ld(qt) if with_transpose else 0,
-              _ptr(scale), _ptr(scale_inv), _stream())
+    _lib.call("hpfp8_quantize_128x128_pow2_bf16" if pow2 else "hpfp8_quantize_128x128_bf16", _ptr(w), r, c, _ptr(q),
+              _ptr(qt), _ld(qt) if with_transpose else 0, _ptr(scale), _ptr(scale_inv), _stream())
     out = (q, scale_inv)
     if with_transpose:
         out += (qt,)
@@ -202,7 +207,7 @@ def transpose_codes(q: torch.Tensor) -> torch.Tensor:
     return qt
 
 
-def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = False):
+def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = False, pow2: bool = False):
     """Transposed re-quantization for wgrad from the bf16 source.
 
     x[M, K] -> (codes_t[K, M], scale_inv_t[K, M/128]); one scale per 128 consecutive rows of a column.
@@ -218,7 +223,11 @@ def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = F
     sshape = (m // BLOCK, k) if kmajor else (k, m // BLOCK)
     scale_inv = torch.empty(sshape, dtype=torch.float32, device=x.device)
     scale = torch.empty_like(scale_inv) if want_scale else None
+    if pow2 and not kmajor:
+        raise ValueError("pow2 scales are written in the block-major layout only (kmajor=True)")
     name = "hpfp8_quantize_128x1_t_kmajor_bf16" if kmajor else "hpfp8_quantize_128x1_t_bf16"
+    if pow2:
+        name = "hpfp8_quantize_128x1_t_kmajor_pow2_bf16"
     _lib.call(name, _ptr(x), m, k, _ptr(qt), _ld(qt), _ptr(scale), _ptr(scale_inv), _stream())
     if kmajor:
         scale_inv = scale_inv.t()
@@ -226,7 +235,7 @@ def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = F
     return (qt, scale, scale_inv) if want_scale else (qt, scale_inv)
 
 
-def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True):
+def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True, pow2: bool = False):
     """Both operand forms of x[M, K] from one read of it.
 
     Returns (codes[M, K], scale_inv[M, K/128], codes_t[K, M], scale_inv_t[K, M/128]), bit-identical to
@@ -242,8 +251,8 @@ def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True):
     qt = _empty_codes_t(k, m, x.device)
     s_inv = torch.empty((k // BLOCK, m) if kmajor else (m, k // BLOCK), dtype=torch.float32, device=x.device)
     st_inv = torch.empty((m // BLOCK, k) if kmajor else (k, m // BLOCK), dtype=torch.float32, device=x.device)
-    _lib.call("hpfp8_quantize_1x128_and_128x1_t_bf16", _ptr(x), m, k, int(kmajor), _ptr(q), None, _ptr(s_inv),
-              _ptr(qt), _ld(qt), None, _ptr(st_inv), _stream())
+    _lib.call("hpfp8_quantize_1x128_and_128x1_t_pow2_bf16" if pow2 else "hpfp8_quantize_1x128_and_128x1_t_bf16", _ptr(x),
+              m, k, int(kmajor), _ptr(q), None, _ptr(s_inv), _ptr(qt), _ld(qt), None, _ptr(st_inv), _stream())
     if kmajor:
         s_inv, st_inv = s_inv.t(), st_inv.t()
     return q, s_inv, qt, st_inv
@@ -310,8 +319,8 @@ def _out_code(dtype: torch.dtype) -> int:
 
 def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor,
                    bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16,
-                   sb_gran: int = 128, out: Optional[torch.Tensor] = None, accumulate: bool = False
-                   ) -> torch.Tensor:
+                   sb_gran: int = 128, out: Optional[torch.Tensor] = None, accumulate: bool = False,
+                   pow2_scales: bool = False) -> torch.Tensor:
     """c[M,N] = sum_kb sa[m,kb] * sb[n//sb_gran, kb] * (a[m, kb] . b[n, kb]) (+ bias).
 
     a[M,K], b[N,K] codes (unit inner stride, any 16-byte-multiple row stride); sa, sb 2-D fp32 views
@@ -349,6 +358,13 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
         out_dtype = out.dtype
     if accumulate and out_dtype != torch.float32:
         raise ValueError("accumulate needs a float32 output")
+    if pow2_scales:
+        if accumulate:
+            raise ValueError("pow2_scales has no accumulate form")
+        _lib.call("hpfp8_gemm_blockwise_pow2", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ld(b),
+                  _ptr(sb), sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
+                  out.stride(0) if m > 1 else n, _out_code(out_dtype), _stream())
+        return out
     _lib.call("hpfp8_gemm_blockwise", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ld(b),
               _ptr(sb), sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
               out.stride(0) if m > 1 else n, _out_code(out_dtype), int(accumulate), _stream())

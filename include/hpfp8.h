@@ -110,6 +110,21 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
                                           float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
                                           float* scale_inv_t, hpfp8_stream_t stream);
 
+/* Power-of-two scales (an optional recipe; the stated one keeps plain fp32 scales): scale_inv is
+ * amax_c / 448 rounded up to the next power of two and scale its exact reciprocal, everything else as in
+ * the entry point of the same name without _pow2.  Such a scale_inv's fp32 exponent field is its E8M0
+ * code, which gfx950's block-scaled matrix instruction applies by itself: hpfp8_gemm_blockwise_pow2
+ * below.  No counterpart in the reference; same call sites as the plain forms. */
+int hpfp8_quantize_1x128_kmajor_pow2_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
+                                          float* scale_inv, hpfp8_stream_t stream);
+int hpfp8_quantize_128x128_pow2_bf16(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
+                                     float* scale, float* scale_inv, hpfp8_stream_t stream);
+int hpfp8_quantize_128x1_t_kmajor_pow2_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t,
+                                            float* scale_t, float* scale_inv_t, hpfp8_stream_t stream);
+int hpfp8_quantize_1x128_and_128x1_t_pow2_bf16(const void* x, int64_t m, int64_t k, int kmajor, void* q, float* scale,
+                                               float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
+                                               float* scale_inv_t, hpfp8_stream_t stream);
+
 /* SwiGLU fused with the 1x128 quantization of its result, the activations of the down projection
  * (the step after the gate/up linear of a DeepSeekV3 MLP; in the reference this is eager
  * F.silu(gate) * up between two aten::linear calls dispatched at
@@ -193,6 +208,17 @@ int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa
                          const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
                          int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
                          int64_t ldc, int out_type, int accumulate, hpfp8_stream_t stream);
+
+/* hpfp8_gemm_blockwise for scales that are powers of two (what the _pow2 quantizers write): the matrix
+ * instruction applies them as E8M0 block scales and sums the k-blocks itself, so the kernel spends no
+ * arithmetic on scaling.  Only the exponent field of a scale is used (mantissa bits are ignored, the
+ * sign must be +).  Same arguments and limits as hpfp8_gemm_blockwise, without accumulate.  Results
+ * agree with hpfp8_gemm_blockwise on the same operands to fp32 rounding (the order of the fp32
+ * additions differs), and are exact on the same integer-valued cases. */
+int hpfp8_gemm_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                              const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
+                              int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
+                              int out_type, hpfp8_stream_t stream);
 
 /* Per-tensor scales: c = (a . b^T) * (sa_inv[0] * sb_inv[0]) (+ bias), accumulation over the whole
  * K inside the matrix cores.  K a multiple of 128, N a multiple of 128. */

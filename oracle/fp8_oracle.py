@@ -41,6 +41,9 @@ How each function is pinned (tests/test_oracle_pins.py)
       every block separately (pure-Python loops on small shapes); the transposed variant
       equals quantize_1x128(x.T); the C restatement (fp8_oracle.c) is a second independent
       implementation compared bit for bit.
+  scales_from_amax(pow2)    : closed form (a power of two, >= amax/448 and < 2 amax/448, times its
+      reciprocal exactly 1, no product beyond 448); the quantizers with it are the ordinary ones
+      with that scale (scalar loop with torch's cast); not in the C restatement.
   gemm_*                    : torch._scaled_mm on CPU for per-tensor scales (library routine);
       exact integer-valued inputs with unit scales reduce to an exact integer matmul; the
       grouped variant equals a loop of dense calls; float64 dequant matmul bounds the rest.
@@ -135,13 +138,23 @@ def amax(x_f32: np.ndarray, axis=None, keepdims=False) -> np.ndarray:
                   keepdims=keepdims).astype(np.float32)
 
 
-def scales_from_amax(am: np.ndarray):
-    """amax -> (scale, scale_inv), two independent correctly rounded fp32 divisions."""
+def scales_from_amax(am: np.ndarray, pow2: bool = False):
+    """amax -> (scale, scale_inv), two independent correctly rounded fp32 divisions.
+
+    pow2 (an optional recipe beyond the stated one, whose scales are plain fp32): scale_inv is rounded
+    up to the next power of two -- its fp32 exponent field is then its E8M0 code, the form gfx950's
+    block-scaled matrix instruction applies by itself -- and scale is its exact reciprocal."""
     am = np.asarray(am, dtype=np.float32)
     amc = np.maximum(am, AMAX_EPS).astype(np.float32)
     with np.errstate(over="ignore"):
         scale = (FP8_MAX / amc).astype(np.float32)
         scale_inv = (amc / FP8_MAX).astype(np.float32)
+    if pow2:
+        u = np.ascontiguousarray(scale_inv).view(np.uint32)
+        up = (u & np.uint32(0xFF800000)) + np.uint32(0x00800000)
+        scale_inv = np.where((u & np.uint32(0x007FFFFF)) != 0, up, u).astype(np.uint32).view(np.float32).reshape(scale_inv.shape)
+        with np.errstate(divide="ignore"):
+            scale = (np.float32(1.0) / scale_inv).astype(np.float32)
     return scale, scale_inv
 
 
@@ -163,7 +176,7 @@ def quantize_per_tensor(x_bits: np.ndarray):
     return _cast(x, scale).reshape(x.shape), scale, scale_inv
 
 
-def quantize_1x128(x_bits: np.ndarray):
+def quantize_1x128(x_bits: np.ndarray, pow2: bool = False):
     """Row-wise groups of 128 along the last (contraction) dim.
 
     x[R, C], C % 128 == 0 -> codes[R, C], scale[R, C/128], scale_inv[R, C/128].
@@ -174,12 +187,12 @@ def quantize_1x128(x_bits: np.ndarray):
         raise ValueError(f"last dim {c} is not a multiple of {BLOCK}")
     g = x.reshape(r, c // BLOCK, BLOCK)
     am = amax(g, axis=2) if g.size else np.zeros((r, c // BLOCK), np.float32)
-    scale, scale_inv = scales_from_amax(am)
+    scale, scale_inv = scales_from_amax(am, pow2)
     codes = _cast(g, scale[:, :, None]).reshape(r, c)
     return codes, scale, scale_inv
 
 
-def quantize_128x128(w_bits: np.ndarray):
+def quantize_128x128(w_bits: np.ndarray, pow2: bool = False):
     """128x128 blocks.  w[R, C] (both % 128 == 0) -> codes[R, C], scale/scale_inv[R/128, C/128]."""
     w = bf16_bits_to_f32(w_bits)
     r, c = w.shape
@@ -187,12 +200,12 @@ def quantize_128x128(w_bits: np.ndarray):
         raise ValueError(f"shape {w.shape} is not a multiple of {BLOCK} in both dims")
     g = w.reshape(r // BLOCK, BLOCK, c // BLOCK, BLOCK)
     am = amax(g, axis=(1, 3)) if g.size else np.zeros((r // BLOCK, c // BLOCK), np.float32)
-    scale, scale_inv = scales_from_amax(am)
+    scale, scale_inv = scales_from_amax(am, pow2)
     codes = _cast(g, scale[:, None, :, None]).reshape(r, c)
     return codes, scale, scale_inv
 
 
-def quantize_128x1_t(x_bits: np.ndarray):
+def quantize_128x1_t(x_bits: np.ndarray, pow2: bool = False):
     """Transposed re-quantization for wgrad, always from the bf16 source.
 
     x[M, K] (M % 128 == 0) -> codes_t[K, M], scale_t/scale_inv_t[K, M/128], where each scale
@@ -204,7 +217,7 @@ def quantize_128x1_t(x_bits: np.ndarray):
         raise ValueError(f"row count {m} is not a multiple of {BLOCK}")
     g = x.reshape(m // BLOCK, BLOCK, k)
     am = amax(g, axis=1) if g.size else np.zeros((m // BLOCK, k), np.float32)   # [M/128, K]
-    scale, scale_inv = scales_from_amax(am)
+    scale, scale_inv = scales_from_amax(am, pow2)
     codes = _cast(g, scale[:, None, :]).reshape(m, k)
     return (np.ascontiguousarray(codes.T), np.ascontiguousarray(scale.T),
             np.ascontiguousarray(scale_inv.T))

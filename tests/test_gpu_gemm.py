@@ -200,6 +200,62 @@ def test_blockwise_forward_shapes(gpu, M, N, K, seed):
     assert rel(U.f32(acc), (ref + 1.5).cpu().numpy()) < TOL_F32
 
 
+@pytest.mark.parametrize("M,N,K", [(320, 384, 512), (2500, 7808, 128), (3000, 5248, 256)])
+def test_power_of_two_scales_through_the_matrix_instruction(gpu, M, N, K):
+    """hpfp8_gemm_blockwise_pow2 hands the scales to the matrix instruction as E8M0 block scales.  On
+    integer-valued operands with power-of-two scales every sum is exact, so both forms (128x128 and
+    per-row b scales) must equal the integer matmul and the kernel that scales with FMAs; only the
+    exponent of a scale may matter (mantissa bits set on purpose change nothing)."""
+    import hpfp8
+    rng = np.random.default_rng(M + N)
+    ai = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    bi = rng.integers(-8, 9, size=(N, K)).astype(np.float32)
+    a, b = O.e4m3_encode(ai), O.e4m3_encode(bi)
+    sa = (2.0 ** rng.integers(-3, 4, size=(M, K // 128))).astype(np.float32)
+    sb = (2.0 ** rng.integers(-3, 4, size=(N // 128, K // 128))).astype(np.float32)
+    sbr = (2.0 ** rng.integers(-3, 4, size=(N, K // 128))).astype(np.float32)
+    aq, bq = fp8(a, gpu), fp8(b, gpu)
+    bias = U.randn_bf16((N,), 9, 4.0).to(gpu)
+    for gran, sb_np in ((128, sb), (1, sbr)):
+        plain = hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, out_dtype=torch.float32)
+        got = hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, out_dtype=torch.float32,
+                                   pow2_scales=True)
+        assert torch.equal(got, plain)
+        if M * N * K <= 64 * 1024 * 1024:
+            want, _ = (O.gemm_blockwise if gran == 128 else O.gemm_rowwise_both)(a, sa, b, sb_np)
+            assert np.array_equal(U.f32(got), want)
+        noisy_a = f32t(sa * np.float32(1.5), gpu)          # same exponents, other mantissas
+        assert torch.equal(hpfp8.gemm_blockwise(aq, noisy_a, bq, f32t(sb_np, gpu), sb_gran=gran, out_dtype=torch.float32,
+                                                pow2_scales=True), plain)
+        wide = torch.full((M, N + 16), 7.0, dtype=torch.bfloat16, device=gpu)
+        out = wide[:, 8:8 + N]
+        hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, bias=bias, out=out, pow2_scales=True)
+        assert torch.equal(out, hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, bias=bias))
+        assert bool((wide[:, :8] == 7.0).all()) and bool((wide[:, 8 + N:] == 7.0).all())
+
+
+def test_power_of_two_recipe_on_real_data(gpu):
+    """Quantized with power-of-two scales, the hardware-scaled GEMM agrees with a float64 dequantized
+    matmul like the FMA-scaled one does (forward / dgrad form and wgrad form)."""
+    import hpfp8
+    M, N, K = 1024, 1536, 2048
+    x = U.randn_bf16((M, K), 81, 1.0, 0.001, 50.0).to(gpu)
+    w = U.randn_bf16((N, K), 82, 0.006).to(gpu)
+    xq, sx = hpfp8.quantize_1x128(x, kmajor=True, pow2=True)
+    wq, sw = hpfp8.quantize_128x128(w, pow2=True)
+    ref = ref_f64_torch(xq, sx, wq, sw.repeat_interleave(128, dim=0), gpu)
+    y32 = hpfp8.gemm_blockwise(xq, sx, wq, sw, out_dtype=torch.float32, pow2_scales=True)
+    assert rel(U.f32(y32), ref.cpu().numpy()) < TOL_F32
+    assert rel(U.f32(hpfp8.gemm_blockwise(xq, sx, wq, sw, pow2_scales=True)), ref.cpu().numpy()) < TOL_BF16
+    assert rel(U.f32(y32), (x.double() @ w.double().t()).cpu().numpy()) < 0.06       # against the unquantized product
+    xt, sxt = hpfp8.quantize_128x1_t(x, kmajor=True, pow2=True)       # [K, M]
+    g = U.randn_bf16((M, N), 83, 1e-3).to(gpu)
+    gt, sgt = hpfp8.quantize_128x1_t(g, kmajor=True, pow2=True)       # [N, M]
+    refw = ref_f64_torch(gt, sgt, xt, sxt, gpu)
+    dw = hpfp8.gemm_blockwise(gt, sgt, xt, sxt, sb_gran=1, out_dtype=torch.float32, pow2_scales=True)
+    assert rel(U.f32(dw), refw.cpu().numpy()) < TOL_F32
+
+
 def test_repeated_launches_give_identical_bits(gpu):
     """The kernels synchronise their LDS buffers by hand (counted waits and one barrier per k-block); a
     missing wait would show as launches of the same problem that differ now and then.  Every form,

@@ -17,7 +17,7 @@ def rel(a, b):
     return np.linalg.norm(a - b) / np.linalg.norm(b)
 
 
-@pytest.mark.parametrize("recipe", ["blockwise", "per_tensor"])
+@pytest.mark.parametrize("recipe", ["blockwise", "per_tensor", "blockwise_pow2"])
 def test_forward_backward_vs_f_linear(gpu, recipe):
     import hpfp8
     x = U.randn_bf16((4, 128, 512), 1).to(gpu).requires_grad_(True)
@@ -155,7 +155,7 @@ def test_weight_gradient_onto_fp32_main_grad(gpu):
         hpfp8.fp8_linear(x, w, recipe="per_tensor", apply_grad_on_fp32_main_grad=True)
 
 
-@pytest.mark.parametrize("recipe", ["blockwise", "per_tensor"])
+@pytest.mark.parametrize("recipe", ["blockwise", "per_tensor", "blockwise_pow2"])
 def test_forward_replays_from_a_captured_graph(gpu, recipe):
     """Every entry point only enqueues kernels on the stream it is given (no allocation, no
     synchronisation, no memset), so a forward pass can be captured into a graph; each replay, with

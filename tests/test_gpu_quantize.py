@@ -104,6 +104,37 @@ def test_seeded_parity_all_quantizers(gpu, shape, seed, std, of, om):
             assert (si1.stride(0) == 1) == kmajor and (sit2.stride(0) == 1) == kmajor
 
 
+@pytest.mark.parametrize("shape,seed,std,of,om", [
+    ((512, 7168), 2, 1.0, 0.001, 50.0),
+    ((384, 640), 3, 0.006, 0.0, 1.0),
+    ((128, 128), 4, 1e-4, 1e-3, 1e3),
+    ((256, 256), 5, 1e30, 0.0, 1.0),
+])
+def test_power_of_two_scale_quantizers(gpu, shape, seed, std, of, om):
+    """The optional recipe with scale_inv rounded up to a power of two: codes and scales of all four
+    entry points bit for bit against the oracle."""
+    import hpfp8
+    x = U.randn_bf16(shape, seed, std, of, om)
+    x[0, :128] = 0                                   # an all-zero group
+    xb = U.bits(x)
+    xg = x.to(gpu)
+    q, s, si = hpfp8.quantize_1x128(xg, want_scale=True, kmajor=True, pow2=True)
+    rq, rs, rsi = O.quantize_1x128(xb, pow2=True)
+    assert np.array_equal(U.codes(q), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    assert not (U.f32_bits(U.f32(si)) & 0x007FFFFF).any()
+    q, si, qt, s = hpfp8.quantize_128x128(xg, with_transpose=True, want_scale=True, pow2=True)
+    rqw, rsw, rsiw = O.quantize_128x128(xb, pow2=True)
+    assert np.array_equal(U.codes(q), rqw) and eq_f32(s, rsw) and eq_f32(si, rsiw) and np.array_equal(U.codes(qt), rqw.T)
+    qt, s, si = hpfp8.quantize_128x1_t(xg, want_scale=True, kmajor=True, pow2=True)
+    rqt, rst, rsit = O.quantize_128x1_t(xb, pow2=True)
+    assert np.array_equal(U.codes(qt), rqt) and eq_f32(s, rst) and eq_f32(si, rsit)
+    q1, si1, qt2, sit2 = hpfp8.quantize_1x128_and_128x1_t(xg, kmajor=True, pow2=True)
+    assert np.array_equal(U.codes(q1), rq) and eq_f32(si1, rsi)
+    assert np.array_equal(U.codes(qt2), rqt) and eq_f32(sit2, rsit)
+    with pytest.raises(ValueError):
+        hpfp8.quantize_1x128(xg, pow2=True)          # only the k-block-major layout
+
+
 @pytest.mark.parametrize("shape", [(512, 7168), (100, 384), (16, 128), (33, 640)])
 def test_kmajor_scale_layouts_hold_the_same_values(gpu, shape):
     import hpfp8

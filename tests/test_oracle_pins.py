@@ -112,6 +112,54 @@ def test_scales_closed_form_and_special_cases():
     assert si7 == np.float32(a / np.float32(448.0)) and si7 != np.float32(np.float32(1.0) / s7)
 
 
+def test_pow2_scales_closed_form():
+    """The optional power-of-two recipe: scale_inv is the smallest power of two that is not below
+    amax_c / 448 (as the fp32 quotient), scale is its exact reciprocal, and no value of the group can
+    come out beyond 448.  Checked with exact arithmetic (math.frexp / Fraction), not with the bit trick."""
+    import math
+    from fractions import Fraction
+    rng = np.random.default_rng(5)
+    am = np.concatenate([
+        np.array([0.0, 1e-13, 1e-12, 1.0, 448.0, 450.0, 446.0, 224.0, 896.0, 1.2e-38, 3.3895e38], np.float32),
+        (448.0 * 2.0 ** rng.integers(-40, 41, size=40)).astype(np.float32),            # exact powers of two times 448
+        np.exp(rng.uniform(-60, 60, size=2000)).astype(np.float32),
+    ])
+    am = U.from_bits(U.bits(torch.from_numpy(am).to(torch.bfloat16))).float().numpy()   # amax of bf16 data is a bf16 value
+    s, si = O.scales_from_amax(am, pow2=True)
+    _, q = O.scales_from_amax(am)
+    for a, sv, siv, qv in zip(am, s, si, q):
+        mant, _ = math.frexp(float(siv))
+        assert mant == 0.5                                      # a power of two
+        assert Fraction(float(siv)) >= Fraction(float(qv)) and Fraction(float(siv)) < 2 * Fraction(float(qv))
+        assert Fraction(float(sv)) * Fraction(float(siv)) == 1
+        assert Fraction(float(a)) * Fraction(float(sv)) <= 448  # exact product: the clamp never acts
+    assert si[4] == 1.0 and si[5] == 2.0 and si[6] == 1.0 and si[7] == 0.5 and si[8] == 2.0
+    assert si[0] == si[1] == si[2] == np.float32(2.0 ** -48)    # eps clamp: 1e-12 / 448 = 2.23e-15 -> 2^-48
+
+
+def test_pow2_quantizers_are_the_ordinary_ones_with_that_scale():
+    x = U.randn_bf16((128, 256), seed=23, outlier_frac=0.01, outlier_mul=50.0)
+    x[:6, :128] = U.special_bf16_rows(128)[:6]
+    xb = U.bits(x)
+    xf = x.float().numpy()
+    q, s, si = O.quantize_1x128(xb, pow2=True)
+    for r in (0, 1, 2, 3, 4, 5, 77, 127):
+        for g in range(2):
+            blk = xf[r, g * 128:(g + 1) * 128]
+            sv, siv = O.scales_from_amax(np.max(np.abs(blk)), pow2=True)
+            want = torch_encode(np.clip(blk * sv, -448.0, 448.0).astype(np.float32))
+            assert np.array_equal(q[r, g * 128:(g + 1) * 128], want) and s[r, g] == sv and si[r, g] == siv
+    qw, sw, siw = O.quantize_128x128(xb, pow2=True)
+    for g in range(2):
+        blk = xf[:, g * 128:(g + 1) * 128]
+        sv, siv = O.scales_from_amax(np.max(np.abs(blk)), pow2=True)
+        assert np.array_equal(qw[:, g * 128:(g + 1) * 128], torch_encode(np.clip(blk * sv, -448.0, 448.0).astype(np.float32)))
+        assert sw[0, g] == sv and siw[0, g] == siv
+    qt, st, sit = O.quantize_128x1_t(xb, pow2=True)
+    q2, s2, si2 = O.quantize_1x128(U.bits(x.t().contiguous()), pow2=True)
+    assert np.array_equal(qt, q2) and np.array_equal(st, s2) and np.array_equal(sit, si2)
+
+
 def test_amax_brute_force():
     x = U.randn_bf16((7, 33), seed=11)
     xf = x.float().numpy()
