@@ -144,6 +144,18 @@ def other_configs(dev):
     ms_bf16 = _time(lambda: _step(lambda: F.linear(xt_, wt_)), iters=20, warm=30)
     res["cfg2_training_step"] = {"fp8_linear_fwd_bwd_ms": ms_fp8, "torch_bf16_linear_fwd_bwd_ms": ms_bf16,
                                  "TFLOP/s": 3 * 2.0 * 4096 * 36864 * 7168 / ms_fp8 / 1e9}
+    # the optional recipe with power-of-two scales (not the benchmarked one): the matrix instruction applies the
+    # scales itself; same tensors, quantized with that recipe
+    wf2_ = hpfp8.quantize_weight(wt_.detach(), pow2=True)
+    ms_p2 = _time(lambda: _step(lambda: hpfp8.fp8_linear(xt_, wt_, recipe="blockwise_pow2", weight_fp8=wf2_)), iters=20, warm=30)
+    xq2_, sx2_ = hpfp8.quantize_1x128(xt_.detach(), kmajor=True, pow2=True)
+    fl2 = 2.0 * 4096 * 36864 * 7168
+    res["recipe_blockwise_pow2"] = {
+        "cfg2_forward_gemm": tf(fl2, _time(lambda: hpfp8.gemm_blockwise(xq2_, sx2_, wf2_.codes, wf2_.scale_inv, pow2_scales=True))),
+        "cfg2_training_step_fwd_bwd_ms": ms_p2,
+        "cfg2_training_step_TFLOP/s": 3 * fl2 / ms_p2 / 1e9,
+    }
+    del wf2_, xq2_, sx2_
     del xt_, wt_, got_, wf_
     torch.cuda.empty_cache()
     # cfg 3: o_proj backward
@@ -171,6 +183,15 @@ def other_configs(dev):
         "dgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq, sgo, wqt, sw.t()))),
         "wgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1))),
     }
+    got2, sgot2 = hpfp8.quantize_128x1_t(go, kmajor=True, pow2=True)
+    xt2, sxt2 = hpfp8.quantize_128x1_t(x, kmajor=True, pow2=True)
+    goq2, sgo2 = hpfp8.quantize_1x128(go, kmajor=True, pow2=True)
+    wq2, sw2, wqt2 = hpfp8.quantize_128x128(w, with_transpose=True, pow2=True)
+    res.setdefault("recipe_blockwise_pow2", {}).update({
+        "cfg3_dgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq2, sgo2, wqt2, sw2.t(), pow2_scales=True))),
+        "cfg3_wgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(got2, sgot2, xt2, sxt2, sb_gran=1, pow2_scales=True))),
+    })
+    del got2, xt2, goq2, wq2, wqt2
     # the same weight gradient added onto an fp32 main gradient (apply_grad_on_fp32_main_grad)
     main_grad = torch.zeros((n, k), dtype=torch.float32, device=dev)
     res["cfg3_backward"]["wgrad_gemm_into_fp32_main_grad"] = tf(
