@@ -219,6 +219,11 @@ def other_configs(dev):
     ms = _time(lambda: hpfp8.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // 128, k // 128), offs), iters=5)
     res["cfg4_moe_grouped"] = dict(tf(2.0 * total * n * k, ms), rows=total, experts=e,
                                    min_rows=int(counts.min()), max_rows=int(counts.max()))
+    sx2 = torch.exp2(torch.ceil(torch.log2(sx)))           # (timing only: the same codes under power-of-two scales)
+    sw2 = torch.exp2(torch.ceil(torch.log2(sw)))
+    ms2 = _time(lambda: hpfp8.gemm_grouped_blockwise(xq, sx2, wq.view(e, n, k), sw2.view(e, n // 128, k // 128), offs,
+                                                     pow2_scales=True), iters=5)
+    res.setdefault("recipe_blockwise_pow2", {})["cfg4_moe_grouped_gemm"] = tf(2.0 * total * n * k, ms2)
     del xq, sx, wq, sw
     torch.cuda.empty_cache()
     # cfg 5: gradient bucket, 2^29 elements

@@ -853,10 +853,10 @@ int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const
   return launch<kScaleTensor, false>(p, out_type, tiles, (hipStream_t)stream);
 }
 
-int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
-                                 const void* b, const float* sb, const int32_t* offs, int experts,
-                                 int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
-                                 hpfp8_stream_t stream) {
+static int gemm_grouped_impl(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                             const void* b, const float* sb, const int32_t* offs, int experts,
+                             int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type, bool pow2,
+                             hpfp8_stream_t stream) {
   HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "gemm_grouped: bad expert count %d", experts);
   int rc = check_common("gemm_grouped", a, lda, b, K, sa, sb, total_m, N, K, nullptr, c, ldc, out_type, 0);
   if (rc <= 0) return rc;
@@ -874,7 +874,24 @@ int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, in
   p.M = (int)total_m; p.N = (int)N; p.K = (int)K;
   // upper bound on row tiles: every expert may add one partial tile
   const int64_t tiles = (total_m / BM + experts) * ((N + BN - 1) / BN);
+  if (pow2) return launch<kScalePow2, true>(p, out_type, tiles, (hipStream_t)stream);
   return launch<kScaleBlock, true>(p, out_type, tiles, (hipStream_t)stream);
+}
+
+int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                                 const void* b, const float* sb, const int32_t* offs, int experts,
+                                 int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
+                                 hpfp8_stream_t stream) {
+  return gemm_grouped_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, sb, offs, experts, total_m, N, K, c, ldc, out_type,
+                           false, stream);
+}
+
+int hpfp8_gemm_grouped_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m,
+                                      int64_t sa_stride_k, const void* b, const float* sb, const int32_t* offs,
+                                      int experts, int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc,
+                                      int out_type, hpfp8_stream_t stream) {
+  return gemm_grouped_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, sb, offs, experts, total_m, N, K, c, ldc, out_type,
+                           true, stream);
 }
 
 }  // extern "C"

@@ -47,6 +47,8 @@ SIGNATURES = {
     "hpfp8_gemm_per_tensor": [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _int, _vp],
     "hpfp8_gemm_grouped_blockwise": [_vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _i64,
                                      _int, _vp],
+    "hpfp8_gemm_grouped_blockwise_pow2": [_vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _i64,
+                                          _int, _vp],
 }
 
 OUT_BF16, OUT_F32 = 0, 1

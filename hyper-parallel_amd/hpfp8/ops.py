@@ -397,7 +397,8 @@ def gemm_per_tensor(a: torch.Tensor, sa_inv: torch.Tensor, b: torch.Tensor, sb_i
 
 
 def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor,
-                           offs: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+                           offs: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                           pow2_scales: bool = False) -> torch.Tensor:
     """MoE grouped GEMM: rows of a[total_m, K] sorted by expert, offs[E] int32 inclusive prefix sums,
     b[E, N, K], sb[E, N/128, K/128], sa[total_m, K/128] -> c[total_m, N].  Rows past offs[-1] are left
     uninitialised (as torch's grouped matmul leaves them)."""
@@ -421,6 +422,6 @@ def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, s
     if tuple(sb.shape) != (e, n // BLOCK, kb) or not sb.is_contiguous():
         raise ValueError(f"sb must be contiguous [{e}, {n // BLOCK}, {kb}]")
     out = torch.empty((total_m, n), dtype=out_dtype, device=a.device)
-    _lib.call("hpfp8_gemm_grouped_blockwise", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
+    _lib.call("hpfp8_gemm_grouped_blockwise_pow2" if pow2_scales else "hpfp8_gemm_grouped_blockwise", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
               _ptr(offs), e, total_m, n, k, _ptr(out), n, _out_code(out_dtype), _stream())
     return out

@@ -237,6 +237,12 @@ int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, in
                                  int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
                                  hpfp8_stream_t stream);
 
+/* The grouped form for power-of-two scales (see hpfp8_gemm_blockwise_pow2); arguments as above. */
+int hpfp8_gemm_grouped_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m,
+                                      int64_t sa_stride_k, const void* b, const float* sb, const int32_t* offs,
+                                      int experts, int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc,
+                                      int out_type, hpfp8_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

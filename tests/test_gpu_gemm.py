@@ -376,6 +376,19 @@ def test_grouped_against_loop_of_dense(gpu, experts, total, N, K, seed):
                                     swi3[e].repeat_interleave(128, dim=0), gpu)
                 assert rel(U.f32(dense), ref.cpu().numpy()) < TOL_F32
         start += cnt
+    # the same with power-of-two scales handed to the matrix instruction: grouped == loop of dense
+    xq, sxi = hpfp8.quantize_1x128(x, kmajor=True, pow2=True)
+    wq, swi = hpfp8.quantize_128x128(w, pow2=True)
+    wq3, swi3 = wq.view(experts, N, K), swi.view(experts, N // 128, K // 128)
+    y = hpfp8.gemm_grouped_blockwise(xq, sxi, wq3, swi3, offs, out_dtype=torch.float32, pow2_scales=True)
+    start = 0
+    for e in range(experts):
+        cnt = int(counts[e])
+        if cnt:
+            dense = hpfp8.gemm_blockwise(xq[start:start + cnt], sxi[start:start + cnt], wq3[e], swi3[e],
+                                         out_dtype=torch.float32, pow2_scales=True)
+            assert torch.equal(y[start:start + cnt], dense), f"expert {e} (power-of-two scales)"
+        start += cnt
 
 
 def test_grouped_leaves_rows_past_the_last_offset_alone(gpu):
