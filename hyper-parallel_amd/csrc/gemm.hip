@@ -143,7 +143,7 @@ __device__ __forceinline__ int expert_end(int off, int prev, int total_rows) {
 
 template <int MODE, bool GROUPED, bool OUT_F32, bool ACC>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
-  static_assert(!ACC || (OUT_F32 && (MODE == kScaleBlock || MODE == kScaleRow)), "accumulating onto c: fp32 output, promoted sums");
+  static_assert(!ACC || (OUT_F32 && MODE != kScaleTensor), "accumulating onto c: fp32 output, sums that start from c's values");
   constexpr int kBStages = b_stages(MODE);
   constexpr bool kRowScales = MODE == kScaleRow || MODE == kScalePow2Row;   // per-row b scales, staged in LDS
   constexpr bool kPromote = MODE == kScaleBlock || MODE == kScaleRow;       // partial sums scaled by FMAs
@@ -727,7 +727,7 @@ template <int MODE, bool GROUPED>
 static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
   dim3 grid((unsigned)persistent_grid(tiles)), block(kGemmThreads);
   if (out_type == HPFP8_OUT_F32) {
-    if constexpr ((MODE == kScaleBlock || MODE == kScaleRow) && !GROUPED) {   // (the per-tensor and grouped entry points have no accumulate)
+    if constexpr (MODE != kScaleTensor && !GROUPED) {   // (the per-tensor and grouped entry points have no accumulate)
       if (p.accumulate) {
         gemm_kernel<MODE, GROUPED, true, true><<<grid, block, 0, stream>>>(p);
         return check_launch("gemm");
@@ -806,7 +806,6 @@ static int gemm_blockwise_impl(const void* a, int64_t lda, const float* sa, int6
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.accumulate = accumulate;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   p.tiles = (int)tiles;
-  HPFP8_REQUIRE(!pow2 || !accumulate, HPFP8_ERR_ARG, "gemm_blockwise_pow2: no accumulate form");
   if (sb_gran == 128) {
     if (pow2) return launch<kScalePow2, false>(p, out_type, tiles, (hipStream_t)stream);
     return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
@@ -834,9 +833,9 @@ int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa
 int hpfp8_gemm_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                               const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
                               int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
-                              int out_type, hpfp8_stream_t stream) {
+                              int out_type, int accumulate, hpfp8_stream_t stream) {
   return gemm_blockwise_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, ldb, sb, sb_stride_n, sb_stride_k, sb_gran, M, N, K,
-                             bias, c, ldc, out_type, 0, true, stream);
+                             bias, c, ldc, out_type, accumulate, true, stream);
 }
 
 int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,

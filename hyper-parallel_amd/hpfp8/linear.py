@@ -118,9 +118,10 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
                 # the fp32 main gradient of hyper_parallel/platform/torch/fully_shard/param.py:134-167: the
                 # first weight gradient creates it, later ones are added onto it by the GEMM itself, and
                 # .grad stays empty
-                param.main_grad = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out_dtype=torch.float32)
+                param.main_grad = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out_dtype=torch.float32,
+                                                     pow2_scales=pow2)
             else:
-                ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=param.main_grad, accumulate=True)
+                ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=param.main_grad, accumulate=True, pow2_scales=pow2)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
         return dx, dw, db, None, None, None, None, None
@@ -190,8 +191,8 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
             raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
     pow2 = recipe == "blockwise_pow2"
     if apply_grad_on_fp32_main_grad:
-        if recipe != "blockwise":
-            raise ValueError("apply_grad_on_fp32_main_grad is only implemented for the blockwise recipe")
+        if recipe == "per_tensor":
+            raise ValueError("apply_grad_on_fp32_main_grad is only implemented for the blockwise recipes")
         mg = getattr(weight, "main_grad", None)
         if mg is not None and (mg.dtype != torch.float32 or tuple(mg.shape) != tuple(weight.shape) or
                                not mg.is_contiguous()):

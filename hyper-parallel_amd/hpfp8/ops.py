@@ -358,15 +358,8 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
         out_dtype = out.dtype
     if accumulate and out_dtype != torch.float32:
         raise ValueError("accumulate needs a float32 output")
-    if pow2_scales:
-        if accumulate:
-            raise ValueError("pow2_scales has no accumulate form")
-        _lib.call("hpfp8_gemm_blockwise_pow2", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ld(b),
-                  _ptr(sb), sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
-                  out.stride(0) if m > 1 else n, _out_code(out_dtype), _stream())
-        return out
-    _lib.call("hpfp8_gemm_blockwise", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ld(b),
-              _ptr(sb), sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
+    _lib.call("hpfp8_gemm_blockwise_pow2" if pow2_scales else "hpfp8_gemm_blockwise", _ptr(a), _ld(a), _ptr(sa),
+              sa.stride(0), sa.stride(1), _ptr(b), _ld(b), _ptr(sb), sb.stride(0), sb.stride(1), sb_gran, m, n, k, _ptr(bias), _ptr(out),
               out.stride(0) if m > 1 else n, _out_code(out_dtype), int(accumulate), _stream())
     return out
 

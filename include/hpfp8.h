@@ -212,13 +212,13 @@ int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa
 /* hpfp8_gemm_blockwise for scales that are powers of two (what the _pow2 quantizers write): the matrix
  * instruction applies them as E8M0 block scales and sums the k-blocks itself, so the kernel spends no
  * arithmetic on scaling.  Only the exponent field of a scale is used (mantissa bits are ignored, the
- * sign must be +).  Same arguments and limits as hpfp8_gemm_blockwise, without accumulate.  Results
+ * sign must be +).  Same arguments and limits as hpfp8_gemm_blockwise.  Results
  * agree with hpfp8_gemm_blockwise on the same operands to fp32 rounding (the order of the fp32
  * additions differs), and are exact on the same integer-valued cases. */
 int hpfp8_gemm_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                               const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
                               int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
-                              int out_type, hpfp8_stream_t stream);
+                              int out_type, int accumulate, hpfp8_stream_t stream);
 
 /* Per-tensor scales: c = (a . b^T) * (sa_inv[0] * sb_inv[0]) (+ bias), accumulation over the whole
  * K inside the matrix cores.  K a multiple of 128, N a multiple of 128. */

@@ -227,6 +227,10 @@ def test_power_of_two_scales_through_the_matrix_instruction(gpu, M, N, K):
         noisy_a = f32t(sa * np.float32(1.5), gpu)          # same exponents, other mantissas
         assert torch.equal(hpfp8.gemm_blockwise(aq, noisy_a, bq, f32t(sb_np, gpu), sb_gran=gran, out_dtype=torch.float32,
                                                 pow2_scales=True), plain)
+        old = torch.from_numpy(rng.integers(-1000, 1001, size=(M, N)).astype(np.float32)).to(gpu)
+        c = old.clone()
+        hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, out=c, accumulate=True, pow2_scales=True)
+        assert torch.equal(c, old + plain)
         wide = torch.full((M, N + 16), 7.0, dtype=torch.bfloat16, device=gpu)
         out = wide[:, 8:8 + N]
         hpfp8.gemm_blockwise(aq, f32t(sa, gpu), bq, f32t(sb_np, gpu), sb_gran=gran, bias=bias, out=out, pow2_scales=True)

@@ -153,6 +153,12 @@ def test_weight_gradient_onto_fp32_main_grad(gpu):
     assert rel(mod.weight.main_grad, 2 * ref_mod.weight.grad.double()) < 3e-3
     with pytest.raises(ValueError):
         hpfp8.fp8_linear(x, w, recipe="per_tensor", apply_grad_on_fp32_main_grad=True)
+    # the power-of-two recipe accumulates the same way
+    w.main_grad = None
+    hpfp8.fp8_linear(x, w, recipe="blockwise_pow2", apply_grad_on_fp32_main_grad=True).backward(go1)
+    once = w.main_grad.clone()
+    hpfp8.fp8_linear(x, w, recipe="blockwise_pow2", apply_grad_on_fp32_main_grad=True).backward(go1)
+    assert w.grad is None and rel(w.main_grad, 2 * once.double()) < 1e-6 and rel(once, grads[0][1]) < 0.1
 
 
 @pytest.mark.parametrize("recipe", ["blockwise", "per_tensor", "blockwise_pow2"])
