@@ -17,6 +17,10 @@
 //   * The grid is persistent: one workgroup per CU walks a list of tiles, and the rounds of
 //     consecutive tiles follow each other without a gap.  Each XCD (own L2) owns a contiguous run
 //     of tile numbers.
+//   * One kernel template, by scale form: per tensor, 128x128 blocks of b (forward, dgrad), per-row
+//     scales on both operands (wgrad), and the two blockwise forms again for scales that are powers of
+//     two, which the matrix instruction applies itself (no promotion FMAs); dense or grouped by expert;
+//     bf16 or fp32 output, optionally added onto what c holds.
 #include <type_traits>
 
 #include "hpfp8_device.h"
