@@ -197,7 +197,8 @@ template <bool KMAJOR>
 __global__ __launch_bounds__(256) void swiglu_quant_1x128_kernel(const uint16_t* __restrict__ h, int64_t ld,
                                                                  uint8_t* __restrict__ q, float* __restrict__ scale,
                                                                  float* __restrict__ scale_inv,
-                                                                 uint16_t* __restrict__ act, int rows, int inter) {
+                                                                 uint16_t* __restrict__ act, int rows, int inter,
+                                                                 int pow2) {
   const int groups = inter >> 7;
   const int gtiles = (groups + 3) >> 2;
   const int g0 = (blockIdx.x % gtiles) * 4, row0 = (blockIdx.x / gtiles) * 16;
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(256) void swiglu_quant_1x128_kernel(const uint16_t*
     a.w = swiglu2(vg[u].w, vu[u].w);
     const uint32_t m = row16_max_u32(mag8(a));
     float s, si;
-    scales_from_amax(__uint_as_float(m << 16), s, si);
+    scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
     if (ok) {
       const int64_t o = (int64_t)row * inter + (g0 + u) * 128 + l16 * 8;
       nt_store8(q + o, cvt8<false>(a, s));
@@ -789,8 +790,8 @@ int hpfp8_quantize_1x128_and_128x1_t_pow2_bf16(const void* x, int64_t m, int64_t
                                stream, q, scale, scale_inv, 1);
 }
 
-int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
-                                     float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
+static int swiglu_quantize_impl(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
+                                float* scale, float* scale_inv, void* act, int pow2, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: negative shape");
   HPFP8_REQUIRE(inter % kBlock == 0, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: width %lld is not a multiple of 128",
                 (long long)inter);
@@ -807,11 +808,21 @@ int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter,
   hipStream_t s = (hipStream_t)stream;
   if (kmajor)
     swiglu_quant_1x128_kernel<true><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)h, ld_h, (uint8_t*)q, scale, scale_inv,
-                                                                     (uint16_t*)act, (int)rows, (int)inter);
+                                                                     (uint16_t*)act, (int)rows, (int)inter, pow2);
   else
     swiglu_quant_1x128_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)h, ld_h, (uint8_t*)q, scale, scale_inv,
-                                                                      (uint16_t*)act, (int)rows, (int)inter);
+                                                                      (uint16_t*)act, (int)rows, (int)inter, pow2);
   return check_launch("swiglu_quantize_1x128");
+}
+
+int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
+                                     float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
+  return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, 0, stream);
+}
+
+int hpfp8_swiglu_quantize_1x128_pow2_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
+                                          float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
+  return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, 1, stream);
 }
 
 int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld, void* q_t, int64_t ld_t,

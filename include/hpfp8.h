@@ -124,6 +124,8 @@ int hpfp8_quantize_128x1_t_kmajor_pow2_bf16(const void* x, int64_t m, int64_t k,
 int hpfp8_quantize_1x128_and_128x1_t_pow2_bf16(const void* x, int64_t m, int64_t k, int kmajor, void* q, float* scale,
                                                float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
                                                float* scale_inv_t, hpfp8_stream_t stream);
+int hpfp8_swiglu_quantize_1x128_pow2_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
+                                          float* scale, float* scale_inv, void* act, hpfp8_stream_t stream);
 
 /* SwiGLU fused with the 1x128 quantization of its result, the activations of the down projection
  * (the step after the gate/up linear of a DeepSeekV3 MLP; in the reference this is eager

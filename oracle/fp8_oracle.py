@@ -297,10 +297,10 @@ def swiglu(h_bits: np.ndarray) -> np.ndarray:
     return f32_to_bf16_bits((s * u).astype(np.float32))
 
 
-def swiglu_quantize_1x128(h_bits: np.ndarray):
+def swiglu_quantize_1x128(h_bits: np.ndarray, pow2: bool = False):
     """(codes, scale, scale_inv, act bits) of the SwiGLU result quantized in 1x128 groups."""
     act = swiglu(h_bits)
-    codes, scale, scale_inv = quantize_1x128(act)
+    codes, scale, scale_inv = quantize_1x128(act, pow2)
     return codes, scale, scale_inv, act
 
 

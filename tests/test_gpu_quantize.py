@@ -297,6 +297,10 @@ def test_swiglu_fused_with_quantize(gpu, shape, kmajor):
     wide[:, :w2] = hg
     q2, si2 = hpfp8.swiglu_quantize_1x128(wide[:, :w2], kmajor=kmajor)
     assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(si2, si)
+    # the optional power-of-two scales
+    q3, si3 = hpfp8.swiglu_quantize_1x128(hg, kmajor=kmajor, pow2=True)
+    rq3, _, rsi3, _ = O.swiglu_quantize_1x128(U.bits(h), pow2=True)
+    assert np.array_equal(U.codes(q3), rq3) and np.array_equal(U.f32_bits(U.f32(si3)), U.f32_bits(rsi3))
 
 
 def test_dequantize_accumulate_into_fp32_main_grad(gpu):
