@@ -134,7 +134,16 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
         xq, _, sx = ops.quantize_per_tensor(x2)
         wq, _, sw = ops.quantize_per_tensor(weight)
         y = ops.gemm_per_tensor(xq, sx, wq, sw, bias=bias)
-        ctx.save_for_backward(x2, weight)
+        # With one scale per tensor the codes of a transposed tensor are the transposed codes, so backward
+        # needs no second quantization of x and W: it keeps the codes (1 byte per element) where their
+        # shapes allow the byte transpose, and the bf16 tensors otherwise.
+        m = x2.shape[0]
+        can_t = m % ops.BLOCK == 0 and m > 0
+        ctx.codes_saved = can_t
+        if can_t:
+            ctx.save_for_backward(xq if weight.requires_grad else None, sx, wq if x.requires_grad else None, sw)
+        else:
+            ctx.save_for_backward(x2, weight)
         ctx.x_shape = x.shape
         ctx.has_bias = bias is not None
         ctx.need = (x.requires_grad, weight.requires_grad)
@@ -142,21 +151,29 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_out):
-        x2, weight = ctx.saved_tensors
         need_dx, need_dw = ctx.need
         go = _flatten(grad_out)
         if go.dtype != torch.bfloat16:
             go = go.to(torch.bfloat16)
         go = go.contiguous()
         dx = dw = db = None
-        if need_dx:
+        if ctx.codes_saved:
+            xq, sx, wq, sw = ctx.saved_tensors
             goq, _, sgo = ops.quantize_per_tensor(go)
-            wtq, _, swt = ops.quantize_per_tensor(weight.t().contiguous())
-            dx = ops.gemm_per_tensor(goq, sgo, wtq, swt).reshape(ctx.x_shape)
-        if need_dw:
-            gotq, _, sgot = ops.quantize_per_tensor(go.t().contiguous())
-            xtq, _, sxt = ops.quantize_per_tensor(x2.t().contiguous())
-            dw = ops.gemm_per_tensor(gotq, sgot, xtq, sxt)
+            if need_dx:
+                dx = ops.gemm_per_tensor(goq, sgo, ops.transpose_codes(wq), sw).reshape(ctx.x_shape)
+            if need_dw:
+                dw = ops.gemm_per_tensor(ops.transpose_codes(goq), sgo, ops.transpose_codes(xq), sx)
+        else:
+            x2, weight = ctx.saved_tensors
+            if need_dx:
+                goq, _, sgo = ops.quantize_per_tensor(go)
+                wtq, _, swt = ops.quantize_per_tensor(weight.t().contiguous())
+                dx = ops.gemm_per_tensor(goq, sgo, wtq, swt).reshape(ctx.x_shape)
+            if need_dw:
+                gotq, _, sgot = ops.quantize_per_tensor(go.t().contiguous())
+                xtq, _, sxt = ops.quantize_per_tensor(x2.t().contiguous())
+                dw = ops.gemm_per_tensor(gotq, sgot, xtq, sxt)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
         return dx, dw, db
