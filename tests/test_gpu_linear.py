@@ -234,3 +234,31 @@ def test_fp8_checkpoint_round_trip(gpu, tmp_path):
     w, wd = model[0].weight.detach().float(), clone[0].weight.detach().float()
     amax = w.view(3, 128, 2, 128).abs().amax(dim=(1, 3), keepdim=True)
     assert bool(((w - wd).view(3, 128, 2, 128).abs() <= amax / 28 + amax / 256).all())
+
+
+def test_policy_record_and_fp8_cast_hook(gpu):
+    """The mixed-precision record keeps the reference's fields and defaults; the cast hook behaves like
+    the reference's for ordinary dtypes and returns codes + scale for an E4M3 target (the per-tensor
+    cast of cfg 1, bit for bit against the oracle)."""
+    import hpfp8
+    pol = hpfp8.Fp8MixedPrecisionPolicy()
+    assert (pol.param_dtype, pol.reduce_dtype, pol.output_dtype) == (None, None, None)
+    assert pol.cast_forward_inputs is True and pol.apply_grad_on_fp32_main_grad is False
+    assert pol.linear_kwargs() == {"recipe": "blockwise", "apply_grad_on_fp32_main_grad": False}
+    with pytest.raises(ValueError):
+        hpfp8.Fp8MixedPrecisionPolicy(fp8_recipe="nope")
+    with pytest.raises(ValueError):
+        hpfp8.Fp8MixedPrecisionPolicy(reduce_dtype="float32")
+    x = U.randn_bf16((256, 384), 91).to(gpu)
+    assert hpfp8.cast_fp_tensor(torch.bfloat16, x) is x
+    assert hpfp8.cast_fp_tensor(torch.float32, x).dtype == torch.float32
+    ints = torch.arange(4, device=gpu)
+    assert hpfp8.cast_fp_tensor(torch.float8_e4m3fn, ints) is ints and hpfp8.cast_fp_tensor(torch.float32, "s") == "s"
+    t = hpfp8.cast_fp_tensor(torch.float8_e4m3fn, x)
+    rq, _, rsi = O.quantize_per_tensor(U.bits(x))
+    assert np.array_equal(U.codes(t.codes), rq) and np.array_equal(U.f32_bits(U.f32(t.scale_inv)), U.f32_bits(rsi))
+    assert rel(t.dequantize(torch.float32), x.float()) < 0.05
+    pol = hpfp8.Fp8MixedPrecisionPolicy(apply_grad_on_fp32_main_grad=True, fp8_recipe="blockwise_pow2")
+    w = U.randn_bf16((256, 384), 92, 0.02).to(gpu).requires_grad_(True)
+    hpfp8.fp8_linear(x, w, **pol.linear_kwargs()).backward(U.randn_bf16((256, 256), 93, 1e-3).to(gpu))
+    assert w.grad is None and w.main_grad.dtype == torch.float32
