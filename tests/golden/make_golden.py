@@ -62,6 +62,20 @@ def main():
     np.savez_compressed(os.path.join(HERE, "fp8_path_golden.npz"), **out)
     print("wrote", os.path.join(HERE, "fp8_path_golden.npz"), {k: v.shape for k, v in out.items() if hasattr(v, "shape")})
 
+    # --- the optional recipe with power-of-two scales, on the same tensor (input: x_bits of the file above)
+    p2 = {}
+    q, s, si = O.quantize_1x128(xb, pow2=True)
+    p2["g1x128_codes"], p2["g1x128_scale"], p2["g1x128_scale_inv"] = q, s, si
+    q, s, si = O.quantize_128x128(xb, pow2=True)
+    p2["b128_codes"], p2["b128_scale"], p2["b128_scale_inv"] = q, s, si
+    q, s, si = O.quantize_128x1_t(xb, pow2=True)
+    p2["t128x1_codes"], p2["t128x1_scale"], p2["t128x1_scale_inv"] = q, s, si
+    aq, _, asi = O.quantize_1x128(U.bits(a), pow2=True)
+    wq, _, wsi = O.quantize_128x128(U.bits(w), pow2=True)
+    p2["gemm_y_f32"], _ = O.gemm_blockwise(aq, asi, wq, wsi, O.bf16_bits_to_f32(U.bits(bias)))
+    np.savez_compressed(os.path.join(HERE, "fp8_pow2_golden.npz"), **p2)
+    print("wrote", os.path.join(HERE, "fp8_pow2_golden.npz"), {k: v.shape for k, v in p2.items()})
+
 
 if __name__ == "__main__":
     torch.manual_seed(0)

@@ -58,6 +58,13 @@ def test_golden_fixtures(gpu):
     assert np.array_equal(U.codes(c), G["bucket_codes"]) and eq_f32(si, G["bucket_scale_inv"])
     back = hpfp8.dequantize_bucket(c, si, grad_scale=0.125)
     assert np.array_equal(U.bits(back), G["bucket_back_bits"])
+    P = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fp8_pow2_golden.npz"))
+    q, s, si = hpfp8.quantize_1x128(x, want_scale=True, kmajor=True, pow2=True)
+    assert np.array_equal(U.codes(q), P["g1x128_codes"]) and eq_f32(s, P["g1x128_scale"]) and eq_f32(si, P["g1x128_scale_inv"])
+    q, si, qt, s = hpfp8.quantize_128x128(x, with_transpose=True, want_scale=True, pow2=True)
+    assert np.array_equal(U.codes(q), P["b128_codes"]) and eq_f32(s, P["b128_scale"]) and eq_f32(si, P["b128_scale_inv"])
+    qt, s, si = hpfp8.quantize_128x1_t(x, want_scale=True, kmajor=True, pow2=True)
+    assert np.array_equal(U.codes(qt), P["t128x1_codes"]) and eq_f32(s, P["t128x1_scale"]) and eq_f32(si, P["t128x1_scale_inv"])
 
 
 @pytest.mark.parametrize("shape,seed,std,of,om", [
