@@ -145,7 +145,9 @@ __device__ __forceinline__ int expert_end(int off, int prev, int total_rows) {
   return lo < total_rows ? lo : total_rows;
 }
 
-template <int MODE, bool GROUPED, bool OUT_F32, bool ACC>
+// SA4: the activation scales have unit stride over rows (the k-block-major layout), so a lane's four
+// of them are one 16-byte load.
+template <int MODE, bool GROUPED, bool OUT_F32, bool ACC, bool SA4>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
   static_assert(!ACC || (OUT_F32 && MODE != kScaleTensor), "accumulating onto c: fp32 output, sums that start from c's values");
   constexpr int kBStages = b_stages(MODE);
@@ -267,7 +269,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     const int q = wave * 4 + i;                       // 8-row group inside the tile
     const int r = q * 8 + (lane >> 3);                // row inside the tile
     const int chunk = (lane & 7) ^ row_swizzle(r);    // logical 16-byte chunk of that row
-    a_off[i] = (uint32_t)r * (uint32_t)p.lda + chunk * 16;
+    // The rows of the a tile are permuted on their way into LDS: LDS row 64 w + 16 j + l holds tile row
+    // 64 w + 4 l + j.  The lane that owns LDS rows 16 j + l16 (j = 0..3) of its wave's 64 then owns four
+    // consecutive rows of a, whose scales are one 16-byte load and whose results are four adjacent
+    // rows of c.  (The b tile keeps its order.)
+    const int ra = (r & ~63) + (r & 15) * 4 + ((r >> 4) & 3);
+    a_off[i] = (uint32_t)ra * (uint32_t)p.lda + chunk * 16;
     b_off[i] = (uint32_t)r * (uint32_t)p.ldb + chunk * 16;
   }
   // wgrad form: the 256 per-row scales of the b tile for one k-block are one more 1 KB transfer
@@ -310,14 +317,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       (void*)p.sa, 0, MODE == kScaleTensor ? 4 : (int)((((int64_t)p.M - 1) * p.sa_sm + ((int64_t)kblocks - 1) * p.sa_sk + 1) * 4),
       0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_sbb = __builtin_amdgcn_make_buffer_rsrc((void*)p.sb, 0, p.sb_bytes, 0x00020000);
-  uint32_t sa_voff[4];         // byte offset of this lane's four rows in sa
+  uint32_t sa_voff[4];         // byte offset of this lane's four rows in sa (SA4: [0] covers all four)
   int sb_soff = 0;             // block form: byte offset of the b tile's scale row
   const int sa_kstep = (int)p.sa_sk * 4, sb_kstep = (int)p.sb_sk * 4;
   auto scale_target = [&](const TileInfo& ti) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int r = ti.row0 + wm * 64 + j * 16 + l16;
-      sa_voff[j] = (uint32_t)(r < p.M ? r : p.M - 1) * (uint32_t)((int)p.sa_sm * 4);
+      const int r = ti.row0 + wm * 64 + l16 * 4 + j;
+      // (SA4 does not clamp: words past the end of the array read as zero, and rows past M are never stored)
+      sa_voff[j] = SA4 ? (uint32_t)r * 4u : (uint32_t)(r < p.M ? r : p.M - 1) * (uint32_t)((int)p.sa_sm * 4);
     }
     int nblk_idx = (ti.n0 + wn * 128) >> 7;
     if (nblk_idx > (N >> 7) - 1) nblk_idx = (N >> 7) - 1;
@@ -327,9 +335,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     if (MODE == kScaleBlock || MODE == kScalePow2)
       raw[4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sbb, 0, sb_soff + kb * sb_kstep, 0));
     if (MODE != kScaleTensor) {
+      if (SA4) {
+        const v4f four = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc_sa, sa_voff[0], kb * sa_kstep, 0));
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        raw[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, sa_voff[j], kb * sa_kstep, 0));
+        for (int j = 0; j < 4; ++j) raw[j] = four[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          raw[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, sa_voff[j], kb * sa_kstep, 0));
+      }
     }
   };
   // kScalePow2: the exponent fields of the scales of the current k-block, which are their E8M0 codes:
@@ -359,7 +373,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     const float* base = reinterpret_cast<const float*>(p.c) + (ok ? (int64_t)ti.row0 * p.ldc + ncol : 0);
     return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
   };
-  const int c_jstep = 16 * (int)p.ldc * 4;                     // bytes between the rows of subtiles j and j + 1
+  const int c_jstep = (int)p.ldc * 4;                          // bytes between the rows of subtiles j and j + 1
   auto old_values = [&](const __amdgpu_buffer_rsrc_t& rs, uint32_t lane_off, int i, int j) {
     return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off + i * 64, j * c_jstep, 0));
   };
@@ -369,7 +383,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     int lane_c = lane;
     asm volatile("" : "+v"(lane_c));    // (keeps the lane offset out of the registers held through the rounds)
     const __amdgpu_buffer_rsrc_t rc = rsrc_c_of(ti);
-    const uint32_t c_lane = ((uint32_t)(wm * 64 + (lane_c & 15)) * (uint32_t)p.ldc + (lane_c >> 4) * 4) * 4u;
+    const uint32_t c_lane = ((uint32_t)(wm * 64 + (lane_c & 15) * 4) * (uint32_t)p.ldc + (lane_c >> 4) * 4) * 4u;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
@@ -672,7 +686,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
           }
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
-            const int m = row0 + wm * 64 + j * 16 + 4 * (k2 + k) + ge;
+            const int m = row0 + wm * 64 + (4 * (k2 + k) + ge) * 4 + j;     // staging row s of pass j is tile row 4 s + j
             if (decltype(full_rows)::value || m < row_end) {
               if (OUT_F32) {
                 float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.c) + (int64_t)m * p.ldc + ncol + h * 64 + l16e * 4);
@@ -727,21 +741,29 @@ static int persistent_grid(int64_t tiles) {
   return (int)g;
 }
 
-template <int MODE, bool GROUPED>
-static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
+template <int MODE, bool GROUPED, bool SA4>
+static int launch_sa(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
   dim3 grid((unsigned)persistent_grid(tiles)), block(kGemmThreads);
   if (out_type == HPFP8_OUT_F32) {
     if constexpr (MODE != kScaleTensor && !GROUPED) {   // (the per-tensor and grouped entry points have no accumulate)
       if (p.accumulate) {
-        gemm_kernel<MODE, GROUPED, true, true><<<grid, block, 0, stream>>>(p);
+        gemm_kernel<MODE, GROUPED, true, true, SA4><<<grid, block, 0, stream>>>(p);
         return check_launch("gemm");
       }
     }
-    gemm_kernel<MODE, GROUPED, true, false><<<grid, block, 0, stream>>>(p);
+    gemm_kernel<MODE, GROUPED, true, false, SA4><<<grid, block, 0, stream>>>(p);
   } else {
-    gemm_kernel<MODE, GROUPED, false, false><<<grid, block, 0, stream>>>(p);
+    gemm_kernel<MODE, GROUPED, false, false, SA4><<<grid, block, 0, stream>>>(p);
   }
   return check_launch("gemm");
+}
+
+template <int MODE, bool GROUPED>
+static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
+  if constexpr (MODE != kScaleTensor) {
+    if (p.sa_sm == 1) return launch_sa<MODE, GROUPED, true>(p, out_type, tiles, stream);
+  }
+  return launch_sa<MODE, GROUPED, false>(p, out_type, tiles, stream);
 }
 
 static int check_common(const char* what, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
