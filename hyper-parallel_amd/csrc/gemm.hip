@@ -619,7 +619,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 #pragma unroll
     for (int j = 0; j < 4; ++j) part_c[j] = zero;
   }
-  // The wave's 64 x 128 results go out 16 rows at a time through its own 4 KB slice of the b buffer
+  // The wave's 64 x 128 results go out 16 rows at a time (pass j: rows 4 s + j, s = 0..15, of the wave's
+  // 64, the a tile's rows being permuted in LDS) through its own 4 KB slice of the b buffer
   // whose k-block was consumed last (nothing is in flight to that buffer, and this wave alone
   // transfers into this slice later), so that a store instruction writes whole rows of 256 bytes
   // instead of 16 pieces of 8 bytes.  The slice holds 16 rows x 256 B, 16-byte chunks XOR-ed with
