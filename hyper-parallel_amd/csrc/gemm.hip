@@ -450,6 +450,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   TileInfo tile_1 = T0;
   __amdgpu_buffer_rsrc_t rs_a1 = rsrc_a_of(T0), rs_a2 = rs_a1, rs_b1 = rsrc_b_of(T0), rs_b2 = rs_b1;
 
+  // per-tensor form: the one multiplier of the store phase, read once (inside the tile loop the loads
+  // would be repeated for every tile and waited for)
+  float tensor_scale = 1.f;
+  if (MODE == kScaleTensor) tensor_scale = p.sa[0] * p.sb[0];
+
   for (int tile = 0; tile < my_tiles; ++tile) {
   if (ACC) load_old_values(T0);
   for (int kb = 0; kb < kblocks; ++kb) {
@@ -625,8 +630,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // transfers into this slice later), so that a store instruction writes whole rows of 256 bytes
   // instead of 16 pieces of 8 bytes.  The slice holds 16 rows x 256 B, 16-byte chunks XOR-ed with
   // the row so that both the fragment-order writes and the row-order reads spread over all banks.
-  float tensor_scale = 1.f;
-  if (MODE == kScaleTensor) tensor_scale = p.sa[0] * p.sb[0];
   const int row0 = T0.row0, row_end = T0.row_end, n0 = T0.n0;
   // Lane coordinates re-derived behind an opaque copy: store addresses built from them would
   // otherwise be hoisted out of the tile loop and held in registers through the main loop.
