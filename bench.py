@@ -155,6 +155,16 @@ def other_configs(dev):
         "cfg2_training_step_fwd_bwd_ms": ms_p2,
         "cfg2_training_step_TFLOP/s": 3 * fl2 / ms_p2 / 1e9,
     }
+    # for orientation: this library's per-tensor GEMM and the vendor library's (hipBLASLt through
+    # torch._scaled_mm, unit scales) on the same codes; neither is the benchmarked recipe
+    one_ = torch.ones((), dtype=torch.float32, device=dev)
+    orient = {"per_tensor_gemm": tf(fl2, _time(lambda: hpfp8.gemm_per_tensor(xq2_, one_, wf2_.codes, one_)))}
+    try:
+        orient["vendor_scaled_mm"] = tf(fl2, _time(lambda: torch._scaled_mm(xq2_, wf2_.codes.t(), scale_a=one_, scale_b=one_,
+                                                                            out_dtype=torch.bfloat16)))
+    except Exception as err:          # (absent or differently named in another torch build)
+        orient["vendor_scaled_mm"] = f"unavailable: {type(err).__name__}"
+    res["cfg2_shape_per_tensor_for_orientation"] = orient
     del wf2_, xq2_, sx2_
     del xt_, wt_, got_, wf_
     torch.cuda.empty_cache()
