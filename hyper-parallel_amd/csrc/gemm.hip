@@ -88,9 +88,12 @@ __device__ __forceinline__ v8i frag_read(const uint8_t* row_base, int pc0) {
   return r;
 }
 
+// two floats -> two bf16 in one word (a low, b high): one v_cvt_pk_bf16_f32 (converted one by one, each
+// value costs a conversion, a shift and an or)
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  __bf16 x = (__bf16)a, y = (__bf16)b;
-  return (uint32_t)__builtin_bit_cast(uint16_t, x) | ((uint32_t)__builtin_bit_cast(uint16_t, y) << 16);
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 
 // Tile number -> (m tile, n tile).  Consecutive numbers (one XCD's CUs at any moment) cover
