@@ -645,13 +645,23 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // that is being refilled (its upper half is filled after these stores).
   uint8_t* stg_hi = kBAhead == 1 ? lds + (stage ^ 1) * kTileBytes + wave * 4096 + 2048 : stg + 2048;
   if (kBAhead == 1) stg += 2048;
-  auto stg_row = [&](int row) { return (row < 8 ? stg : stg_hi) + (row & 7) * 256; };
+  auto stg_row = [&](int row) { return (row < 8 ? stg : stg_hi) + (row & 7) * 256; };   // (row = l16e: the write side)
   const int ncol = n0 + wn * 128;                 // first column of the wave tile
   const bool cols_ok = ncol < N;
   constexpr int kHalves = OUT_F32 ? 2 : 1;       // fp32 rows of 128 columns take two slices
   constexpr int kPerHalf = 8 / kHalves;           // n-subtiles per slice
   const uint32_t stg_w = (uint32_t)(uintptr_t)(lds_ptr_t)stg_row(l16e);   // LDS byte address of this lane's row
-  auto store_tile = [&](auto with_bias, auto full_rows) {
+  // Rows leave through a buffer resource that starts at the wave tile's first element and ends with the
+  // tile's last valid row: the lane part of a store address is one offset computed once per tile, the
+  // rest scalar, and rows past the end of a ragged tile (or of an expert) are dropped by the range check.
+  constexpr int kEsize = OUT_F32 ? 4 : 2;
+  const int rows_valid = row_end - row0 < BM ? row_end - row0 : BM;
+  const __amdgpu_buffer_rsrc_t rsrc_st = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(reinterpret_cast<uint8_t*>(p.c) + ((int64_t)row0 * p.ldc + ncol) * kEsize), 0,
+      cols_ok && rows_valid > 0 ? (int)((((int64_t)rows_valid - 1) * p.ldc + 128) * kEsize) : 0, 0x00020000);
+  const uint32_t st_lane = (uint32_t)(((wm * 64 + ge * 4) * (int)p.ldc) * kEsize + l16e * 16);
+  const int st_row = (int)p.ldc * kEsize;        // bytes from one row of c to the next
+  auto store_tile = [&](auto with_bias) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -688,34 +698,25 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
           v4i val[2];
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
+            // staging row 4 (k2 + k) + ge; which half of the staging area it lies in does not depend on the lane
             const int row = 4 * (k2 + k) + ge;
-            val[k] = *reinterpret_cast<const v4i*>(stg_row(row) + ((l16e ^ row) * 16));
+            const uint8_t* half = (k2 + k) < 2 ? stg : stg_hi;
+            val[k] = *reinterpret_cast<const v4i*>(half + (4 * ((k2 + k) & 1) + ge) * 256 + ((l16e ^ row) * 16));
           }
 #pragma unroll
           for (int k = 0; k < 2; ++k) {
-            const int m = row0 + wm * 64 + (4 * (k2 + k) + ge) * 4 + j;     // staging row s of pass j is tile row 4 s + j
-            if (decltype(full_rows)::value || m < row_end) {
-              if (OUT_F32) {
-                float4* dst = reinterpret_cast<float4*>(reinterpret_cast<float*>(p.c) + (int64_t)m * p.ldc + ncol + h * 64 + l16e * 4);
-                const v4f fv = __builtin_bit_cast(v4f, val[k]);   // (a cast of the whole vector, not of its elements)
-                // streaming stores: the output is not read again here, and as ordinary stores a tile's
-                // 128-256 KB would push operand panels out of the L2
-                __builtin_nontemporal_store(fv, reinterpret_cast<v4f*>(dst));
-              } else {
-                __builtin_nontemporal_store(
-                    val[k], reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.c) + (int64_t)m * p.ldc + ncol + l16e * 8));
-              }
-            }
+            // staging row s of pass j is tile row 4 s + j (s = 4 (k2 + k) + ge: the ge part is in st_lane).
+            // Streaming stores: the output is not read again here, and as ordinary stores a tile's
+            // 128-256 KB would push operand panels out of the L2.
+            __builtin_amdgcn_raw_buffer_store_b128(val[k], rsrc_st, st_lane, (16 * (k2 + k) + j) * st_row + h * 256, 2);
           }
         }
       }
     }
   };
   if (cols_ok) {
-    // common case first: no bias, all 256 rows of the tile exist (no per-row predicate)
-    if (!p.bias && row0 + BM <= row_end) store_tile(std::false_type{}, std::true_type{});
-    else if (!p.bias) store_tile(std::false_type{}, std::false_type{});
-    else store_tile(std::true_type{}, std::false_type{});
+    if (!p.bias) store_tile(std::false_type{});
+    else store_tile(std::true_type{});
   } else {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -798,9 +799,8 @@ static int check_common(const char* what, const void* a, int64_t lda, const void
   HPFP8_REQUIRE(BM * lda < (int64_t)0x7FFFFFFF && BN * ldb < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
                 "%s: a row stride of 8 MiB or more is not supported", what);
   HPFP8_REQUIRE(M < (int64_t)0x7FFFFF00 && N < (int64_t)0x7FFFFF00, HPFP8_ERR_SHAPE, "%s: M or N too large", what);
-  // the old values of a tile are read with 32-bit byte offsets (256 rows of c)
-  HPFP8_REQUIRE(!accumulate || BM * ldc * 4 < (int64_t)0x7FFFF000, HPFP8_ERR_SHAPE,
-                "%s: accumulate needs a row stride of c below 8 MiB", what);
+  // a tile's 256 rows of c are stored (and its old values read) with 32-bit byte offsets
+  HPFP8_REQUIRE(BM * ldc * 4 < (int64_t)0x7FFFF000, HPFP8_ERR_SHAPE, "%s: the row stride of c must stay below 8 MiB", what);
   return 1;
 }
 
