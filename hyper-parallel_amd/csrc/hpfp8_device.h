@@ -74,19 +74,20 @@ __device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w &
 // pow2: the inverse is rounded up to the next power of two (its exponent field is then its E8M0 code,
 // which the matrix instruction can apply by itself) and the multiplier is its exact reciprocal.
 __device__ __forceinline__ void scales_from_amax(float amax, float& scale, float& scale_inv, int pow2 = 0) {
-  float amc = fmaxf(amax, kAmaxEps);
+  float amc = amax < kAmaxEps ? kAmaxEps : amax;   // (not fmaxf: a NaN amax must stay NaN, so that the group's scales and codes are NaN)
   scale = kFp8Max / amc;
   scale_inv = amc / kFp8Max;
   if (pow2) {
     uint32_t u = __float_as_uint(scale_inv);
-    if (u & 0x007FFFFFu) u = (u & 0xFF800000u) + 0x00800000u;
+    if ((u & 0x007FFFFFu) && u < 0x7F800000u) u = (u & 0xFF800000u) + 0x00800000u;   // (a NaN stays as it is)
     scale_inv = __uint_as_float(u);
     scale = 1.0f / scale_inv;
   }
 }
 
 __device__ __forceinline__ float clamp448(float y) {
-  return __builtin_amdgcn_fmed3f(y, -kFp8Max, kFp8Max);
+  const float c = __builtin_amdgcn_fmed3f(y, -kFp8Max, kFp8Max);   // of a NaN and two numbers the median instruction returns a number
+  return y != y ? y : c;                                            // NaN stays NaN (and is cast to the NaN code)
 }
 
 // Two bf16 in one word -> two E4M3 codes in the chosen half of `old`.

@@ -11,6 +11,10 @@
  *   scale          : fp32, quantize multiplier   448 / max(amax, 1e-12)
  *   scale_inv      : fp32, dequantize multiplier max(amax, 1e-12) / 448   (what the GEMMs consume)
  *   code           : e4m3_rne(clamp(float(x) * scale, -448, 448))
+ *   non-finite x   : IEEE rules with amax and clamp keeping NaN: a NaN in a scaling group makes the group's
+ *                    scale, scale_inv and codes NaN; +-Inf gives scale 0, scale_inv Inf, codes +-0 for the
+ *                    finite elements and NaN for the infinite ones.  Dequantized values and GEMM outputs fed
+ *                    by such a group are NaN.  The sign bit of a NaN code is unspecified.
  *
  * What each entry point stands in for.  The reference (mindspore-ai/hyper-parallel) has no FP8
  * kernels and no C/FFI boundary on its torch platform: a linear there is aten::linear called at

@@ -73,7 +73,7 @@ uint8_t hpo_e4m3_encode(float x) {
 static inline float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 static inline void scales(float amax, float* scale, float* scale_inv) {
-  float amc = amax > kAmaxEps ? amax : kAmaxEps;
+  float amc = amax < kAmaxEps ? kAmaxEps : amax;   /* a NaN amax stays NaN */
   *scale = kFp8Max / amc;
   *scale_inv = amc / kFp8Max;
 }
@@ -87,7 +87,7 @@ float hpo_amax_bf16(const uint16_t* x, int64_t n) {
   float am = 0.0f;
   for (int64_t i = 0; i < n; ++i) {
     float a = fabsf(bf16_to_f32(x[i]));
-    if (a > am) am = a;
+    if (a > am || a != a) am = a;   /* NaN wins and then stays */
   }
   return am;
 }
@@ -126,7 +126,7 @@ void hpo_quantize_128x128(const uint16_t* w, int64_t rows, int64_t cols, uint8_t
     float am = 0.0f, s, si;
     for (int i = 0; i < HPO_BLOCK; ++i) {
       float a = hpo_amax_bf16(w + (r0 + i) * cols + c0, HPO_BLOCK);
-      if (a > am) am = a;
+      if (a > am || a != a) am = a;   /* NaN wins and then stays */
     }
     scales(am, &s, &si);
     scale[b] = s;
@@ -147,7 +147,7 @@ void hpo_quantize_128x1_t(const uint16_t* x, int64_t m, int64_t k, uint8_t* qt, 
       float am = 0.0f, s, si;
       for (int i = 0; i < HPO_BLOCK; ++i) {
         float a = fabsf(bf16_to_f32(x[(b * HPO_BLOCK + i) * k + col]));
-        if (a > am) am = a;
+        if (a > am || a != a) am = a;   /* NaN wins and then stays */
       }
       scales(am, &s, &si);
       scale_t[col * mb + b] = s;

@@ -27,7 +27,12 @@ Numeric conventions (all fp32, IEEE, round-to-nearest-even, denormals kept):
   gemm      = sum over 128-wide k-blocks, ascending, of
               (sum_k decode(a)*decode(b)) * (sa_inv * sb_inv); bias added in fp32; one final
               rounding to bf16.
-Inputs are required to be finite; NaN/Inf behaviour is left unspecified.
+Non-finite inputs follow from the same formulas under IEEE rules, with amax and clamp keeping NaN as
+torch's eager amax / clamp do: a NaN in a scaling group makes the group's scale, scale_inv and all of
+its codes NaN; +-Inf makes scale 0 and scale_inv Inf, the group's finite elements +-0 and the
+infinite ones NaN.  Either way the dequantized group (and every GEMM output row or column it feeds)
+is NaN throughout, so an overflow check downstream sees it.  Which of the two NaN codes (0x7F, 0xFF)
+a cast writes is not specified.
 
 How each function is pinned (tests/test_oracle_pins.py)
 -------------------------------------------------------
@@ -36,7 +41,7 @@ How each function is pinned (tests/test_oracle_pins.py)
       256 codes, all 65536 bf16 bit patterns, every rounding midpoint and its fp32
       neighbours, and a hand-written known-answer table.
   amax, scales              : brute force on tiny inputs; special cases amax = 0 and
-      amax < 448/FLT_MAX.
+      amax < 448/FLT_MAX; NaN / Inf groups against the recipe written with torch's eager operators.
   quantize_*                : each blocked variant equals the per-tensor quantizer applied to
       every block separately (pure-Python loops on small shapes); the transposed variant
       equals quantize_1x128(x.T); the C restatement (fp8_oracle.c) is a second independent
@@ -152,14 +157,14 @@ def scales_from_amax(am: np.ndarray, pow2: bool = False):
     if pow2:
         u = np.ascontiguousarray(scale_inv).view(np.uint32)
         up = (u & np.uint32(0xFF800000)) + np.uint32(0x00800000)
-        scale_inv = np.where((u & np.uint32(0x007FFFFF)) != 0, up, u).astype(np.uint32).view(np.float32).reshape(scale_inv.shape)
+        scale_inv = np.where(((u & np.uint32(0x007FFFFF)) != 0) & (u < np.uint32(0x7F800000)), up, u).astype(np.uint32).view(np.float32).reshape(scale_inv.shape)
         with np.errstate(divide="ignore"):
             scale = (np.float32(1.0) / scale_inv).astype(np.float32)
     return scale, scale_inv
 
 
 def _cast(x_f32: np.ndarray, scale: np.ndarray) -> np.ndarray:
-    with np.errstate(over="ignore"):      # a product beyond fp32 range becomes +-Inf and is clamped next
+    with np.errstate(over="ignore", invalid="ignore"):   # beyond fp32 range: +-Inf, clamped next; Inf * 0 and NaN stay NaN
         y = (np.asarray(x_f32, dtype=np.float32) * np.asarray(scale, dtype=np.float32)).astype(np.float32)
     y = np.clip(y, -FP8_MAX, FP8_MAX).astype(np.float32)
     return e4m3_encode(y)
@@ -224,7 +229,8 @@ def quantize_128x1_t(x_bits: np.ndarray, pow2: bool = False):
 
 
 def _to_bf16_bits_product(vals_f32: np.ndarray, mult: np.ndarray) -> np.ndarray:
-    return f32_to_bf16_bits((vals_f32 * np.asarray(mult, np.float32)).astype(np.float32))
+    with np.errstate(invalid="ignore"):                 # 0 * Inf of a group that held an Inf stays NaN
+        return f32_to_bf16_bits((vals_f32 * np.asarray(mult, np.float32)).astype(np.float32))
 
 
 def dequantize_per_tensor(codes: np.ndarray, scale_inv) -> np.ndarray:

@@ -60,3 +60,33 @@ def special_bf16_rows(cols=128) -> torch.Tensor:
     r = torch.full((cols,), 1e-12); r[7] = 2e-12; rows.append(r)                 # around the eps clamp
     r = torch.full((cols,), 1e-13); rows.append(r)                               # below the eps clamp
     return torch.stack(rows).to(torch.bfloat16)
+
+
+def nonfinite_bf16(rows=256, cols=512, seed=5) -> torch.Tensor:
+    """Seeded normal data with NaN, +Inf and -Inf planted in known 128-wide groups (and groups left
+    clean beside them): (0, 0..127) a NaN, (1, 128..255) +Inf, (2, 256..383) -Inf and a NaN,
+    (130, 0..127) -Inf, (131, 384..511) a negative NaN."""
+    x = randn_bf16((rows, cols), seed).clone()
+    x[0, 5] = float("nan")
+    x[1, 128 + 77] = float("inf")
+    x[2, 256 + 1] = float("-inf")
+    x[2, 256 + 100] = float("nan")
+    x[130, 127] = float("-inf")
+    v = x.view(torch.int16)
+    v[131, 384 + 64] = -64                 # 0xFFC0: a NaN with its sign bit set
+    return x
+
+
+def canon_nan_codes(c: np.ndarray) -> np.ndarray:
+    """E4M3 codes with the sign of NaN codes dropped (0xFF -> 0x7F): which of the two a cast writes for
+    a NaN is not part of the numeric recipe."""
+    c = np.asarray(c, dtype=np.uint8)
+    return np.where((c & 0x7F) == 0x7F, np.uint8(0x7F), c)
+
+
+def same_f32_or_nan(a, b) -> bool:
+    """fp32 arrays equal bit for bit where both are numbers, and NaN in the same places."""
+    a = np.asarray(a, dtype=np.float32).reshape(-1)
+    b = np.asarray(b, dtype=np.float32).reshape(-1)
+    na, nb = np.isnan(a), np.isnan(b)
+    return a.shape == b.shape and np.array_equal(na, nb) and np.array_equal(a[~na].view(np.uint32), b[~nb].view(np.uint32))

@@ -74,6 +74,55 @@ def test_exact_on_integer_inputs(gpu):
     assert np.array_equal(U.f32(small), O.bf16_bits_to_f32(O.f32_to_bf16_bits(w)))
 
 
+def test_non_finite_groups_make_their_output_rows_nan_and_no_others(gpu):
+    """Activations with NaN / +-Inf planted in rows 0, 1, 2, 130 and 131: exactly those rows of the
+    output are NaN, in every scale mode, and all other rows are what they are without the planted values
+    (a NaN group must not leak into rows that share its tile, its wave or its scale loads)."""
+    import hpfp8
+    x = U.nonfinite_bf16(256, 512)
+    w = U.randn_bf16((384, 512), 31, 0.02)
+    bad_rows = np.zeros(256, bool)
+    bad_rows[[0, 1, 2, 130, 131]] = True
+    xg, wg = x.to(gpu), w.to(gpu)
+    xc = x.clone()
+    xc[bad_rows] = 1.0
+    xcg = xc.to(gpu)
+    for pow2 in (False, True):
+        xq, sx = hpfp8.quantize_1x128(xg, kmajor=True, pow2=pow2)
+        cq, sc = hpfp8.quantize_1x128(xcg, kmajor=True, pow2=pow2)
+        wq, sw = hpfp8.quantize_128x128(wg, pow2=pow2)
+        w1, sw1 = hpfp8.quantize_1x128(wg, kmajor=True, pow2=pow2)
+        for out_dtype in (torch.bfloat16, torch.float32):
+            for kw, bq, sb in (({}, wq, sw), ({"sb_gran": 1}, w1, sw1)):
+                y = hpfp8.gemm_blockwise(xq, sx, bq, sb, out_dtype=out_dtype, pow2_scales=pow2, **kw)
+                yc = hpfp8.gemm_blockwise(cq, sc, bq, sb, out_dtype=out_dtype, pow2_scales=pow2, **kw)
+                nan = torch.isnan(y).cpu().numpy()
+                assert nan[bad_rows].all() and not nan[~bad_rows].any(), (pow2, out_dtype, kw)
+                assert torch.equal(y[~torch.from_numpy(bad_rows).to(gpu)], yc[~torch.from_numpy(bad_rows).to(gpu)])
+        # the planted values on the other operand: columns of the output (x as the b operand, row scales)
+        y = hpfp8.gemm_blockwise(w1, sw1, xq, sx, sb_gran=1, out_dtype=torch.float32, pow2_scales=pow2)
+        nan = torch.isnan(y).cpu().numpy()
+        assert nan[:, bad_rows].all() and not nan[:, ~bad_rows].any()
+        # accumulate: NaN rows stay NaN, the others add up as usual
+        acc = torch.ones((256, 384), dtype=torch.float32, device=gpu)
+        hpfp8.gemm_blockwise(xq, sx, w1, sw1, sb_gran=1, out=acc, accumulate=True, pow2_scales=pow2)
+        nan = torch.isnan(acc).cpu().numpy()
+        assert nan[bad_rows].all() and not nan[~bad_rows].any()
+    # against the oracle, codes and scales as the oracle makes them
+    rq, _, rsi = O.quantize_1x128(U.bits(x))
+    rw, _, rswi = O.quantize_128x128(U.bits(w))
+    want, _ = O.gemm_blockwise(rq, rsi, rw, rswi)
+    assert np.array_equal(np.isnan(want).all(axis=1), bad_rows) and not np.isnan(want[~bad_rows]).any()
+    xq, sx = hpfp8.quantize_1x128(xg, kmajor=True)
+    wq, sw = hpfp8.quantize_128x128(wg)
+    got = U.f32(hpfp8.gemm_blockwise(xq, sx, wq, sw, out_dtype=torch.float32))
+    assert rel(got[~bad_rows], want[~bad_rows]) < TOL_F32
+    # per tensor: one NaN anywhere makes the scale, and with it every output, NaN
+    xq, _, sxi = hpfp8.quantize_per_tensor(xg)
+    wq, _, swi = hpfp8.quantize_per_tensor(wg)
+    assert bool(torch.isnan(hpfp8.gemm_per_tensor(xq, sxi, wq, swi)).all())
+
+
 def test_golden_gemm(gpu):
     import os
     import hpfp8

@@ -198,6 +198,84 @@ def test_special_values_and_edge_shapes(gpu):
         hpfp8.quantize_128x1_t(torch.zeros((100, 128), dtype=torch.bfloat16, device=gpu))
 
 
+def test_non_finite_inputs_every_quantizer(gpu):
+    """NaN and +-Inf planted in known groups: scales bit for bit (NaN where the oracle's are NaN), codes
+    byte for byte up to the sign of NaN codes, for every quantizer; groups beside the planted ones keep
+    ordinary codes; dequantized, the planted groups are NaN throughout."""
+    import hpfp8
+    x = U.nonfinite_bf16(256, 512)
+    xb = U.bits(x)
+    xg = x.to(gpu)
+
+    def same(q, rq, scales, rscales):
+        assert np.array_equal(U.canon_nan_codes(U.codes(q)), U.canon_nan_codes(rq))
+        for a, b in zip(scales, rscales):
+            assert U.same_f32_or_nan(U.f32(a), b)
+
+    rq, rs, rsi = O.quantize_1x128(xb)
+    for kmajor in (False, True):
+        q, s, si = hpfp8.quantize_1x128(xg, want_scale=True, kmajor=kmajor)
+        same(q, rq, (s, si), (rs, rsi))
+    clean = np.isfinite(rsi)
+    assert clean.sum() == rsi.size - 5
+    assert not ((U.codes(q).reshape(256, 4, 128)[clean] & 0x7F) == 0x7F).any()
+    d = U.f32(hpfp8.dequantize_1x128(q, si.contiguous()).float()).reshape(256, 4, 128)
+    assert np.isnan(d[~clean]).all() and np.isfinite(d[clean]).all()
+    rqw, rsw, rsiw = O.quantize_128x128(xb)
+    q, si, qt, s = hpfp8.quantize_128x128(xg, with_transpose=True, want_scale=True)
+    same(q, rqw, (s, si), (rsw, rsiw))
+    same(qt, rqw.T, (), ())
+    rqt, rst, rsit = O.quantize_128x1_t(xb)
+    for kmajor in (False, True):
+        qt, s, si = hpfp8.quantize_128x1_t(xg, want_scale=True, kmajor=kmajor)
+        same(qt, rqt, (s, si), (rst, rsit))
+        q1, si1, qt2, sit2 = hpfp8.quantize_1x128_and_128x1_t(xg, kmajor=kmajor)
+        same(q1, rq, (si1,), (rsi,))
+        same(qt2, rqt, (sit2,), (rsit,))
+    # the power-of-two recipe: the same groups are NaN / Inf
+    rq2, rs2, rsi2 = O.quantize_1x128(xb, pow2=True)
+    q, s, si = hpfp8.quantize_1x128(xg, want_scale=True, kmajor=True, pow2=True)
+    same(q, rq2, (s, si), (rs2, rsi2))
+    # per tensor: a NaN anywhere makes every code and both scales NaN; with only an Inf the scale is 0
+    q, s, si = hpfp8.quantize_per_tensor(xg)
+    rqp, rsp, rsip = O.quantize_per_tensor(xb)
+    same(q, rqp, (s, si), (rsp, rsip))
+    assert np.isnan(U.f32(s)).all() and ((U.codes(q) & 0x7F) == 0x7F).all()
+    xi = xb[1:2].copy()
+    q, s, si = hpfp8.quantize_per_tensor(U.from_bits(xi, gpu))
+    rqp, rsp, rsip = O.quantize_per_tensor(xi)
+    same(q, rqp, (s, si), (rsp, rsip))
+    assert float(s) == 0.0 and np.isposinf(U.f32(si)).all()
+    # a caller-supplied amax (the clamped cast): NaN elements stay NaN, infinite ones saturate
+    am = torch.tensor(3.0, dtype=torch.float32, device=gpu)
+    q, s, si = hpfp8.quantize_per_tensor(xg, amax_in=am)
+    scale, _ = O.scales_from_amax(np.float32(3.0))
+    want = O._cast(O.bf16_bits_to_f32(xb), scale)
+    same(q, want, (), ())
+    got = U.codes(q)
+    assert (got[0, 5] & 0x7F) == 0x7F and got[1, 128 + 77] == 0x7E and got[2, 256 + 1] == 0xFE and ((got & 0x7F) == 0x7F).sum() == 3
+    # SwiGLU fused with the quantizer: x as [gate | up], so planted values sit in gates and in ups
+    q, si, act = hpfp8.swiglu_quantize_1x128(xg, kmajor=True, want_act=True)
+    with np.errstate(all="ignore"):
+        rqs, _, rsis, ract = O.swiglu_quantize_1x128(xb)
+    same(q, rqs, (si,), (rsis,))
+    assert U.same_f32_or_nan(U.f32(act.float()), O.bf16_bits_to_f32(ract))
+    assert np.isnan(rsis).sum() + np.isinf(rsis).sum() == 5
+    # gradient bucket: quantize, and the fused pack / unpack of the same elements
+    flat = xg.reshape(-1)
+    c, si = hpfp8.quantize_bucket(flat)
+    same(c, rq.reshape(-1), (si,), (rsi,))
+    back = hpfp8.dequantize_bucket(c, si, grad_scale=0.5)
+    assert np.array_equal(np.isnan(U.f32(back.float())).reshape(256, 4, 128).all(axis=2), ~clean)
+    bucket = hpfp8.Fp8GradBucket([flat.numel()], shard_size=1, grad_scale=0.5)
+    qb, sib = bucket.pack([flat])
+    same(qb, rq.reshape(1, -1), (sib,), (rsi,))
+    out = [torch.zeros(flat.numel(), dtype=torch.bfloat16, device=gpu)]
+    bucket.unpack(qb[0].contiguous(), sib[0].contiguous(), out)
+    assert np.array_equal(np.isnan(U.f32(out[0].float())).reshape(256, 4, 128).all(axis=2), ~clean)
+    assert np.array_equal(U.bits(out[0])[np.repeat(clean.reshape(-1), 128)], U.bits(back)[np.repeat(clean.reshape(-1), 128)])
+
+
 def test_bucket_full_size_properties(gpu):
     """2^29-element bucket (cfg 5): properties that do not need a CPU pass over 1 GiB:
     a strided sample of groups against the oracle, idempotence of quantize(dequantize(.)) on the

@@ -285,6 +285,50 @@ def test_c_per_tensor_and_dequant_bit_exact():
     assert np.array_equal(O.dequantize_1x128(q, si), C.dequantize_1x128(q, si))
 
 
+# ---------------------------------------------------------------- non-finite inputs
+def _torch_eager_quantize_groups(x: torch.Tensor):
+    """The recipe spelled with torch's eager operators on [G, 128] groups: amax and clamp keep NaN."""
+    xf = x.float()
+    amc = xf.abs().amax(dim=1, keepdim=True).clamp(min=1e-12)
+    scale = torch.tensor(448.0) / amc
+    scale_inv = amc / torch.tensor(448.0)
+    q = (xf * scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+    return q.numpy(), scale.numpy().reshape(-1), scale_inv.numpy().reshape(-1)
+
+
+def test_non_finite_inputs_follow_ieee_like_torch_eager_and_c():
+    """NaN in a group: scale, scale_inv and every code of the group are NaN.  +-Inf: scale 0, scale_inv
+    Inf, finite elements become +-0 and the infinite ones NaN.  Groups beside them are untouched."""
+    x = U.nonfinite_bf16(256, 512)
+    xb = U.bits(x)
+    q, s, si = O.quantize_1x128(xb)
+    tq, ts, tsi = _torch_eager_quantize_groups(x.reshape(-1, 128))
+    assert np.array_equal(U.canon_nan_codes(q).reshape(-1, 128), U.canon_nan_codes(tq))
+    assert U.same_f32_or_nan(s, ts) and U.same_f32_or_nan(si, tsi)
+    assert np.isnan(s[0, 0]) and np.isnan(si[0, 0]) and ((q[0, :128] & 0x7F) == 0x7F).all()
+    assert s[1, 1] == 0 and np.isposinf(si[1, 1]) and (q[1, 128 + 77] & 0x7F) == 0x7F
+    assert ((np.delete(q[1, 128:256], 77) & 0x7F) == 0).all()
+    assert np.isnan(s[2, 2]) and np.isnan(s[131, 3]) and np.isposinf(si[130, 0])
+    clean = np.isfinite(si)
+    assert clean.sum() == si.size - 5 and not ((q.reshape(256, 4, 128)[clean] & 0x7F) == 0x7F).any()
+    # the other quantizers and the C restatement
+    for name in ("quantize_1x128", "quantize_128x128", "quantize_128x1_t"):
+        a, b = getattr(O, name)(xb), getattr(C, name)(xb)
+        assert np.array_equal(U.canon_nan_codes(a[0]), U.canon_nan_codes(b[0])), name
+        assert U.same_f32_or_nan(a[1], b[1]) and U.same_f32_or_nan(a[2], b[2]), name
+    qw, sw, siw = O.quantize_128x128(xb)
+    assert np.isnan(siw[0, 0]) and np.isnan(siw[0, 2]) and np.isposinf(siw[0, 1]) and np.isposinf(siw[1, 0]) and np.isnan(siw[1, 3])
+    assert np.isfinite(siw).sum() == 3
+    qt, st, sit = O.quantize_128x1_t(xb)
+    q2, s2, si2 = O.quantize_1x128(np.ascontiguousarray(xb.T))
+    assert np.array_equal(qt, q2) and U.same_f32_or_nan(sit, si2)
+    a, b = O.quantize_per_tensor(xb), C.quantize_per_tensor(xb)
+    assert np.isnan(a[1]) and np.isnan(b[1]) and ((a[0] & 0x7F) == 0x7F).all() and ((b[0] & 0x7F) == 0x7F).all()
+    # dequantized, every affected group is NaN throughout: an overflow check on the result sees it
+    d = O.bf16_bits_to_f32(O.dequantize_1x128(q, si)).reshape(256, 4, 128)
+    assert np.isnan(d[~clean]).all() and np.isfinite(d[clean]).all()
+
+
 # ---------------------------------------------------------------- GEMMs
 def test_gemm_per_tensor_against_torch_scaled_mm():
     x = U.randn_bf16((64, 256), seed=81)
