@@ -125,6 +125,8 @@ def other_configs(dev):
     hgu = torch.randn((4096, 36864), generator=g, device=dev).to(torch.bfloat16)
     res["cfg2_swiglu_quantize"] = gb(4096 * 18432 * 5 + 4096 * (18432 // 128) * 4,
                                      _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True)))
+    res["cfg2_swiglu_quantize_fast"] = gb(4096 * 18432 * 5 + 4096 * (18432 // 128) * 4,
+                                          _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True, fast=True)))
     del hgu
     # cfg 2 as a training step of the module: forward + backward through fp8_linear (the weight's FP8 form
     # made beforehand, as Fp8Linear's cache does), beside torch's bf16 F.linear on the same tensors

@@ -179,21 +179,32 @@ __device__ __forceinline__ float exp_spec(float t) {
   return (p * __uint_as_float((uint32_t)((int)k + 126) << 23)) * 2.0f;
 }
 
+// silu(g) = g / (1 + exp(-g)).  FAST: with the hardware's base-2 exponential and reciprocal (each within one
+// unit in the last place of fp32), 4 instructions instead of about 35; the result can differ from the exactly
+// specified one in the last bits of fp32, which moves roughly one bf16 rounding in several thousand.
+template <bool FAST>
+__device__ __forceinline__ float silu_f32(float g) {
+  if (FAST) return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504f));
+  return g / (1.0f + exp_spec(-g));
+}
+
 // bf16(bf16(silu(g)) * u) for two (g, u) pairs packed like their sources: the two roundings of the
 // unfused bf16 graph (silu, then the product).
+template <bool FAST>
 __device__ __forceinline__ uint32_t swiglu2(uint32_t gw, uint32_t uw) {
-  const float g0 = bf16lo(gw), g1 = bf16hi(gw);
-  const __bf16 s0 = (__bf16)(g0 / (1.0f + exp_spec(-g0)));
-  const __bf16 s1 = (__bf16)(g1 / (1.0f + exp_spec(-g1)));
-  const __bf16 a0 = (__bf16)((float)s0 * bf16lo(uw));
-  const __bf16 a1 = (__bf16)((float)s1 * bf16hi(uw));
-  return (uint32_t)__builtin_bit_cast(uint16_t, a0) | ((uint32_t)__builtin_bit_cast(uint16_t, a1) << 16);
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  // both values of a pair through one conversion instruction, rounded to nearest even like the scalar cast
+  const f32x2 sf = {silu_f32<FAST>(bf16lo(gw)), silu_f32<FAST>(bf16hi(gw))};
+  const uint32_t sw = __builtin_bit_cast(uint32_t, __builtin_convertvector(sf, bf16x2));
+  const f32x2 af = {bf16lo(sw) * bf16lo(uw), bf16hi(sw) * bf16hi(uw)};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(af, bf16x2));
 }
 
 // h[rows, 2 * inter] (row stride ld elements): gate = columns [0, inter), up = [inter, 2 inter).
 // q[rows, inter] = codes of act = silu(gate) * up in 1x128 groups; scales [rows, inter/128], or
 // [inter/128, rows] with KMAJOR.  Work split as in quant_1x128_kmajor_kernel.
-template <bool KMAJOR>
+template <bool KMAJOR, bool FAST>
 __global__ __launch_bounds__(256) void swiglu_quant_1x128_kernel(const uint16_t* __restrict__ h, int64_t ld,
                                                                  uint8_t* __restrict__ q, float* __restrict__ scale,
                                                                  float* __restrict__ scale_inv,
@@ -217,10 +228,10 @@ __global__ __launch_bounds__(256) void swiglu_quant_1x128_kernel(const uint16_t*
   for (int u = 0; u < 4; ++u) {
     const bool ok = row < rows && g0 + u < groups;
     uint4 a;
-    a.x = swiglu2(vg[u].x, vu[u].x);
-    a.y = swiglu2(vg[u].y, vu[u].y);
-    a.z = swiglu2(vg[u].z, vu[u].z);
-    a.w = swiglu2(vg[u].w, vu[u].w);
+    a.x = swiglu2<FAST>(vg[u].x, vu[u].x);
+    a.y = swiglu2<FAST>(vg[u].y, vu[u].y);
+    a.z = swiglu2<FAST>(vg[u].z, vu[u].z);
+    a.w = swiglu2<FAST>(vg[u].w, vu[u].w);
     const uint32_t m = row16_max_u32(mag8(a));
     float s, si;
     scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
@@ -791,7 +802,7 @@ int hpfp8_quantize_1x128_and_128x1_t_pow2_bf16(const void* x, int64_t m, int64_t
 }
 
 static int swiglu_quantize_impl(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
-                                float* scale, float* scale_inv, void* act, int pow2, hpfp8_stream_t stream) {
+                                float* scale, float* scale_inv, void* act, int pow2, int fast, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: negative shape");
   HPFP8_REQUIRE(inter % kBlock == 0, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: width %lld is not a multiple of 128",
                 (long long)inter);
@@ -806,23 +817,31 @@ static int swiglu_quantize_impl(const void* h, int64_t rows, int64_t inter, int6
   const int64_t blocks = ((groups + 3) / 4) * ((rows + 15) / 16);
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "swiglu_quantize_1x128: tensor too large");
   hipStream_t s = (hipStream_t)stream;
-  if (kmajor)
-    swiglu_quant_1x128_kernel<true><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)h, ld_h, (uint8_t*)q, scale, scale_inv,
-                                                                     (uint16_t*)act, (int)rows, (int)inter, pow2);
-  else
-    swiglu_quant_1x128_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)h, ld_h, (uint8_t*)q, scale, scale_inv,
-                                                                      (uint16_t*)act, (int)rows, (int)inter, pow2);
+  auto launch = [&](auto kernel) {
+    kernel<<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)h, ld_h, (uint8_t*)q, scale, scale_inv, (uint16_t*)act,
+                                            (int)rows, (int)inter, pow2);
+  };
+  if (kmajor && fast) launch(swiglu_quant_1x128_kernel<true, true>);
+  else if (kmajor) launch(swiglu_quant_1x128_kernel<true, false>);
+  else if (fast) launch(swiglu_quant_1x128_kernel<false, true>);
+  else launch(swiglu_quant_1x128_kernel<false, false>);
   return check_launch("swiglu_quantize_1x128");
 }
 
 int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
                                      float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
-  return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, 0, stream);
+  return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, 0, 0, stream);
 }
 
 int hpfp8_swiglu_quantize_1x128_pow2_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
                                           float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
-  return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, 1, stream);
+  return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, 1, 0, stream);
+}
+
+int hpfp8_swiglu_quantize_1x128_fast_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, int pow2,
+                                          void* q, float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(pow2 == 0 || pow2 == 1, HPFP8_ERR_ARG, "swiglu_quantize_1x128_fast: pow2 must be 0 or 1");
+  return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, pow2, 1, stream);
 }
 
 int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld, void* q_t, int64_t ld_t,

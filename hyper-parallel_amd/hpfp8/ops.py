@@ -176,9 +176,14 @@ def quantize_128x128(w: torch.Tensor, with_transpose: bool = False, want_scale: 
     return out
 
 
-def swiglu_quantize_1x128(h: torch.Tensor, kmajor: bool = True, want_act: bool = False, pow2: bool = False):
+def swiglu_quantize_1x128(h: torch.Tensor, kmajor: bool = True, want_act: bool = False, pow2: bool = False,
+                          fast: bool = False):
     """h[M, 2I] bf16 (gate | up halves; any row stride that is a multiple of 8) ->
-    (codes[M, I], scale_inv[M, I/128]) of act = silu(gate) * up, plus act itself (bf16) if asked for."""
+    (codes[M, I], scale_inv[M, I/128]) of act = silu(gate) * up, plus act itself (bf16) if asked for.
+
+    ``fast``: silu from the hardware's exponential and reciprocal approximations instead of the exactly
+    specified sequence (about twice as fast; the rounded silu may differ by one bf16 unit in the last place, act by
+    two, in about one element per ten thousand; codes and scales are the exact quantization of that act)."""
     h = _check_bf16(h, "h", contiguous=False)
     if h.dim() != 2 or h.shape[1] % (2 * BLOCK):
         raise ValueError("h must be 2-D with a width that is a multiple of 256")
@@ -188,8 +193,13 @@ def swiglu_quantize_1x128(h: torch.Tensor, kmajor: bool = True, want_act: bool =
     q = torch.empty((m, inter), dtype=FP8, device=h.device)
     s_inv = torch.empty((inter // BLOCK, m) if kmajor else (m, inter // BLOCK), dtype=torch.float32, device=h.device)
     act = torch.empty((m, inter), dtype=torch.bfloat16, device=h.device) if want_act else None
-    _lib.call("hpfp8_swiglu_quantize_1x128_pow2_bf16" if pow2 else "hpfp8_swiglu_quantize_1x128_bf16", _ptr(h), m, inter, h.stride(0) if m > 1 else 2 * inter, int(kmajor),
-              _ptr(q), None, _ptr(s_inv), _ptr(act), _stream())
+    ld_h = h.stride(0) if m > 1 else 2 * inter
+    if fast:
+        _lib.call("hpfp8_swiglu_quantize_1x128_fast_bf16", _ptr(h), m, inter, ld_h, int(kmajor), int(pow2),
+                  _ptr(q), None, _ptr(s_inv), _ptr(act), _stream())
+    else:
+        _lib.call("hpfp8_swiglu_quantize_1x128_pow2_bf16" if pow2 else "hpfp8_swiglu_quantize_1x128_bf16", _ptr(h), m,
+                  inter, ld_h, int(kmajor), _ptr(q), None, _ptr(s_inv), _ptr(act), _stream())
     if kmajor:
         s_inv = s_inv.t()
     return (q, s_inv, act) if want_act else (q, s_inv)

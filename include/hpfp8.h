@@ -142,6 +142,14 @@ int hpfp8_swiglu_quantize_1x128_pow2_bf16(const void* h, int64_t rows, int64_t i
  * (kmajor != 0) [inter/128, rows].  act (bf16 [rows, inter]) is also written when not NULL. */
 int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, void* q,
                                      float* scale, float* scale_inv, void* act, hpfp8_stream_t stream);
+/* The same with silu from the hardware's base-2 exponential and reciprocal approximations (each within
+ * one unit in the last place of fp32) instead of the exactly specified sequence: the kernel is then bound by
+ * memory, not arithmetic (about twice as fast).  the bf16 silu can differ from the exact form's by one unit in the last
+ * place (act, its product with up, by two) in about one element per ten thousand, as two GPU implementations of the eager graph differ from each
+ * other; q, scale and scale_inv are the exact 1x128 quantization of the act this call writes.  pow2 (0 / 1)
+ * selects power-of-two scales as in hpfp8_swiglu_quantize_1x128_pow2_bf16. */
+int hpfp8_swiglu_quantize_1x128_fast_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, int pow2,
+                                          void* q, float* scale, float* scale_inv, void* act, hpfp8_stream_t stream);
 
 /* Byte transpose of a code matrix: q[rows, cols] (row stride ld) -> q_t[cols, rows] (row stride ld_t);
  * rows, cols multiples of 128.  128x128 scaling blocks are symmetric, so this turns the codes of a

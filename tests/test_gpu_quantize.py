@@ -388,6 +388,46 @@ def test_swiglu_fused_with_quantize(gpu, shape, kmajor):
     assert np.array_equal(U.codes(q3), rq3) and np.array_equal(U.f32_bits(U.f32(si3)), U.f32_bits(rsi3))
 
 
+@pytest.mark.parametrize("pow2", [False, True])
+def test_swiglu_fast_form(gpu, pow2):
+    """The form with the hardware's exponential and reciprocal: the bf16 silu within one unit in the last
+    place of the exactly specified form's, hence act within two (and so against torch's eager graph),
+    differing at all in well under 0.1 % of the elements; codes and scales are bit for bit the oracle's 1x128 quantization of the act it wrote;
+    special inputs (zeros, 88.5, +-200, NaN, +-Inf) give what the exact form gives, -88.5 a zero."""
+    import hpfp8
+    import torch.nn.functional as F
+    h = U.randn_bf16((512, 7168), 5, 2.0, 0.001, 30.0)
+    h[0, :6] = torch.tensor([0.0, -0.0, 88.5, -88.5, -200.0, 200.0], dtype=torch.bfloat16)
+    h[1, 0] = float("nan")
+    h[2, 1] = float("inf")
+    h[3, 2] = float("-inf")
+    h[4, 3584 + 7] = float("inf")
+    hg = h.to(gpu)
+    q, si, act = hpfp8.swiglu_quantize_1x128(hg, kmajor=True, want_act=True, pow2=pow2, fast=True)
+    qe, sie, acte = hpfp8.swiglu_quantize_1x128(hg, kmajor=True, want_act=True, pow2=pow2)
+    a, e = act.view(torch.int16).int(), acte.view(torch.int16).int()
+    nan_a, nan_e = torch.isnan(act), torch.isnan(acte)
+    assert torch.equal(nan_a, nan_e) and int(nan_a.sum()) >= 2
+    d = (a - e).abs()[~nan_a]
+    # (the reciprocal instruction returns 0 where 1 + exp(-g) exceeds 2^126, g < -87.3, where the exact form
+    # still gives |silu| ~ 1e-37: both are zero for every purpose, but far apart counted in bf16 steps)
+    tiny = ((act.float().abs() < 1e-30) & (acte.float().abs() < 1e-30))[~nan_a]
+    # one step in the bf16 rounding of silu (a near-tie decided the other way) can become two in the product
+    assert bool(((d <= 2) | tiny).all())
+    assert float(((d != 0) & ~tiny).float().mean()) < 1e-3 and float(((d > 1) & ~tiny).float().mean()) < 1e-4
+    assert torch.equal(act[0, :3], acte[0, :3]) and torch.equal(act[0, 4:6], acte[0, 4:6]) and float(act[0, 3].abs()) < 1e-30
+    ref = F.silu(hg[:, :3584]) * hg[:, 3584:]
+    dr = (a - ref.view(torch.int16).int()).abs()[~nan_a]
+    assert float((dr > 2).float().mean()) < 1e-5 and float((dr > 1).float().mean()) < 1e-4 and float((dr != 0).float().mean()) < 3e-3
+    # the quantizer half stays exact: codes and scales of the act that was written
+    with np.errstate(all="ignore"):
+        rq, _, rsi = O.quantize_1x128(U.bits(act), pow2=pow2)
+    assert np.array_equal(U.canon_nan_codes(U.codes(q)), U.canon_nan_codes(rq)) and U.same_f32_or_nan(U.f32(si), rsi)
+    # without act, and with row-major scales: same codes
+    q2, si2 = hpfp8.swiglu_quantize_1x128(hg, kmajor=False, pow2=pow2, fast=True)
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and U.same_f32_or_nan(U.f32(si2), U.f32(si))
+
+
 def test_dequantize_accumulate_into_fp32_main_grad(gpu):
     import hpfp8
     g = U.randn_bf16((300, 640), 71, 1e-3, 0.002, 100.0)
