@@ -73,6 +73,21 @@ def cpu_baseline(x_bits, w_bits, target_seconds=15.0):
     C.gemm_blockwise(xq, sxi, wq, swi)
     t_g = time.perf_counter() - t0
     step_seconds = t_qw + (t_qx + t_g) * (M / ms)
+    # beside it, what the reference executes on a CPU today for this layer: aten::linear in bf16
+    # (hyper_parallel/core/shard/_op_dispatch.py:283), on as many of the first rows as take about 3 s
+    import torch
+    import torch.nn.functional as F
+    torch.set_num_threads(threads)
+    xt = torch.from_numpy(np.ascontiguousarray(x_bits).view(np.int16)).view(torch.bfloat16)
+    wt = torch.from_numpy(w_bits.view(np.int16)).view(torch.bfloat16)
+    F.linear(xt[:64], wt)
+    t0 = time.perf_counter()
+    F.linear(xt[:64], wt)
+    t64 = max(time.perf_counter() - t0, 1e-6)
+    xt = xt[:max(64, min(xt.shape[0], int(3.0 / t64) * 64))]          # about 3 s of work
+    t0 = time.perf_counter()
+    F.linear(xt, wt)
+    t_lin = max(time.perf_counter() - t0, 1e-6)
     return {
         "value": 2.0 * M * N * K / step_seconds / 1e12,
         "unit": "TFLOP/s",
@@ -81,6 +96,8 @@ def cpu_baseline(x_bits, w_bits, target_seconds=15.0):
         "sample": f"quantize W[{N},{K}] ({t_qw:.1f} s) + quantize x[:{ms}] ({t_qx:.2f} s) + scaled GEMM of those "
                   f"{ms} rows against all of W ({t_g:.1f} s), {threads} OpenMP threads; whole step extrapolated "
                   f"linearly in rows to {step_seconds:.0f} s",
+        "aten_linear_bf16_on_cpu": {"value": 2.0 * xt.shape[0] * N * K / t_lin / 1e12, "unit": "TFLOP/s", "cores": threads,
+                                    "sample": f"F.linear(x[:{xt.shape[0]}], W) in bf16, {t_lin:.2f} s"},
     }
 
 
