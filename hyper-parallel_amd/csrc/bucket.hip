@@ -66,21 +66,23 @@ __global__ __launch_bounds__(256) void bucket_pack_quant_kernel(const BucketBatc
     }
   }
   const int64_t row_vec0 = b.first_vec[e];
+  static_assert(kBucketUnroll == 4, "scales4_from_amax serves four groups per 16-lane row");
+  uint32_t m[4];
 #pragma unroll
-  for (int u = 0; u < kBucketUnroll; ++u) {
+  for (int u = 0; u < 4; ++u) m[u] = row16_max_u32(mag8(v[u]));
+  const int l16 = threadIdx.x & 15;
+  float s[4], mine, mine_inv;
+  scales4_from_amax(m, l16, 0, s, mine, mine_inv);
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
     const int64_t i = vec0 + u * 256 + threadIdx.x;
-    const uint32_t m = row16_max_u32(mag8(v[u]));
-    float s, si;
-    scales_from_amax(__uint_as_float(m << 16), s, si);
-    if (i < span) {
-      const int64_t rv = row_vec0 + i;                // vector inside the row
-      nt_store8(q + (int64_t)shard * row_elems + rv * 8, cvt8<false>(v[u], s));
-      if ((threadIdx.x & 15) == 0) {
-        const int64_t g = (int64_t)shard * (row_elems >> 7) + (rv >> 4);
-        if (scale) scale[g] = s;
-        scale_inv[g] = si;
-      }
-    }
+    if (i < span) nt_store8(q + (int64_t)shard * row_elems + (row_vec0 + i) * 8, cvt8<false>(v[u], s[u]));   // (row_vec0 + i: vector inside the row)
+  }
+  const int64_t i_mine = vec0 + l16 * 256 + threadIdx.x - l16;   // first vector of the group whose scales this lane holds
+  if (l16 < 4 && i_mine < span) {
+    const int64_t g = (int64_t)shard * (row_elems >> 7) + ((row_vec0 + i_mine) >> 4);
+    if (scale) scale[g] = mine;
+    scale_inv[g] = mine_inv;
   }
 }
 

@@ -85,6 +85,22 @@ __device__ __forceinline__ void scales_from_amax(float amax, float& scale, float
   }
 }
 
+// Scales of the four groups that the 16 lanes of a row share (m[u] = the row's amax bits of group u, the same
+// in all 16 lanes): lane l computes the pair of group l % 4 only, so the divisions run once per lane instead of
+// four times, and every lane receives the four quantize multipliers through quad broadcasts.  mine / mine_inv
+// are the lane's own pair (lanes 0..3 of a row hold groups 0..3).
+__device__ __forceinline__ void scales4_from_amax(const uint32_t m[4], int l16, int pow2, float s[4], float& mine,
+                                                  float& mine_inv) {
+  const int u = l16 & 3;
+  const uint32_t mm = u == 0 ? m[0] : (u == 1 ? m[1] : (u == 2 ? m[2] : m[3]));
+  scales_from_amax(__uint_as_float(mm << 16), mine, mine_inv, pow2);
+  const uint32_t sb = __float_as_uint(mine);
+  s[0] = __uint_as_float(dpp_u32<0x00>(sb));   // quad_perm:[0,0,0,0]
+  s[1] = __uint_as_float(dpp_u32<0x55>(sb));   // quad_perm:[1,1,1,1]
+  s[2] = __uint_as_float(dpp_u32<0xAA>(sb));   // quad_perm:[2,2,2,2]
+  s[3] = __uint_as_float(dpp_u32<0xFF>(sb));   // quad_perm:[3,3,3,3]
+}
+
 __device__ __forceinline__ float clamp448(float y) {
   const float c = __builtin_amdgcn_fmed3f(y, -kFp8Max, kFp8Max);   // of a NaN and two numbers the median instruction returns a number
   return y != y ? y : c;                                            // NaN stays NaN (and is cast to the NaN code)

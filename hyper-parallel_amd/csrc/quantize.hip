@@ -98,19 +98,22 @@ __global__ __launch_bounds__(256) void quant_1x128_kernel(const uint4* __restric
     int64_t i = base + u * 256;
     v[u] = i < nvec ? nt_load16(&x[i]) : make_uint4(0, 0, 0, 0);
   }
+  static_assert(UNROLL == 4, "scales4_from_amax serves four groups per 16-lane row");
+  uint32_t m[4];
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
+  for (int u = 0; u < 4; ++u) m[u] = row16_max_u32(mag8(v[u]));
+  const int l16 = threadIdx.x & 15;
+  float s[4], mine, mine_inv;
+  scales4_from_amax(m, l16, 0, s, mine, mine_inv);
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
     int64_t i = base + u * 256;
-    uint32_t m = row16_max_u32(mag8(v[u]));
-    float s, si;
-    scales_from_amax(__uint_as_float(m << 16), s, si);
-    if (i < nvec) {
-      nt_store8(&q[i], cvt8<false>(v[u], s));
-      if ((threadIdx.x & 15) == 0) {
-        if (scale) scale[i >> 4] = s;
-        scale_inv[i >> 4] = si;
-      }
-    }
+    if (i < nvec) nt_store8(&q[i], cvt8<false>(v[u], s[u]));
+  }
+  const int64_t i_mine = base - l16 + l16 * 256;      // first vector of the group whose scales this lane holds
+  if (l16 < 4 && i_mine < nvec) {
+    if (scale) scale[i_mine >> 4] = mine;
+    scale_inv[i_mine >> 4] = mine_inv;
   }
 }
 
@@ -134,17 +137,19 @@ __global__ __launch_bounds__(256) void quant_1x128_kmajor_kernel(const uint16_t*
     const bool ok = row < rows && g0 + u < groups;
     v[u] = ok ? nt_load16(x + (int64_t)row * cols + (g0 + u) * 128 + l16 * 8) : make_uint4(0, 0, 0, 0);
   }
+  uint32_t m[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) m[u] = row16_max_u32(mag8(v[u]));
+  float s[4], mine, mine_inv;
+  scales4_from_amax(m, l16, pow2, s, mine, mine_inv);
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const bool ok = row < rows && g0 + u < groups;
-    uint32_t m = row16_max_u32(mag8(v[u]));
-    float s, si;
-    scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
-    if (ok) nt_store8(q + (int64_t)row * cols + (g0 + u) * 128 + l16 * 8, cvt8<false>(v[u], s));
-    if (l16 == 0) {
-      s_s[u][r] = s;
-      s_si[u][r] = si;
-    }
+    if (ok) nt_store8(q + (int64_t)row * cols + (g0 + u) * 128 + l16 * 8, cvt8<false>(v[u], s[u]));
+  }
+  if (l16 < 4) {
+    s_s[l16][r] = mine;
+    s_si[l16][r] = mine_inv;
   }
   __syncthreads();
   if (threadIdx.x < 64) {
@@ -224,26 +229,29 @@ __global__ __launch_bounds__(256) void swiglu_quant_1x128_kernel(const uint16_t*
     vg[u] = ok ? nt_load16(src) : make_uint4(0, 0, 0, 0);
     vu[u] = ok ? nt_load16(src + inter) : make_uint4(0, 0, 0, 0);
   }
+  uint4 a[4];
+  uint32_t m[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
-    const bool ok = row < rows && g0 + u < groups;
-    uint4 a;
-    a.x = swiglu2<FAST>(vg[u].x, vu[u].x);
-    a.y = swiglu2<FAST>(vg[u].y, vu[u].y);
-    a.z = swiglu2<FAST>(vg[u].z, vu[u].z);
-    a.w = swiglu2<FAST>(vg[u].w, vu[u].w);
-    const uint32_t m = row16_max_u32(mag8(a));
-    float s, si;
-    scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
-    if (ok) {
+    a[u].x = swiglu2<FAST>(vg[u].x, vu[u].x);
+    a[u].y = swiglu2<FAST>(vg[u].y, vu[u].y);
+    a[u].z = swiglu2<FAST>(vg[u].z, vu[u].z);
+    a[u].w = swiglu2<FAST>(vg[u].w, vu[u].w);
+    m[u] = row16_max_u32(mag8(a[u]));
+  }
+  float s[4], mine, mine_inv;
+  scales4_from_amax(m, l16, pow2, s, mine, mine_inv);
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    if (row < rows && g0 + u < groups) {
       const int64_t o = (int64_t)row * inter + (g0 + u) * 128 + l16 * 8;
-      nt_store8(q + o, cvt8<false>(a, s));
-      if (act) nt_store16(act + o, a);
+      nt_store8(q + o, cvt8<false>(a[u], s[u]));
+      if (act) nt_store16(act + o, a[u]);
     }
-    if (l16 == 0) {
-      s_s[u][r] = s;
-      s_si[u][r] = si;
-    }
+  }
+  if (l16 < 4) {
+    s_s[l16][r] = mine;
+    s_si[l16][r] = mine_inv;
   }
   __syncthreads();
   if (threadIdx.x < 64) {
@@ -435,15 +443,21 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
     if (DUAL) {
       // the 16 threads of a row quad hold a whole 128-column group of each of their 8 rows
 #pragma unroll
-      for (int p = 0; p < 8; ++p) {
-        const int row = tile_row(rq, p);
-        const uint32_t mr = row16_max_u32(mag8(v[p]));
-        float s, si;
-        scales_from_amax(__uint_as_float(mr << 16), s, si, pow2);
-        *reinterpret_cast<uint2*>(q + ((int64_t)tr * 128 + row) * k + tc * 128 + cg * 8) = cvt8<false>(v[p], s);
-        if (cg == 0) {
-          s_row[row] = s;
-          s_row[128 + row] = si;
+      for (int half = 0; half < 2; ++half) {
+        uint32_t mr[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) mr[p] = row16_max_u32(mag8(v[4 * half + p]));
+        float s[4], mine, mine_inv;
+        scales4_from_amax(mr, cg, pow2, s, mine, mine_inv);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const int row = tile_row(rq, 4 * half + p);
+          *reinterpret_cast<uint2*>(q + ((int64_t)tr * 128 + row) * k + tc * 128 + cg * 8) = cvt8<false>(v[4 * half + p], s[p]);
+        }
+        if (cg < 4) {
+          const int row = tile_row(rq, 4 * half + cg);
+          s_row[row] = mine;
+          s_row[128 + row] = mine_inv;
         }
       }
     }
