@@ -544,3 +544,32 @@ def test_activation_matrix_larger_than_2_gib(gpu):
         assert torch.equal(y[r0:r0 + 256], part), r0
     ref = ref_f64_torch(a[M - 256:], sa[M - 256:], wq, sw.repeat_interleave(128, dim=0), gpu)
     assert rel(U.f32(y[M - 256:]), ref.cpu().numpy()) < TOL_BF16
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_output_matrix_larger_than_4_gib(gpu, out_dtype):
+    """A tile's stores are addressed relative to the tile's first element (32-bit offsets inside the tile,
+    64-bit base), so c as a whole may exceed 4 GiB: rows whose byte offset lies beyond 2^32 hold the same
+    bits as the same rows computed on their own, and the accumulate form adds onto them in place."""
+    import hpfp8
+    f32 = out_dtype == torch.float32
+    M, N, K = (33024, 36864, 128) if f32 else (65792, 36864, 128)      # c is 4.5 GiB either way
+    g = torch.Generator(device=gpu).manual_seed(11)
+    a = torch.randint(0, 0x7F, (M, K), generator=g, device=gpu, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    sa = (torch.rand((1, M), generator=g, device=gpu) + 0.5).t()
+    w = (torch.randn((N, K), generator=g, device=gpu) * 0.01).to(torch.bfloat16)
+    wq, sw = hpfp8.quantize_128x128(w)
+    y = hpfp8.gemm_blockwise(a, sa, wq, sw, out_dtype=out_dtype)
+    assert y.numel() * y.element_size() > (1 << 32)
+    first_beyond = (1 << 32) // (N * y.element_size())                 # the row that contains byte 2^32
+    for r0 in (0, first_beyond - 128, M - 256, M - 100):
+        part = hpfp8.gemm_blockwise(a[r0:r0 + 256], sa[r0:r0 + 256], wq, sw, out_dtype=out_dtype)
+        assert torch.equal(y[r0:r0 + 256], part), r0
+    ref = ref_f64_torch(a[M - 256:], sa[M - 256:], wq, sw.repeat_interleave(128, dim=0), gpu)
+    assert rel(U.f32(y[M - 256:].float()), ref.cpu().numpy()) < (TOL_F32 if f32 else TOL_BF16)
+    if f32:
+        w1, sw1 = hpfp8.quantize_1x128(w, kmajor=True)
+        before = y[M - 256:].clone()
+        add = hpfp8.gemm_blockwise(a[M - 256:], sa[M - 256:], w1, sw1, sb_gran=1, out_dtype=torch.float32)
+        hpfp8.gemm_blockwise(a, sa, w1, sw1, sb_gran=1, out=y, accumulate=True)
+        assert rel(U.f32(y[M - 256:]), U.f32(before + add)) < 1e-6
