@@ -440,3 +440,47 @@ def test_dequantize_accumulate_into_fp32_main_grad(gpu):
     again = hpfp8.dequantize_1x128_accumulate(q, si, got, grad_scale=1.0)
     want2 = O.dequantize_1x128_accumulate(U.codes(q), U.f32(si), want, 1.0)
     assert np.array_equal(U.f32_bits(U.f32(again)), U.f32_bits(want2))
+
+
+def test_tensors_beyond_2_31_elements(gpu):
+    """4.3 GB of bf16 (2.15e9 elements): element offsets no longer fit 32 bits.  Every quantizer gives, on
+    row blocks at the start, across the 2^31-element mark and at the end, the bits it gives for those rows
+    passed on their own; the last rows are also checked against the oracle."""
+    import hpfp8
+    rows, cols = 300032, 7168                        # 2344 x 128 rows
+    g = torch.Generator(device=gpu).manual_seed(3)
+    x = torch.empty((rows, cols), dtype=torch.bfloat16, device=gpu)
+    for r in range(0, rows, 37504):                  # filled in pieces: no 8.6 GB fp32 temporary
+        x[r:r + 37504] = torch.randn((37504, cols), generator=g, device=gpu).to(torch.bfloat16)
+    assert x.numel() > (1 << 31)
+    cross = ((1 << 31) // cols) // 128 * 128         # the 128-row block that contains element 2^31
+    blocks = (0, cross, rows - 128)
+    u8 = lambda t: t.view(torch.uint8)
+    for kmajor in (False, True):
+        q, s, si = hpfp8.quantize_1x128(x, want_scale=True, kmajor=kmajor)
+        for r0 in blocks:
+            pq, ps, psi = hpfp8.quantize_1x128(x[r0:r0 + 128], want_scale=True, kmajor=kmajor)
+            assert torch.equal(u8(q[r0:r0 + 128]), u8(pq)) and torch.equal(si[r0:r0 + 128], psi) and torch.equal(s[r0:r0 + 128], ps)
+    rq, rs, rsi = O.quantize_1x128(U.bits(x[rows - 128:]))
+    assert np.array_equal(U.codes(q[rows - 128:]), rq) and eq_f32(si[rows - 128:], rsi)
+    back = hpfp8.dequantize_1x128(q, si.contiguous())
+    assert np.array_equal(U.bits(back[rows - 128:]), O.dequantize_1x128(rq, rsi))
+    del q, s, si, back
+    q, si, qt, s = hpfp8.quantize_128x128(x, with_transpose=True, want_scale=True)
+    for r0 in blocks:
+        pq, psi, pqt, ps = hpfp8.quantize_128x128(x[r0:r0 + 128], with_transpose=True, want_scale=True)
+        assert torch.equal(u8(q[r0:r0 + 128]), u8(pq)) and torch.equal(si[r0 // 128], psi[0]) and torch.equal(s[r0 // 128], ps[0])
+        assert torch.equal(u8(qt[:, r0:r0 + 128]), u8(pqt))
+    del q, si, qt, s
+    for kmajor in (False, True):
+        q1, si1, qt, sit = hpfp8.quantize_1x128_and_128x1_t(x, kmajor=kmajor)
+        for r0 in blocks:
+            p1, psi1, pqt, psit = hpfp8.quantize_1x128_and_128x1_t(x[r0:r0 + 128], kmajor=kmajor)
+            assert torch.equal(u8(q1[r0:r0 + 128]), u8(p1)) and torch.equal(si1[r0:r0 + 128], psi1)
+            assert torch.equal(u8(qt[:, r0:r0 + 128]), u8(pqt)) and torch.equal(sit[:, r0 // 128], psit[:, 0])
+        del q1, si1, qt, sit
+    qt, sit = hpfp8.quantize_128x1_t(x, kmajor=True)
+    rqt, _, rsit = O.quantize_128x1_t(U.bits(x[rows - 128:]))
+    assert np.array_equal(U.codes(qt[:, rows - 128:]), rqt) and eq_f32(sit[:, -1], rsit[:, 0])
+    am = hpfp8.amax(x)
+    assert float(am) == float(x.view(torch.int16).bitwise_and(0x7FFF).max().view(torch.bfloat16).float())
