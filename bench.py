@@ -144,6 +144,22 @@ def other_configs(dev):
                                      _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True)))
     res["cfg2_swiglu_quantize_fast"] = gb(4096 * 18432 * 5 + 4096 * (18432 // 128) * 4,
                                           _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True, fast=True)))
+    # the whole dense-MLP block forward: gate/up linear, SwiGLU, down linear [7168 <- 18432]
+    import torch.nn.functional as F
+    wd_bf16 = (torch.randn((7168, 18432), device=dev) * 0.006).to(torch.bfloat16)
+    wgu_bf16 = (torch.randn((36864, 7168), device=dev) * 0.006).to(torch.bfloat16)
+    x_mlp = torch.randn((4096, 7168), device=dev).to(torch.bfloat16)
+    gu_q, dn_q = hpfp8.quantize_weight(wgu_bf16, with_transpose=False), hpfp8.quantize_weight(wd_bf16, with_transpose=False)
+
+    def torch_mlp():
+        h = F.linear(x_mlp, wgu_bf16)
+        return F.linear(F.silu(h[:, :18432]) * h[:, 18432:], wd_bf16)
+    mlp_flop = 2.0 * 4096 * 7168 * (36864 + 18432)
+    t_fp8 = _time(lambda: hpfp8.fp8_swiglu_mlp(x_mlp, gu_q, dn_q, fast=True), iters=20)
+    t_bf16 = _time(torch_mlp, iters=20)
+    res["cfg2_mlp_block_forward"] = {"fp8_ms": t_fp8, "TFLOP/s": mlp_flop / t_fp8 / 1e9, "torch_bf16_ms": t_bf16,
+                                     "note": "weights prequantized; x quantize + 2 GEMMs + fused SwiGLU/quantize (fast form)"}
+    del wd_bf16, wgu_bf16, x_mlp, gu_q, dn_q
     del hgu
     # cfg 2 as a training step of the module: forward + backward through fp8_linear (the weight's FP8 form
     # made beforehand, as Fp8Linear's cache does), beside torch's bf16 F.linear on the same tensors

@@ -283,3 +283,27 @@ def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Te
     e, n, k = weight.shape
     wq, sw = ops.quantize_128x128(weight.reshape(e * n, k))
     return ops.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), offs)
+
+
+def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True) -> torch.Tensor:
+    """Forward of a SwiGLU MLP block (DeepSeekV3 dense MLP; inference, no autograd graph is recorded):
+    ``F.linear(F.silu(gate) * up, w_down)`` with ``gate | up = F.linear(input, w_gate_up)`` -- in the
+    reference two aten::linear calls dispatched at hyper_parallel/core/shard/_op_dispatch.py:277-283 with
+    eager bf16 elementwise ops between them.  Here the activation is computed and quantized for the down
+    projection in one pass over the gate/up output, and never exists in bf16.
+
+    w_gate_up [2I, K] (gate rows first) and w_down [N, I]: bf16 tensors or `Fp8Weight`s (quantized once,
+    e.g. by `quantize_weight(w, with_transpose=False)`).  ``fast`` selects the SwiGLU kernel that uses the
+    hardware exponential and reciprocal."""
+    gu = w_gate_up if isinstance(w_gate_up, Fp8Weight) else quantize_weight(w_gate_up.detach(), with_transpose=False)
+    dn = w_down if isinstance(w_down, Fp8Weight) else quantize_weight(w_down.detach(), with_transpose=False)
+    inter = gu.codes.shape[0] // 2
+    if gu.codes.shape[0] % (2 * ops.BLOCK) or dn.codes.shape[1] != inter:
+        raise ValueError("w_gate_up must be [2I, K] with I a multiple of 128 and w_down [N, I]")
+    with torch.no_grad():
+        x2 = _flatten(input)
+        xq, sx = ops.quantize_1x128(x2, kmajor=True, pow2=gu.pow2)
+        h = ops.gemm_blockwise(xq, sx, gu.codes, gu.scale_inv, pow2_scales=gu.pow2)
+        aq, sa = ops.swiglu_quantize_1x128(h, kmajor=True, pow2=dn.pow2, fast=fast)
+        y = ops.gemm_blockwise(aq, sa, dn.codes, dn.scale_inv, pow2_scales=dn.pow2)
+    return y.reshape(input.shape[:-1] + (dn.codes.shape[0],))

@@ -262,3 +262,35 @@ def test_policy_record_and_fp8_cast_hook(gpu):
     w = U.randn_bf16((256, 384), 92, 0.02).to(gpu).requires_grad_(True)
     hpfp8.fp8_linear(x, w, **pol.linear_kwargs()).backward(U.randn_bf16((256, 256), 93, 1e-3).to(gpu))
     assert w.grad is None and w.main_grad.dtype == torch.float32
+
+
+@pytest.mark.parametrize("fast", [False, True])
+def test_swiglu_mlp_forward(gpu, fast):
+    """The fused MLP forward is the chain of its parts bit for bit (quantize, GEMM, SwiGLU + quantize, GEMM),
+    prequantized weights give the same output as bf16 weights, and the result stays within FP8 quantization
+    noise of torch's bf16 MLP."""
+    import hpfp8
+    import torch.nn.functional as F
+    g = torch.Generator(device="cpu").manual_seed(4)
+    m, k, inter, n = 384, 512, 768, 640
+    x = torch.randn((2, m // 2, k), generator=g).to(torch.bfloat16).to(gpu)
+    wgu = (torch.randn((2 * inter, k), generator=g) * 0.05).to(torch.bfloat16).to(gpu)
+    wd = (torch.randn((n, inter), generator=g) * 0.05).to(torch.bfloat16).to(gpu)
+    y = hpfp8.fp8_swiglu_mlp(x, wgu, wd, fast=fast)
+    assert y.shape == (2, m // 2, n) and y.dtype == torch.bfloat16 and not y.requires_grad
+    # the chain of its parts
+    xq, sx = hpfp8.quantize_1x128(x.reshape(m, k), kmajor=True)
+    gq, gs = hpfp8.quantize_128x128(wgu)
+    dq, ds = hpfp8.quantize_128x128(wd)
+    h = hpfp8.gemm_blockwise(xq, sx, gq, gs)
+    aq, sa = hpfp8.swiglu_quantize_1x128(h, kmajor=True, fast=fast)
+    want = hpfp8.gemm_blockwise(aq, sa, dq, ds)
+    assert torch.equal(y.reshape(m, n), want)
+    y2 = hpfp8.fp8_swiglu_mlp(x, hpfp8.quantize_weight(wgu, with_transpose=False), hpfp8.quantize_weight(wd, with_transpose=False), fast=fast)
+    assert torch.equal(y, y2)
+    hr = F.linear(x, wgu)
+    ref = F.linear(F.silu(hr[..., :inter]) * hr[..., inter:], wd)
+    err = float((y.float() - ref.float()).norm() / ref.float().norm())
+    assert err < 0.08, err
+    with pytest.raises(ValueError):
+        hpfp8.fp8_swiglu_mlp(x, wgu, wd[:, :640])
