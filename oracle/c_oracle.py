@@ -48,6 +48,12 @@ def lib():
         l.hpo_gemm_blockwise.argtypes = [_u8p, _f32p, _u8p, _f32p, _i64, _i64, _i64, ctypes.c_int,
                                          _f32p, _f32p, _u16p]
         l.hpo_num_threads.restype = ctypes.c_int
+        l.hpo_scales_pow2.argtypes = [ctypes.c_float, _f32p, _f32p]
+        l.hpo_scales_pow2.restype = None
+        l.hpo_exp_spec.argtypes = [ctypes.c_float]
+        l.hpo_exp_spec.restype = ctypes.c_float
+        l.hpo_swiglu.argtypes = [_u16p, _i64, _i64, _u16p]
+        l.hpo_swiglu.restype = None
         for name in ("hpo_quantize_per_tensor", "hpo_quantize_1x128", "hpo_quantize_128x128",
                      "hpo_quantize_128x1_t", "hpo_dequantize_1x128", "hpo_gemm_blockwise"):
             getattr(l, name).restype = None
@@ -135,3 +141,30 @@ def gemm_blockwise(a, sa_inv, b, sb_inv, sb_per_row=False, bias_f32=None):
                              int(bool(sb_per_row)), None if bias is None else _p(bias, _f32p),
                              _p(out, _f32p), _p(out_b, _u16p))
     return out, out_b
+
+
+def scales_pow2(amax: np.ndarray):
+    """(scale, scale_inv) of the power-of-two recipe for every amax of an array."""
+    l = lib()
+    flat = _c(amax, np.float32).reshape(-1)
+    s = np.empty(flat.size, np.float32)
+    si = np.empty(flat.size, np.float32)
+    a, b = ctypes.c_float(), ctypes.c_float()
+    for i, v in enumerate(flat):
+        l.hpo_scales_pow2(float(v), ctypes.byref(a), ctypes.byref(b))
+        s[i], si[i] = a.value, b.value
+    return s.reshape(np.shape(amax)), si.reshape(np.shape(amax))
+
+
+def exp_spec(t: np.ndarray) -> np.ndarray:
+    l = lib()
+    flat = _c(t, np.float32).reshape(-1)
+    return np.array([l.hpo_exp_spec(float(v)) for v in flat], dtype=np.float32).reshape(np.shape(t))
+
+
+def swiglu(h_bits: np.ndarray) -> np.ndarray:
+    h = _c(h_bits, np.uint16)
+    rows, w2 = h.shape
+    act = np.empty((rows, w2 // 2), np.uint16)
+    lib().hpo_swiglu(_p(h, _u16p), rows, w2 // 2, _p(act, _u16p))
+    return act

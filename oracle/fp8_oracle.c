@@ -3,8 +3,8 @@
  *
  * It is a second, independently written implementation of the arithmetic in fp8_oracle.py (the
  * E4M3 encoder here rounds with nearbyintf on a scaled magnitude instead of integer bit
- * tricks), so the two pin each other bit for bit; both are pinned to torch's float8_e4m3fn
- * cast by tests/test_oracle_pins.py.
+ * tricks, the power-of-two scales come from frexpf / ldexpf instead of exponent-field arithmetic), so the
+ * two pin each other bit for bit; both are pinned to torch's float8_e4m3fn cast by tests/test_oracle_pins.py.
  *
  * The reference checkout has no FP8 arithmetic.  The recipe follows the benchmark
  * configuration text (scale = 448/amax, E4M3 cast, fp32 accumulation, bf16 output, 1x128 /
@@ -207,6 +207,60 @@ void hpo_gemm_blockwise(const uint8_t* a, const float* sa_inv, const uint8_t* b,
     free(arow);
     free(brow);
   }
+}
+
+/* Power-of-two scales (the optional recipe): scale_inv = the smallest power of two >= max(amax, eps) / 448,
+ * found with frexpf instead of the exponent-field arithmetic of the Python form; scale = 1 / scale_inv.
+ * NaN and Inf pass through unchanged. */
+void hpo_scales_pow2(float amax, float* scale, float* scale_inv) {
+  float amc = amax < kAmaxEps ? kAmaxEps : amax;
+  float si = amc / kFp8Max;
+  if (!isnan(si) && !isinf(si)) {
+    int e;
+    float f = frexpf(si, &e);            /* si = f * 2^e, f in [0.5, 1) */
+    si = (f == 0.5f) ? si : ldexpf(1.0f, e);
+  }
+  *scale_inv = si;
+  *scale = 1.0f / si;
+}
+
+/* exp(t) as the SwiGLU kernel defines it, one IEEE fp32 operation per step (no contraction: see the build
+ * flags), written with the C library's rounding, scaling and ordered-comparison routines where the Python form
+ * uses array operations and exponent-field arithmetic. */
+float hpo_exp_spec(float t) {
+  volatile float r, p, kk;
+  float k;
+  if (t < -86.0f) t = -86.0f;            /* (a NaN passes both comparisons and stays) */
+  if (t > 89.0f) t = 89.0f;
+  k = nearbyintf(t * 1.44269504f);
+  kk = k * 0.693359375f;
+  r = t - kk;
+  kk = k * -2.12194440e-4f;
+  r = r - kk;
+  p = 1.0f / 720.0f;
+  {
+    const float c[6] = {1.0f / 120.0f, 1.0f / 24.0f, 1.0f / 6.0f, 0.5f, 1.0f, 1.0f};
+    for (int i = 0; i < 6; ++i) {
+      p = p * r;
+      p = p + c[i];
+    }
+  }
+  p = p * ldexpf(1.0f, (int)k - 1);      /* k - 1 >= -125: a normal number */
+  return p * 2.0f;
+}
+
+/* act = bf16(bf16(silu(gate)) * up), h[rows, 2 * inter] = gate | up, silu(g) = g / (1 + exp_spec(-g)) */
+void hpo_swiglu(const uint16_t* h, int64_t rows, int64_t inter, uint16_t* act) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t c = 0; c < inter; ++c) {
+      float g = bf16_to_f32(h[r * 2 * inter + c]), u = bf16_to_f32(h[r * 2 * inter + inter + c]);
+      volatile float den = 1.0f + hpo_exp_spec(-g);
+      volatile float s = g / den;
+      float sb = bf16_to_f32(f32_to_bf16(s));
+      volatile float prod = sb * u;
+      act[r * inter + c] = f32_to_bf16(prod);
+    }
 }
 
 int hpo_num_threads(void) {

@@ -48,7 +48,10 @@ How each function is pinned (tests/test_oracle_pins.py)
       implementation compared bit for bit.
   scales_from_amax(pow2)    : closed form (a power of two, >= amax/448 and < 2 amax/448, times its
       reciprocal exactly 1, no product beyond 448); the quantizers with it are the ordinary ones
-      with that scale (scalar loop with torch's cast); not in the C restatement.
+      with that scale (scalar loop with torch's cast); the C restatement derives the same scales from
+      frexpf / ldexpf.
+  exp_spec, swiglu          : numpy's exp and torch's eager F.silu(gate) * up within their rounding; the C
+      restatement (nearbyintf, ldexpf, scalar loop) bit for bit.
   gemm_*                    : torch._scaled_mm on CPU for per-tensor scales (library routine);
       exact integer-valued inputs with unit scales reduce to an exact integer matmul; the
       grouped variant equals a loop of dense calls; float64 dequant matmul bounds the rest.

@@ -475,3 +475,24 @@ def test_swiglu_restatement_against_numpy_and_torch():
     diff = np.abs(mine.astype(np.int32) - ref_bits.astype(np.int32))
     same_sign_zero = (mine & 0x7FFF) + (ref_bits & 0x7FFF) == 0
     assert ((diff <= 1) | same_sign_zero).all() and (diff != 0).mean() < 2e-3
+
+
+def test_c_restatement_of_pow2_scales_and_swiglu_bit_exact():
+    """Second implementations written differently (frexpf / ldexpf / nearbyintf and scalar loops against
+    exponent-field arithmetic and array operations): power-of-two scales, the specified exponential, and
+    the SwiGLU activation agree bit for bit."""
+    rng = np.random.default_rng(0)
+    am = np.concatenate([np.float32(2.0) ** rng.integers(-60, 60, 300) * rng.uniform(0.5, 2, 300).astype(np.float32),
+                         np.float32([0, 1e-13, 1e-12, 448, 224, 448 * 2.0 ** -20, 3.39e38, np.inf, np.nan,
+                                     447.99997, 448.00003])]).astype(np.float32)
+    s, si = O.scales_from_amax(am, pow2=True)
+    cs, csi = C.scales_pow2(am)
+    assert U.same_f32_or_nan(s, cs) and U.same_f32_or_nan(si, csi)
+    t = np.concatenate([rng.uniform(-100, 100, 20000), rng.normal(0, 3, 20000),
+                        [0, -0.0, 88.5, -88.5, 89, -86, 88.72284, 1e-30, np.inf, -np.inf]]).astype(np.float32)
+    with np.errstate(all="ignore"):
+        a, b = O.exp_spec(t), C.exp_spec(t)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    h = U.randn_bf16((64, 512), 5, 2.0, 0.01, 30.0)
+    h[0, :6] = torch.tensor([0.0, -0.0, 88.5, -88.5, -200.0, 200.0], dtype=torch.bfloat16)
+    assert np.array_equal(O.swiglu(U.bits(h)), C.swiglu(U.bits(h)))
