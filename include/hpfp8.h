@@ -213,11 +213,11 @@ int hpfp8_bucket_unpack_dequantize_bf16(void* const* grads, const int64_t* numel
  *                 then be k-block-major: sb_stride_n = 1, sb_stride_k >= N (what the *_kmajor quantizers write)
  * bias: bf16[N] or NULL.  out_type HPFP8_OUT_BF16 / HPFP8_OUT_F32; ldc = row stride of c in
  * elements, a multiple of 8 (bf16) or 4 (fp32): rows are written in 16-byte pieces.  Scale strides are
- * non-negative; each scale array must span less than 2 GiB and a row stride of a or b stay below 8 MiB
- * (HPFP8_ERR_SHAPE otherwise); the code matrices themselves may be of any size.  accumulate != 0 (fp32 output only) adds onto c instead of overwriting it, the fp32
- * main-grad bookkeeping of hyper_parallel/platform/torch/fully_shard/param.py:134-167: the old value of
- * an element is the starting value of its sum, the k-blocks are added onto it in ascending order (c's row
- * stride must then stay below 8 MiB). */
+ * non-negative; each scale array must span less than 2 GiB and a row stride of a, b or c stay below 8 MiB
+ * (HPFP8_ERR_SHAPE otherwise); the code matrices and c themselves may be of any size.  accumulate != 0
+ * (fp32 output only) adds onto c instead of overwriting it, the fp32 main-grad bookkeeping of
+ * hyper_parallel/platform/torch/fully_shard/param.py:134-167: the old value of an element is the starting
+ * value of its sum, the k-blocks are added onto it in ascending order. */
 int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                          const void* b, int64_t ldb, const float* sb, int64_t sb_stride_n, int64_t sb_stride_k,
                          int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
