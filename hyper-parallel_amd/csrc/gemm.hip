@@ -736,14 +736,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 // Workgroups to launch for `tiles` tiles: one per CU, a multiple of 8 (one share per XCD) unless
 // there are fewer than 8 tiles.
 static int persistent_grid(int64_t tiles) {
-  static int cus = 0;
-  if (cus == 0) {
+  static const int cus = [] {           // (initialised once, also when the first calls come from several threads)
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
       n = 256;
-    cus = n;
-  }
+    return n;
+  }();
   int64_t g = tiles < cus ? tiles : cus;
   if (g >= kXcds) g -= g % kXcds;
   return (int)g;
