@@ -68,8 +68,8 @@ class Fp8GradBucket:
             raise ValueError(f"expected {len(self.numels)} tensors, got {len(tensors)}")
         ptrs = (ctypes.c_void_p * max(len(tensors), 1))()
         for e, (t, n) in enumerate(zip(tensors, per_tensor_elems)):
-            if not t.is_cuda or t.dtype != torch.bfloat16 or not t.is_contiguous():
-                raise TypeError(f"gradient {e} must be a contiguous bfloat16 GPU tensor")
+            if not t.is_cuda or t.device.index != torch.cuda.current_device() or t.dtype != torch.bfloat16 or not t.is_contiguous():
+                raise TypeError(f"gradient {e} must be a contiguous bfloat16 tensor on the current GPU")
             if t.numel() != n:
                 raise ValueError(f"gradient {e} has {t.numel()} elements, expected {n}")
             ptrs[e] = t.data_ptr()

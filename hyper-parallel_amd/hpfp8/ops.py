@@ -28,11 +28,20 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
+def _check_device(x: torch.Tensor, name: str) -> None:
+    """Kernels are launched on the current device and its current stream: a tensor that lives on another
+    GPU must be used under ``torch.cuda.device(x.device)``."""
+    if not x.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {x.device}); this path has no CPU fallback")
+    if x.device.index != torch.cuda.current_device():
+        raise ValueError(f"{name} lives on {x.device} but the current device is cuda:{torch.cuda.current_device()}; "
+                         f"call under torch.cuda.device({name}.device)")
+
+
 def _check_bf16(x: torch.Tensor, name: str, contiguous: bool = True) -> torch.Tensor:
     if not isinstance(x, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor")
-    if not x.is_cuda:
-        raise ValueError(f"{name} must live on the GPU (got device {x.device}); this path has no CPU fallback")
+    _check_device(x, name)
     if x.dtype != torch.bfloat16:
         raise TypeError(f"{name} must be bfloat16, got {x.dtype}")
     if not contiguous:
@@ -41,8 +50,7 @@ def _check_bf16(x: torch.Tensor, name: str, contiguous: bool = True) -> torch.Te
 
 
 def _check_fp8(x: torch.Tensor, name: str) -> torch.Tensor:
-    if not x.is_cuda:
-        raise ValueError(f"{name} must live on the GPU")
+    _check_device(x, name)
     if x.dtype not in (FP8, torch.uint8):
         raise TypeError(f"{name} must be float8_e4m3fn (or uint8 codes), got {x.dtype}")
     if not x.is_contiguous():
@@ -52,8 +60,7 @@ def _check_fp8(x: torch.Tensor, name: str) -> torch.Tensor:
 
 def _check_codes_2d(x: torch.Tensor, name: str) -> torch.Tensor:
     """A GEMM operand: 2-D codes with unit inner stride; the row stride may exceed the row length."""
-    if not x.is_cuda:
-        raise ValueError(f"{name} must live on the GPU")
+    _check_device(x, name)
     if x.dtype not in (FP8, torch.uint8):
         raise TypeError(f"{name} must be float8_e4m3fn (or uint8 codes), got {x.dtype}")
     if x.dim() != 2 or (x.shape[1] > 1 and x.stride(1) != 1) or (x.shape[0] > 1 and x.stride(0) % 16):
@@ -77,8 +84,9 @@ def _empty_codes_t(rows: int, cols: int, device) -> torch.Tensor:
 
 
 def _check_f32(x: torch.Tensor, name: str) -> torch.Tensor:
-    if not x.is_cuda or x.dtype != torch.float32:
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32:
         raise TypeError(f"{name} must be a float32 GPU tensor")
+    _check_device(x, name)
     return x
 
 
