@@ -159,7 +159,24 @@ def other_configs(dev):
     t_bf16 = _time(torch_mlp, iters=20)
     res["cfg2_mlp_block_forward"] = {"fp8_ms": t_fp8, "TFLOP/s": mlp_flop / t_fp8 / 1e9, "torch_bf16_ms": t_bf16,
                                      "note": "weights prequantized; x quantize + 2 GEMMs + fused SwiGLU/quantize (fast form)"}
-    del wd_bf16, wgu_bf16, x_mlp, gu_q, dn_q
+    # the same block in training: forward + backward (weights quantized inside, as in an optimizer step)
+    xg_, wgu_p, wd_p = x_mlp.clone().requires_grad_(True), wgu_bf16.clone().requires_grad_(True), wd_bf16.clone().requires_grad_(True)
+    go_mlp = (torch.randn((4096, 7168), device=dev) * 1e-3).to(torch.bfloat16)
+
+    def fp8_train():
+        hpfp8.fp8_swiglu_mlp(xg_, wgu_p, wd_p).backward(go_mlp)
+        xg_.grad = wgu_p.grad = wd_p.grad = None
+
+    def bf16_train():
+        h = F.linear(xg_, wgu_p)
+        F.linear(F.silu(h[:, :18432]) * h[:, 18432:], wd_p).backward(go_mlp)
+        xg_.grad = wgu_p.grad = wd_p.grad = None
+    t_fp8 = _time(fp8_train, iters=10, warm=15)
+    t_bf16 = _time(bf16_train, iters=10, warm=15)
+    res["cfg2_mlp_block_forward_backward"] = {"fp8_ms": t_fp8, "TFLOP/s": 3 * mlp_flop / t_fp8 / 1e9, "torch_bf16_ms": t_bf16}
+    dact = torch.randn((4096, 18432), device=dev).to(torch.bfloat16)
+    res["cfg2_swiglu_backward"] = gb(4096 * 18432 * 10, _time(lambda: hpfp8.ops.swiglu_backward(hgu, dact)))
+    del wd_bf16, wgu_bf16, x_mlp, gu_q, dn_q, xg_, wgu_p, wd_p, go_mlp, dact
     del hgu
     # cfg 2 as a training step of the module: forward + backward through fp8_linear (the weight's FP8 form
     # made beforehand, as Fp8Linear's cache does), beside torch's bf16 F.linear on the same tensors

@@ -264,6 +264,66 @@ __global__ __launch_bounds__(256) void swiglu_quant_1x128_kernel(const uint16_t*
   }
 }
 
+// Backward of act = silu(gate) * up for two (gate, up, d act) triples packed like their sources:
+//   d up   = d act * bf16(silu(g))                (the rounded silu is what forward multiplied with)
+//   d gate = d act * up * (sig + silu * (1 - sig)),  sig = 1 / (1 + exp(-g)), silu = g * sig
+// in fp32 with the hardware's base-2 exponential and reciprocal, each result rounded to bf16 once.
+__device__ __forceinline__ void swiglu_bwd2(uint32_t gw, uint32_t uw, uint32_t dw, uint32_t& dgw, uint32_t& duw) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const float g[2] = {bf16lo(gw), bf16hi(gw)}, u[2] = {bf16lo(uw), bf16hi(uw)}, d[2] = {bf16lo(dw), bf16hi(dw)};
+  float sig[2], silu[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    sig[t] = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g[t] * -1.44269504f));
+    silu[t] = g[t] * sig[t];
+  }
+  const f32x2 sf = {silu[0], silu[1]};
+  const uint32_t sw = __builtin_bit_cast(uint32_t, __builtin_convertvector(sf, bf16x2));
+  const f32x2 du = {d[0] * bf16lo(sw), d[1] * bf16hi(sw)};
+  const f32x2 dg = {(d[0] * u[0]) * (sig[0] + silu[0] * (1.0f - sig[0])), (d[1] * u[1]) * (sig[1] + silu[1] * (1.0f - sig[1]))};
+  duw = __builtin_bit_cast(uint32_t, __builtin_convertvector(du, bf16x2));
+  dgw = __builtin_bit_cast(uint32_t, __builtin_convertvector(dg, bf16x2));
+}
+
+// h[rows, 2 * inter] (row stride ld_h), dact[rows, inter] -> dh[rows, 2 * inter] (row stride ld_dh) = d gate | d up.
+// One 16-byte vector of 8 activations per thread and step; three streams in, two out.
+__global__ __launch_bounds__(256) void swiglu_backward_kernel(const uint16_t* __restrict__ h, int64_t ld_h,
+                                                              const uint16_t* __restrict__ dact,
+                                                              uint16_t* __restrict__ dh, int64_t ld_dh, int64_t nvec,
+                                                              int inter) {
+  const int vec_per_row = inter >> 3;
+  constexpr int UNROLL = 2;
+  const int64_t base = (int64_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  uint4 vg[UNROLL], vu[UNROLL], vd[UNROLL];
+  int64_t row[UNROLL];
+  int col[UNROLL];
+#pragma unroll
+  for (int k = 0; k < UNROLL; ++k) {
+    const int64_t i = base + k * 256;
+    const bool ok = i < nvec;
+    row[k] = ok ? i / vec_per_row : 0;
+    col[k] = ok ? (int)(i - row[k] * vec_per_row) * 8 : 0;
+    const uint16_t* src = h + row[k] * ld_h + col[k];
+    vg[k] = ok ? nt_load16(src) : make_uint4(0, 0, 0, 0);
+    vu[k] = ok ? nt_load16(src + inter) : make_uint4(0, 0, 0, 0);
+    vd[k] = ok ? nt_load16(dact + row[k] * (int64_t)inter + col[k]) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int k = 0; k < UNROLL; ++k) {
+    uint4 dg, du;
+    swiglu_bwd2(vg[k].x, vu[k].x, vd[k].x, dg.x, du.x);
+    swiglu_bwd2(vg[k].y, vu[k].y, vd[k].y, dg.y, du.y);
+    swiglu_bwd2(vg[k].z, vu[k].z, vd[k].z, dg.z, du.z);
+    swiglu_bwd2(vg[k].w, vu[k].w, vd[k].w, dg.w, du.w);
+    if (base + k * 256 < nvec) {
+      uint16_t* dst = dh + row[k] * ld_dh + col[k];
+      nt_store16(dst, dg);
+      nt_store16(dst + inter, du);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // shared by the two tile kernels below: 128x128 tile, 256 threads
 // ---------------------------------------------------------------------------------------------
@@ -856,6 +916,26 @@ int hpfp8_swiglu_quantize_1x128_fast_bf16(const void* h, int64_t rows, int64_t i
                                           void* q, float* scale, float* scale_inv, void* act, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(pow2 == 0 || pow2 == 1, HPFP8_ERR_ARG, "swiglu_quantize_1x128_fast: pow2 must be 0 or 1");
   return swiglu_quantize_impl(h, rows, inter, ld_h, kmajor, q, scale, scale_inv, act, pow2, 1, stream);
+}
+
+int hpfp8_swiglu_backward_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, const void* dact, void* dh,
+                               int64_t ld_dh, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "swiglu_backward: negative shape");
+  HPFP8_REQUIRE(inter % 8 == 0, HPFP8_ERR_SHAPE, "swiglu_backward: width %lld is not a multiple of 8", (long long)inter);
+  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 30), HPFP8_ERR_SHAPE, "swiglu_backward: dimension too large");
+  if (rows == 0 || inter == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(ld_h >= 2 * inter && ld_h % 8 == 0 && ld_dh >= 2 * inter && ld_dh % 8 == 0, HPFP8_ERR_SHAPE,
+                "swiglu_backward: ld_h=%lld and ld_dh=%lld must be multiples of 8 and at least twice the width",
+                (long long)ld_h, (long long)ld_dh);
+  HPFP8_REQUIRE(h && dact && dh, HPFP8_ERR_ARG, "swiglu_backward: null buffer");
+  HPFP8_REQUIRE(aligned16(h) && aligned16(dact) && aligned16(dh), HPFP8_ERR_ALIGN,
+                "swiglu_backward: buffers must be 16-byte aligned");
+  const int64_t nvec = rows * (inter / 8);
+  const int64_t blocks = (nvec + 511) / 512;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "swiglu_backward: tensor too large");
+  swiglu_backward_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t*)h, ld_h, (const uint16_t*)dact,
+                                                                           (uint16_t*)dh, ld_dh, nvec, (int)inter);
+  return check_launch("swiglu_backward");
 }
 
 int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld, void* q_t, int64_t ld_t,

@@ -285,16 +285,75 @@ def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Te
     return ops.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), offs)
 
 
-def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True) -> torch.Tensor:
-    """Forward of a SwiGLU MLP block (DeepSeekV3 dense MLP; inference, no autograd graph is recorded):
-    ``F.linear(F.silu(gate) * up, w_down)`` with ``gate | up = F.linear(input, w_gate_up)`` -- in the
-    reference two aten::linear calls dispatched at hyper_parallel/core/shard/_op_dispatch.py:277-283 with
-    eager bf16 elementwise ops between them.  Here the activation is computed and quantized for the down
-    projection in one pass over the gate/up output, and never exists in bf16.
+class _Fp8SwiGLUDown(torch.autograd.Function):
+    """y = F.linear(silu(gate) * up, w_down) for h = [gate | up] (blockwise recipe): the activation is computed and
+    quantized for the GEMM in one pass over h; backward quantizes grad_out once for both of its GEMMs, rebuilds
+    the activation's transposed 128x1 codes from the saved h, and ends with the gradient of SwiGLU itself."""
 
-    w_gate_up [2I, K] (gate rows first) and w_down [N, I]: bf16 tensors or `Fp8Weight`s (quantized once,
-    e.g. by `quantize_weight(w, with_transpose=False)`).  ``fast`` selects the SwiGLU kernel that uses the
-    hardware exponential and reciprocal."""
+    @staticmethod
+    def forward(ctx, h, weight, fast=True):
+        h2 = _flatten(h)
+        aq, sa = ops.swiglu_quantize_1x128(h2, kmajor=True, fast=fast)
+        if h.requires_grad:
+            wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
+        else:
+            wq, sw = ops.quantize_128x128(weight)
+            wqt = None
+        y = ops.gemm_blockwise(aq, sa, wq, sw)
+        ctx.save_for_backward(h2, wqt, sw)
+        ctx.fast = fast
+        ctx.h_shape = h.shape
+        ctx.need = (h.requires_grad, weight.requires_grad)
+        return y.reshape(h.shape[:-1] + (weight.shape[0],))
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        h2, wqt, sw = ctx.saved_tensors
+        need_dh, need_dw = ctx.need
+        go = _flatten(grad_out)
+        if go.dtype != torch.bfloat16:
+            go = go.to(torch.bfloat16)
+        go = go.contiguous()
+        m = go.shape[0]
+        if need_dw and m % ops.BLOCK:
+            raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
+        dh = dw = None
+        goq = sgo = got = sgot = None
+        if need_dh and need_dw:
+            goq, sgo, got, sgot = ops.quantize_1x128_and_128x1_t(go, kmajor=True)
+        elif need_dh:
+            goq, sgo = ops.quantize_1x128(go, kmajor=True)
+        elif need_dw:
+            got, sgot = ops.quantize_128x1_t(go, kmajor=True)
+        if need_dw:
+            # the activation again (bf16 this time), for its 128x1 codes along the tokens
+            _, _, act = ops.swiglu_quantize_1x128(h2, kmajor=True, want_act=True, fast=ctx.fast)
+            at, sat = ops.quantize_128x1_t(act, kmajor=True)
+            del act
+            dw = ops.gemm_blockwise(got, sgot, at, sat, sb_gran=1)
+        if need_dh:
+            dact = ops.gemm_blockwise(goq, sgo, wqt, sw.t())
+            dh = ops.swiglu_backward(h2, dact).reshape(ctx.h_shape)
+        return dh, dw, None
+
+
+def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True) -> torch.Tensor:
+    """A SwiGLU MLP block (DeepSeekV3 dense MLP): ``F.linear(F.silu(gate) * up, w_down)`` with
+    ``gate | up = F.linear(input, w_gate_up)`` -- in the reference two aten::linear calls dispatched at
+    hyper_parallel/core/shard/_op_dispatch.py:277-283 with eager bf16 elementwise ops between them.  Here the
+    activation is computed and quantized for the down projection in one pass over the gate/up output, and
+    never exists in bf16 in forward.
+
+    w_gate_up [2I, K] (gate rows first) and w_down [N, I]: bf16 tensors, or `Fp8Weight`s (quantized once,
+    e.g. by `quantize_weight(w, with_transpose=False)`) for inference.  With bf16 weights and gradients
+    enabled the result carries an autograd graph (blockwise recipe).  ``fast`` selects the SwiGLU kernel that
+    uses the hardware exponential and reciprocal."""
+    fp8_weights = isinstance(w_gate_up, Fp8Weight) or isinstance(w_down, Fp8Weight)
+    if not fp8_weights and torch.is_grad_enabled() and (input.requires_grad or w_gate_up.requires_grad or w_down.requires_grad):
+        if w_gate_up.shape[0] % (2 * ops.BLOCK) or w_down.shape[1] != w_gate_up.shape[0] // 2:
+            raise ValueError("w_gate_up must be [2I, K] with I a multiple of 128 and w_down [N, I]")
+        h = fp8_linear(input, w_gate_up)
+        return _Fp8SwiGLUDown.apply(h, w_down, fast)
     gu = w_gate_up if isinstance(w_gate_up, Fp8Weight) else quantize_weight(w_gate_up.detach(), with_transpose=False)
     dn = w_down if isinstance(w_down, Fp8Weight) else quantize_weight(w_down.detach(), with_transpose=False)
     inter = gu.codes.shape[0] // 2

@@ -213,6 +213,21 @@ def swiglu_quantize_1x128(h: torch.Tensor, kmajor: bool = True, want_act: bool =
     return (q, s_inv, act) if want_act else (q, s_inv)
 
 
+def swiglu_backward(h: torch.Tensor, dact: torch.Tensor) -> torch.Tensor:
+    """Gradient of act = silu(gate) * up with respect to h = [gate | up]: h[M, 2I], dact[M, I] -> dh[M, 2I], bf16."""
+    h = _check_bf16(h, "h", contiguous=False)
+    dact = _check_bf16(dact, "dact")
+    if h.dim() != 2 or h.shape[1] % 16 or dact.shape != (h.shape[0], h.shape[1] // 2):
+        raise ValueError("h must be [M, 2I] with I a multiple of 8 and dact [M, I]")
+    if h.stride(1) != 1 or h.stride(0) % 8 or h.data_ptr() % 16:
+        h = h.contiguous()
+    m, inter = dact.shape
+    dh = torch.empty((m, 2 * inter), dtype=torch.bfloat16, device=h.device)
+    _lib.call("hpfp8_swiglu_backward_bf16", _ptr(h), m, inter, h.stride(0) if m > 1 else 2 * inter, _ptr(dact), _ptr(dh),
+              2 * inter, _stream())
+    return dh
+
+
 def transpose_codes(q: torch.Tensor) -> torch.Tensor:
     """codes[R, C] -> codes_t[C, R] (byte transpose; R, C multiples of 128).  With 128x128 scaling blocks
     the transposed codes of a weight are its dgrad operand, scales reused with swapped strides."""

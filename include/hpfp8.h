@@ -151,6 +151,14 @@ int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter,
 int hpfp8_swiglu_quantize_1x128_fast_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, int pow2,
                                           void* q, float* scale, float* scale_inv, void* act, hpfp8_stream_t stream);
 
+/* Backward of act = silu(gate) * up (the autograd of the same eager graph): h[rows, 2 * inter] = gate | up as in the
+ * forward call, dact[rows, inter] the gradient of act (contiguous), dh[rows, 2 * inter] (row stride ld_dh) receives
+ * d gate | d up, all bf16:  d up = dact * bf16(silu(gate)),  d gate = dact * up * (sig + silu * (1 - sig)) with
+ * sig = 1 / (1 + exp(-gate)) from the hardware's exponential and reciprocal, in fp32, one rounding each.
+ * inter a multiple of 8. */
+int hpfp8_swiglu_backward_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, const void* dact, void* dh,
+                               int64_t ld_dh, hpfp8_stream_t stream);
+
 /* Byte transpose of a code matrix: q[rows, cols] (row stride ld) -> q_t[cols, rows] (row stride ld_t);
  * rows, cols multiples of 128.  128x128 scaling blocks are symmetric, so this turns the codes of a
  * weight into its dgrad operand without requantizing, e.g. after FP8 shards were all-gathered: the

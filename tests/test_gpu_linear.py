@@ -294,3 +294,66 @@ def test_swiglu_mlp_forward(gpu, fast):
     assert err < 0.08, err
     with pytest.raises(ValueError):
         hpfp8.fp8_swiglu_mlp(x, wgu, wd[:, :640])
+
+
+def test_swiglu_backward_kernel_vs_torch_autograd(gpu):
+    """d gate | d up of the kernel against autograd of the same function evaluated in fp32 (results rounded
+    to bf16 once on both sides): equal up to bf16 rounding of values that differ in the last bits of fp32;
+    a strided h gives the same bits."""
+    import hpfp8
+    m, inter = 300, 1024
+    h = U.randn_bf16((m, 2 * inter), 7, 2.0, 0.001, 20.0).to(gpu)
+    h[0, :4] = torch.tensor([0.0, -0.0, 30.0, -30.0], dtype=torch.bfloat16)
+    da = U.randn_bf16((m, inter), 8, 1e-2).to(gpu)
+    dh = hpfp8.ops.swiglu_backward(h, da)
+    assert dh.shape == (m, 2 * inter) and dh.dtype == torch.bfloat16
+    g = h[:, :inter].float().requires_grad_(True)
+    u = h[:, inter:].float()
+    F.silu(g).backward(da.float() * u)                                  # d gate = (d act * up) * silu'(gate), all fp32
+    dg_ref = g.grad.to(torch.bfloat16)
+    silu_b = F.silu(h[:, :inter].float()).to(torch.bfloat16).float()   # forward multiplied up with the rounded silu
+    du_f32 = da.float() * silu_b
+    du_ref = du_f32.to(torch.bfloat16)
+    # one bf16 step, or -- where silu' passes through zero (gate near -1.28) and its two terms cancel -- an
+    # absolute error far below one step of the factor d act * up that it scales
+    scale = (da.float() * u).abs()
+    for got, want, slack in ((dh[:, :inter], dg_ref, 1e-3 * scale), (dh[:, inter:], du_ref, 0 * scale)):
+        d = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        small = (got.float() - want.float()).abs() <= slack + 1e-30
+        # (d up: where the bf16 rounding of silu is a near-tie decided the other way, one step there is up to two here)
+        assert bool(((d <= 2) | small).all()) and float(((d > 1) & ~small).float().mean()) < 1e-4
+        assert float(((d != 0) & ~small).float().mean()) < 0.02
+    assert rel(dh[:, :inter], g.grad) < 5e-3 and rel(dh[:, inter:], du_f32) < 5e-3
+    wide = torch.zeros((m, 2 * inter + 64), dtype=torch.bfloat16, device=gpu)
+    wide[:, :2 * inter] = h
+    assert torch.equal(hpfp8.ops.swiglu_backward(wide[:, :2 * inter], da), dh)
+    with pytest.raises(ValueError):
+        hpfp8.ops.swiglu_backward(h, da[:, :512])
+
+
+def test_swiglu_mlp_training_step_vs_torch(gpu):
+    """Forward and the three gradients of the MLP block against torch's fp32 autograd of the same graph, within
+    FP8 quantization noise; the forward value equals the inference path's bit for bit."""
+    import hpfp8
+    g = torch.Generator(device="cpu").manual_seed(5)
+    m, k, inter, n = 256, 512, 640, 384
+    x = torch.randn((2, m // 2, k), generator=g).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    wgu = (torch.randn((2 * inter, k), generator=g) * 0.05).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    wd = (torch.randn((n, inter), generator=g) * 0.05).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    go = (torch.randn((2, m // 2, n), generator=g) * 1e-2).to(torch.bfloat16).to(gpu)
+    y = hpfp8.fp8_swiglu_mlp(x, wgu, wd)
+    assert y.requires_grad and y.shape == (2, m // 2, n)
+    with torch.no_grad():
+        assert torch.equal(y, hpfp8.fp8_swiglu_mlp(x, wgu, wd))
+    y.backward(go)
+    gx, ggu, gd = x.grad.clone(), wgu.grad.clone(), wd.grad.clone()
+    x.grad = wgu.grad = wd.grad = None
+    hr = F.linear(x.float(), wgu.float())
+    yr = F.linear(F.silu(hr[..., :inter]) * hr[..., inter:], wd.float())
+    yr.backward(go.float())
+    assert rel(y, yr) < 0.08 and rel(gx, x.grad) < 0.1 and rel(ggu, wgu.grad) < 0.1 and rel(gd, wd.grad) < 0.08
+    # only the input needs a gradient (frozen weights)
+    x2 = x.detach().clone().requires_grad_(True)
+    y2 = hpfp8.fp8_swiglu_mlp(x2, wgu.detach(), wd.detach())
+    y2.backward(go)
+    assert torch.equal(y2, y) and rel(x2.grad, gx) < 1e-6
