@@ -291,14 +291,16 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
     the activation's transposed 128x1 codes from the saved h, and ends with the gradient of SwiGLU itself."""
 
     @staticmethod
-    def forward(ctx, h, weight, fast=True):
+    def forward(ctx, h, weight, fast=True, wq=None, sw=None, wqt=None):
         h2 = _flatten(h)
         aq, sa = ops.swiglu_quantize_1x128(h2, kmajor=True, fast=fast)
-        if h.requires_grad:
-            wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
-        else:
-            wq, sw = ops.quantize_128x128(weight)
-            wqt = None
+        if wq is None:                          # no prequantized form of the weight was passed in
+            if h.requires_grad:
+                wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
+            else:
+                wq, sw = ops.quantize_128x128(weight)
+        elif h.requires_grad and wqt is None:
+            wqt = ops.transpose_codes(wq)
         y = ops.gemm_blockwise(aq, sa, wq, sw)
         ctx.save_for_backward(h2, wqt, sw)
         ctx.fast = fast
@@ -334,10 +336,11 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
         if need_dh:
             dact = ops.gemm_blockwise(goq, sgo, wqt, sw.t())
             dh = ops.swiglu_backward(h2, dact).reshape(ctx.h_shape)
-        return dh, dw, None
+        return dh, dw, None, None, None, None
 
 
-def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True) -> torch.Tensor:
+def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True,
+                   gate_up_fp8: Optional[Fp8Weight] = None, down_fp8: Optional[Fp8Weight] = None) -> torch.Tensor:
     """A SwiGLU MLP block (DeepSeekV3 dense MLP): ``F.linear(F.silu(gate) * up, w_down)`` with
     ``gate | up = F.linear(input, w_gate_up)`` -- in the reference two aten::linear calls dispatched at
     hyper_parallel/core/shard/_op_dispatch.py:277-283 with eager bf16 elementwise ops between them.  Here the
@@ -346,16 +349,24 @@ def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True)
 
     w_gate_up [2I, K] (gate rows first) and w_down [N, I]: bf16 tensors, or `Fp8Weight`s (quantized once,
     e.g. by `quantize_weight(w, with_transpose=False)`) for inference.  With bf16 weights and gradients
-    enabled the result carries an autograd graph (blockwise recipe).  ``fast`` selects the SwiGLU kernel that
-    uses the hardware exponential and reciprocal."""
+    enabled the result carries an autograd graph (blockwise recipe); ``gate_up_fp8`` / ``down_fp8`` are then the
+    weights' FP8 forms made earlier by `quantize_weight` (e.g. once per optimizer step for all its micro-batches),
+    as `fp8_linear`'s ``weight_fp8``.  ``fast`` selects the SwiGLU kernel that uses the hardware exponential and
+    reciprocal."""
     fp8_weights = isinstance(w_gate_up, Fp8Weight) or isinstance(w_down, Fp8Weight)
     if not fp8_weights and torch.is_grad_enabled() and (input.requires_grad or w_gate_up.requires_grad or w_down.requires_grad):
         if w_gate_up.shape[0] % (2 * ops.BLOCK) or w_down.shape[1] != w_gate_up.shape[0] // 2:
             raise ValueError("w_gate_up must be [2I, K] with I a multiple of 128 and w_down [N, I]")
-        h = fp8_linear(input, w_gate_up)
-        return _Fp8SwiGLUDown.apply(h, w_down, fast)
-    gu = w_gate_up if isinstance(w_gate_up, Fp8Weight) else quantize_weight(w_gate_up.detach(), with_transpose=False)
-    dn = w_down if isinstance(w_down, Fp8Weight) else quantize_weight(w_down.detach(), with_transpose=False)
+        for f8 in (gate_up_fp8, down_fp8):
+            if f8 is not None and f8.pow2:
+                raise ValueError("the training path of fp8_swiglu_mlp uses the blockwise recipe with plain fp32 scales")
+        h = fp8_linear(input, w_gate_up, weight_fp8=gate_up_fp8)
+        d8 = down_fp8
+        if d8 is not None and d8.codes.shape != w_down.shape:
+            raise ValueError("down_fp8 does not belong to w_down")
+        return _Fp8SwiGLUDown.apply(h, w_down, fast, *((d8.codes, d8.scale_inv, d8.codes_t) if d8 is not None else ()))
+    gu = w_gate_up if isinstance(w_gate_up, Fp8Weight) else (gate_up_fp8 or quantize_weight(w_gate_up.detach(), with_transpose=False))
+    dn = w_down if isinstance(w_down, Fp8Weight) else (down_fp8 or quantize_weight(w_down.detach(), with_transpose=False))
     inter = gu.codes.shape[0] // 2
     if gu.codes.shape[0] % (2 * ops.BLOCK) or dn.codes.shape[1] != inter:
         raise ValueError("w_gate_up must be [2I, K] with I a multiple of 128 and w_down [N, I]")

@@ -352,6 +352,13 @@ def test_swiglu_mlp_training_step_vs_torch(gpu):
     yr = F.linear(F.silu(hr[..., :inter]) * hr[..., inter:], wd.float())
     yr.backward(go.float())
     assert rel(y, yr) < 0.08 and rel(gx, x.grad) < 0.1 and rel(ggu, wgu.grad) < 0.1 and rel(gd, wd.grad) < 0.08
+    # weights quantized ahead of the step: same bits
+    wgu.grad = wd.grad = None
+    x3 = x.detach().clone().requires_grad_(True)
+    y3 = hpfp8.fp8_swiglu_mlp(x3, wgu, wd, gate_up_fp8=hpfp8.quantize_weight(wgu), down_fp8=hpfp8.quantize_weight(wd))
+    y3.backward(go)
+    assert torch.equal(y3, y) and torch.equal(x3.grad, gx) and torch.equal(wgu.grad, ggu) and torch.equal(wd.grad, gd)
+    wgu.grad = wd.grad = None
     # only the input needs a gradient (frozen weights)
     x2 = x.detach().clone().requires_grad_(True)
     y2 = hpfp8.fp8_swiglu_mlp(x2, wgu.detach(), wd.detach())
