@@ -484,3 +484,26 @@ def test_tensors_beyond_2_31_elements(gpu):
     assert np.array_equal(U.codes(qt[:, rows - 128:]), rqt) and eq_f32(sit[:, -1], rsit[:, 0])
     am = hpfp8.amax(x)
     assert float(am) == float(x.view(torch.int16).bitwise_and(0x7FFF).max().view(torch.bfloat16).float())
+    del qt, sit
+    # the remaining entry points: per-tensor cast, 128x128 dequantize, byte transpose, SwiGLU forms
+    q, s, si = hpfp8.quantize_per_tensor(x)
+    pq, _, _ = hpfp8.quantize_per_tensor(x[rows - 128:], amax_in=am)
+    assert torch.equal(u8(q[rows - 128:]), u8(pq)) and float(si) == float(np.float32(float(am)) / np.float32(448.0))
+    del q
+    q, si = hpfp8.quantize_128x128(x)
+    back = hpfp8.dequantize_128x128(q, si)
+    qt = hpfp8.transpose_codes(q)
+    for r0 in blocks:
+        pq, psi = hpfp8.quantize_128x128(x[r0:r0 + 128])
+        assert torch.equal(back[r0:r0 + 128], hpfp8.dequantize_128x128(pq, psi))
+        assert torch.equal(u8(qt[:, r0:r0 + 128]), u8(hpfp8.transpose_codes(pq)))
+    del q, si, back, qt
+    for fast in (False, True):
+        q, si, act = hpfp8.swiglu_quantize_1x128(x, kmajor=True, want_act=True, fast=fast)
+        for r0 in blocks:
+            pq, psi, pact = hpfp8.swiglu_quantize_1x128(x[r0:r0 + 128], kmajor=True, want_act=True, fast=fast)
+            assert torch.equal(u8(q[r0:r0 + 128]), u8(pq)) and torch.equal(si[r0:r0 + 128], psi) and torch.equal(act[r0:r0 + 128], pact)
+        del q, si
+    dh = hpfp8.ops.swiglu_backward(x, act)
+    for r0 in blocks:
+        assert torch.equal(dh[r0:r0 + 128], hpfp8.ops.swiglu_backward(x[r0:r0 + 128], act[r0:r0 + 128]))
