@@ -573,3 +573,30 @@ def test_output_matrix_larger_than_4_gib(gpu, out_dtype):
         add = hpfp8.gemm_blockwise(a[M - 256:], sa[M - 256:], w1, sw1, sb_gran=1, out_dtype=torch.float32)
         hpfp8.gemm_blockwise(a, sa, w1, sw1, sb_gran=1, out=y, accumulate=True)
         assert rel(U.f32(y[M - 256:]), U.f32(before + add)) < 1e-6
+
+
+def test_weight_matrix_larger_than_2_gib(gpu):
+    """The b operand beyond 2^31 bytes (dense, and as the stacked weights of a grouped call): columns of c
+    that belong to weight rows past that mark equal the same rows passed on their own."""
+    import hpfp8
+    M, N, K = 256, 327680, 7168                      # b is 2.19 GiB
+    g = torch.Generator(device=gpu).manual_seed(12)
+    b = torch.randint(0, 0x7F, (N, K), generator=g, device=gpu, dtype=torch.uint8)
+    b |= torch.randint(0, 2, (N, K), generator=g, device=gpu, dtype=torch.uint8) << 7
+    b = b.view(torch.float8_e4m3fn)
+    sb = torch.rand((N // 128, K // 128), generator=g, device=gpu) + 0.5
+    x = torch.randn((M, K), generator=g, device=gpu).to(torch.bfloat16)
+    xq, sx = hpfp8.quantize_1x128(x, kmajor=True)
+    y = hpfp8.gemm_blockwise(xq, sx, b, sb)
+    for n0 in (0, 299520, N - 256):                  # 299520 * 7168 is just below 2^31
+        part = hpfp8.gemm_blockwise(xq, sx, b[n0:n0 + 256], sb[n0 // 128:n0 // 128 + 2])
+        assert torch.equal(y[:, n0:n0 + 256], part), n0
+    ref = ref_f64_torch(xq, sx, b[N - 256:], sb[(N - 256) // 128:].repeat_interleave(128, dim=0), gpu)
+    assert rel(U.f32(y[:, N - 256:]), ref.cpu().numpy()) < TOL_BF16
+    # the same bytes as 80 experts of 4096 rows each: the last expert's weights lie beyond 2^31
+    E, Ne = 80, 4096
+    offs = torch.zeros(E, dtype=torch.int32, device=gpu)
+    offs[-2:] = torch.tensor([100, M], dtype=torch.int32)       # experts 0..77 empty, 78 gets 100 rows, 79 the rest
+    yg = hpfp8.gemm_grouped_blockwise(xq, sx, b.view(E, Ne, K), sb.view(E, Ne // 128, K // 128), offs)
+    assert torch.equal(yg[:100], hpfp8.gemm_blockwise(xq[:100], sx[:100], b[78 * Ne:79 * Ne], sb[78 * 32:79 * 32]))
+    assert torch.equal(yg[100:], hpfp8.gemm_blockwise(xq[100:], sx[100:], b[79 * Ne:], sb[79 * 32:]))
