@@ -144,6 +144,8 @@ def other_configs(dev):
                                      _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True)))
     res["cfg2_swiglu_quantize_fast"] = gb(4096 * 18432 * 5 + 4096 * (18432 // 128) * 4,
                                           _time(lambda: hpfp8.swiglu_quantize_1x128(hgu, kmajor=True, fast=True)))
+    res["cfg2_swiglu_quantize_both_forms_fast"] = gb(4096 * 18432 * 6 + 2 * 4096 * (18432 // 128) * 4, _time(
+        lambda: hpfp8.ops.swiglu_quantize_1x128_and_128x1_t(hgu, fast=True)))
     # the whole dense-MLP block forward: gate/up linear, SwiGLU, down linear [7168 <- 18432]
     import torch.nn.functional as F
     wd_bf16 = (torch.randn((7168, 18432), device=dev) * 0.006).to(torch.bfloat16)

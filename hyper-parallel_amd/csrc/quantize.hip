@@ -451,8 +451,12 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // With DUAL the same pass also writes the 1x128 quantization of x itself (codes q[M,K], one scale per
 // row and 128 columns: [M, K/128], or [K/128, M] with KMAJOR): forward / dgrad operand and wgrad
 // operand from one read of the bf16 source.
-template <bool KMAJOR, bool DUAL>
-__global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int m, int k,
+// With SW (1: exactly specified silu, 2: hardware exponential and reciprocal) the source is h[M, 2K] = gate | up
+// and what is quantized is act = silu(gate) * up, computed as the tile is loaded: both operand forms of the
+// down projection's input from one read of the gate/up output, the bf16 activation never written.
+// ld_src: row stride of the source in elements (K, or at least 2K with SW).
+template <bool KMAJOR, bool DUAL, int SW = 0>
+__global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int m, int k,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale_t,
                                                             float* __restrict__ scale_inv_t,
@@ -472,9 +476,19 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
   const int t1 = t0 + kTilesPerBlock < total ? t0 + kTilesPerBlock : total;
   auto load_tile = [&](int t, uint4 v[8]) {
     const int tc = t / mb, tr = t % mb;
-    const int64_t off = (int64_t)tr * 128 * k + tc * 128 + cg * 8;
+    const int64_t off = (int64_t)tr * 128 * ld_src + tc * 128 + cg * 8;
 #pragma unroll
-    for (int p = 0; p < 8; ++p) v[p] = nt_load16(x + off + (int64_t)tile_row(rq, p) * k);
+    for (int p = 0; p < 8; ++p) v[p] = nt_load16(x + off + (int64_t)tile_row(rq, p) * ld_src);
+    if (SW) {
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const uint4 u = nt_load16(x + off + (int64_t)tile_row(rq, p) * ld_src + k);
+        v[p].x = swiglu2<SW == 2>(v[p].x, u.x);
+        v[p].y = swiglu2<SW == 2>(v[p].y, u.y);
+        v[p].z = swiglu2<SW == 2>(v[p].z, u.z);
+        v[p].w = swiglu2<SW == 2>(v[p].w, u.w);
+      }
+    }
   };
   uint4 v[8], vn[8];
   load_tile(t0, v);
@@ -831,15 +845,43 @@ static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, i
   uint8_t* q8 = (uint8_t*)q;
   if (q) {
     if (kmajor)
-      quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
+      quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
     else
-      quant_128x1_t_kernel<false, true><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
+      quant_128x1_t_kernel<false, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
   } else {
     if (kmajor)
-      quant_128x1_t_kernel<true, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
+      quant_128x1_t_kernel<true, false><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
     else
-      quant_128x1_t_kernel<false, false><<<grid, 256, 0, s>>>(xs, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
+      quant_128x1_t_kernel<false, false><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
   }
+  return check_launch(what);
+}
+
+int hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int fast,
+                                                 void* q, float* scale, float* scale_inv, void* q_t, int64_t ld_t,
+                                                 float* scale_t, float* scale_inv_t, hpfp8_stream_t stream) {
+  const char* what = "swiglu_quantize_1x128_and_128x1_t";
+  HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
+  HPFP8_REQUIRE(rows % kBlock == 0 && inter % kBlock == 0, HPFP8_ERR_SHAPE,
+                "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)rows, (long long)inter);
+  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 30), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
+  const int64_t blocks = (rows / kBlock) * (inter / kBlock);
+  if (blocks == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
+  HPFP8_REQUIRE(h && q && scale_inv && q_t && scale_inv_t, HPFP8_ERR_ARG, "%s: null buffer", what);
+  HPFP8_REQUIRE(aligned16(h) && aligned16(q) && aligned16(q_t), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
+  HPFP8_REQUIRE(ld_h >= 2 * inter && ld_h % 8 == 0, HPFP8_ERR_SHAPE,
+                "%s: ld_h=%lld must be a multiple of 8 and at least twice the width", what, (long long)ld_h);
+  HPFP8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, HPFP8_ERR_SHAPE, "%s: ld_t=%lld must be a multiple of 16 and at least rows",
+                what, (long long)ld_t);
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned grid = (unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock);
+  if (fast)
+    quant_128x1_t_kernel<true, true, 2><<<grid, 256, 0, s>>>((const uint16_t*)h, ld_h, (int)rows, (int)inter, (uint8_t*)q_t, ld_t,
+                                                            scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0);
+  else
+    quant_128x1_t_kernel<true, true, 1><<<grid, 256, 0, s>>>((const uint16_t*)h, ld_h, (int)rows, (int)inter, (uint8_t*)q_t, ld_t,
+                                                            scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0);
   return check_launch(what);
 }
 

@@ -287,13 +287,21 @@ def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Te
 
 class _Fp8SwiGLUDown(torch.autograd.Function):
     """y = F.linear(silu(gate) * up, w_down) for h = [gate | up] (blockwise recipe): the activation is computed and
-    quantized for the GEMM in one pass over h; backward quantizes grad_out once for both of its GEMMs, rebuilds
-    the activation's transposed 128x1 codes from the saved h, and ends with the gradient of SwiGLU itself."""
+    quantized for the GEMM in one pass over h, which also makes the activation's transposed 128x1 codes for wgrad;
+    backward quantizes grad_out once for both of its GEMMs and ends with the gradient of SwiGLU itself."""
 
     @staticmethod
     def forward(ctx, h, weight, fast=True, wq=None, sw=None, wqt=None):
         h2 = _flatten(h)
-        aq, sa = ops.swiglu_quantize_1x128(h2, kmajor=True, fast=fast)
+        m = h2.shape[0]
+        # With a weight gradient to come and a token count that allows it, the gate/up output is read once for
+        # both forms of the activation: its 1x128 codes for this GEMM and its transposed 128x1 codes, kept for wgrad.
+        fused = weight.requires_grad and m % ops.BLOCK == 0 and m > 0
+        if fused:
+            aq, sa, at, sat = ops.swiglu_quantize_1x128_and_128x1_t(h2, fast=fast)
+        else:
+            aq, sa = ops.swiglu_quantize_1x128(h2, kmajor=True, fast=fast)
+            at = sat = None
         if wq is None:                          # no prequantized form of the weight was passed in
             if h.requires_grad:
                 wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True)
@@ -302,7 +310,7 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
         elif h.requires_grad and wqt is None:
             wqt = ops.transpose_codes(wq)
         y = ops.gemm_blockwise(aq, sa, wq, sw)
-        ctx.save_for_backward(h2, wqt, sw)
+        ctx.save_for_backward(h2 if h.requires_grad or (weight.requires_grad and not fused) else None, wqt, sw, at, sat)
         ctx.fast = fast
         ctx.h_shape = h.shape
         ctx.need = (h.requires_grad, weight.requires_grad)
@@ -310,7 +318,7 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_out):
-        h2, wqt, sw = ctx.saved_tensors
+        h2, wqt, sw, at, sat = ctx.saved_tensors
         need_dh, need_dw = ctx.need
         go = _flatten(grad_out)
         if go.dtype != torch.bfloat16:
@@ -328,10 +336,11 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
         elif need_dw:
             got, sgot = ops.quantize_128x1_t(go, kmajor=True)
         if need_dw:
-            # the activation again (bf16 this time), for its 128x1 codes along the tokens
-            _, _, act = ops.swiglu_quantize_1x128(h2, kmajor=True, want_act=True, fast=ctx.fast)
-            at, sat = ops.quantize_128x1_t(act, kmajor=True)
-            del act
+            if at is None:
+                # the activation again (bf16 this time), for its 128x1 codes along the tokens
+                _, _, act = ops.swiglu_quantize_1x128(h2, kmajor=True, want_act=True, fast=ctx.fast)
+                at, sat = ops.quantize_128x1_t(act, kmajor=True)
+                del act
             dw = ops.gemm_blockwise(got, sgot, at, sat, sb_gran=1)
         if need_dh:
             dact = ops.gemm_blockwise(goq, sgo, wqt, sw.t())

@@ -213,6 +213,25 @@ def swiglu_quantize_1x128(h: torch.Tensor, kmajor: bool = True, want_act: bool =
     return (q, s_inv, act) if want_act else (q, s_inv)
 
 
+def swiglu_quantize_1x128_and_128x1_t(h: torch.Tensor, fast: bool = False):
+    """Both quantized forms of act = silu(gate) * up from one read of h[M, 2I] = gate | up:
+    (codes[M, I], scale_inv[M, I/128], codes_t[I, M], scale_inv_t[I, M/128]), k-block-major scales, bit-identical to
+    ``swiglu_quantize_1x128(h, fast=fast)`` and to ``quantize_128x1_t`` of its activation.  M and I multiples of 128."""
+    h = _check_bf16(h, "h", contiguous=False)
+    if h.dim() != 2 or h.shape[1] % (2 * BLOCK) or h.shape[0] % BLOCK:
+        raise ValueError("h must be [M, 2I] with M and I multiples of 128")
+    if h.stride(1) != 1 or h.stride(0) % 8 or h.data_ptr() % 16:
+        h = h.contiguous()
+    m, inter = h.shape[0], h.shape[1] // 2
+    q = torch.empty((m, inter), dtype=FP8, device=h.device)
+    qt = _empty_codes_t(inter, m, h.device)
+    s_inv = torch.empty((inter // BLOCK, m), dtype=torch.float32, device=h.device)
+    st_inv = torch.empty((m // BLOCK, inter), dtype=torch.float32, device=h.device)
+    _lib.call("hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16", _ptr(h), m, inter, h.stride(0) if m > 1 else 2 * inter,
+              int(fast), _ptr(q), None, _ptr(s_inv), _ptr(qt), _ld(qt), None, _ptr(st_inv), _stream())
+    return q, s_inv.t(), qt, st_inv.t()
+
+
 def swiglu_backward(h: torch.Tensor, dact: torch.Tensor) -> torch.Tensor:
     """Gradient of act = silu(gate) * up with respect to h = [gate | up]: h[M, 2I], dact[M, I] -> dh[M, 2I], bf16."""
     h = _check_bf16(h, "h", contiguous=False)

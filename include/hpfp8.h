@@ -151,6 +151,16 @@ int hpfp8_swiglu_quantize_1x128_bf16(const void* h, int64_t rows, int64_t inter,
 int hpfp8_swiglu_quantize_1x128_fast_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int kmajor, int pow2,
                                           void* q, float* scale, float* scale_inv, void* act, hpfp8_stream_t stream);
 
+/* SwiGLU fused with both quantized forms of its result (training: the down projection's forward operand and
+ * its wgrad operand from one read of the gate/up output; the bf16 activation is never written): the results of
+ * hpfp8_swiglu_quantize_1x128_bf16 (fast == 0) or _fast_bf16 (fast != 0) with k-block-major scales
+ * (q[rows, inter], scale / scale_inv [inter/128, rows]) and of hpfp8_quantize_128x1_t_kmajor_bf16 applied to that
+ * activation (q_t[inter, rows] with row stride ld_t, scale_t / scale_inv_t [rows/128, inter]), bit for bit.
+ * rows and inter multiples of 128. */
+int hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, int fast,
+                                                 void* q, float* scale, float* scale_inv, void* q_t, int64_t ld_t,
+                                                 float* scale_t, float* scale_inv_t, hpfp8_stream_t stream);
+
 /* Backward of act = silu(gate) * up (the autograd of the same eager graph): h[rows, 2 * inter] = gate | up as in the
  * forward call, dact[rows, inter] the gradient of act (contiguous), dh[rows, 2 * inter] (row stride ld_dh) receives
  * d gate | d up, all bf16:  d up = dact * bf16(silu(gate)),  d gate = dact * up * (sig + silu * (1 - sig)) with

@@ -428,6 +428,34 @@ def test_swiglu_fast_form(gpu, pow2):
     assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and U.same_f32_or_nan(U.f32(si2), U.f32(si))
 
 
+@pytest.mark.parametrize("fast", [False, True])
+def test_swiglu_with_both_quantized_forms(gpu, fast):
+    """One read of the gate/up output gives the 1x128 codes and the transposed 128x1 codes of the activation:
+    bit for bit what the SwiGLU quantizer and the transposing quantizer of its bf16 activation give (and, in
+    the exact form, what the oracle gives); a strided source gives the same."""
+    import hpfp8
+    h = U.randn_bf16((256, 1536), 6, 2.0, 0.001, 30.0)
+    h[0, :6] = torch.tensor([0.0, -0.0, 88.5, -88.5, -200.0, 200.0], dtype=torch.bfloat16)
+    hg = h.to(gpu)
+    q, si, qt, sit = hpfp8.ops.swiglu_quantize_1x128_and_128x1_t(hg, fast=fast)
+    q1, si1, act = hpfp8.swiglu_quantize_1x128(hg, kmajor=True, want_act=True, fast=fast)
+    qt1, sit1 = hpfp8.quantize_128x1_t(act, kmajor=True)
+    assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(si, si1)
+    assert torch.equal(qt.view(torch.uint8), qt1.view(torch.uint8)) and torch.equal(sit, sit1)
+    assert si.stride(0) == 1 and sit.stride(0) == 1
+    if not fast:
+        rq, _, rsi, ract = O.swiglu_quantize_1x128(U.bits(h))
+        rqt, _, rsit = O.quantize_128x1_t(ract)
+        assert np.array_equal(U.codes(q), rq) and eq_f32(si, rsi) and np.array_equal(U.codes(qt), rqt) and eq_f32(sit, rsit)
+    wide = torch.zeros((256, 1536 + 64), dtype=torch.bfloat16, device=gpu)
+    wide[:, :1536] = hg
+    q2, si2, qt2, sit2 = hpfp8.ops.swiglu_quantize_1x128_and_128x1_t(wide[:, :1536], fast=fast)
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(qt2.view(torch.uint8), qt.view(torch.uint8))
+    assert torch.equal(si2, si) and torch.equal(sit2, sit)
+    with pytest.raises(ValueError):
+        hpfp8.ops.swiglu_quantize_1x128_and_128x1_t(hg[:100], fast=fast)
+
+
 def test_dequantize_accumulate_into_fp32_main_grad(gpu):
     import hpfp8
     g = U.randn_bf16((300, 640), 71, 1e-3, 0.002, 100.0)
