@@ -364,3 +364,42 @@ def test_swiglu_mlp_training_step_vs_torch(gpu):
     y2 = hpfp8.fp8_swiglu_mlp(x2, wgu.detach(), wd.detach())
     y2.backward(go)
     assert torch.equal(y2, y) and rel(x2.grad, gx) < 1e-6
+
+
+def test_mlp_training_step_replays_from_a_captured_graph(gpu):
+    """Forward and backward of the MLP block captured into one graph (weights prequantized outside it): every
+    replay, with eager work and synchronisations in between, gives the eager step's output and gradients for
+    the input of the moment."""
+    import hpfp8
+    g = torch.Generator(device="cpu").manual_seed(6)
+    m, k, inter, n = 256, 512, 640, 384
+    wgu = (torch.randn((2 * inter, k), generator=g) * 0.05).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    wd = (torch.randn((n, inter), generator=g) * 0.05).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    gu8, d8 = hpfp8.quantize_weight(wgu.detach()), hpfp8.quantize_weight(wd.detach())
+    xs = [torch.randn((m, k), generator=g).mul(1.0 + i).to(torch.bfloat16).to(gpu) for i in range(4)]
+    go = (torch.randn((m, n), generator=g) * 1e-2).to(torch.bfloat16).to(gpu)
+    x_static = xs[0].clone().requires_grad_(True)
+
+    def step(x):
+        y = hpfp8.fp8_swiglu_mlp(x, wgu, wd, gate_up_fp8=gu8, down_fp8=d8)
+        gx, ggu, gd = torch.autograd.grad(y, (x, wgu, wd), go)
+        return y, gx, ggu, gd
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(x_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step(x_static)
+    for x in xs[1:] + xs[:2]:
+        with torch.no_grad():
+            x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = step(x.clone().requires_grad_(True))
+        for a, b in zip(outs, want):
+            assert torch.equal(a, b)
