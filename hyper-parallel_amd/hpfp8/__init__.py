@@ -10,7 +10,8 @@ from .ops import (amax, quantize_per_tensor, quantize_1x128, quantize_128x128, q
                   quantize_1x128_and_128x1_t, transpose_codes, swiglu_quantize_1x128,
                   dequantize_1x128, dequantize_1x128_accumulate, dequantize_128x128, gemm_blockwise, gemm_per_tensor,
                   gemm_grouped_blockwise)
-from .linear import fp8_linear, Fp8Linear, fp8_grouped_linear, fp8_swiglu_mlp, Fp8Weight, quantize_weight  # noqa: E402
+from .linear import (fp8_linear, Fp8Linear, fp8_grouped_linear, fp8_swiglu_mlp, Fp8SwiGLUMLP, Fp8Weight,  # noqa: E402
+                     quantize_weight)
 from . import fsdp, checkpoint  # noqa: E402
 from .bucket import quantize_bucket, dequantize_bucket, Fp8GradBucket  # noqa: E402
 from .policy import Fp8MixedPrecisionPolicy, Fp8Tensor, cast_fp_tensor  # noqa: E402
@@ -20,6 +21,6 @@ __all__ = [
     "amax", "quantize_per_tensor", "quantize_1x128", "quantize_128x128", "quantize_128x1_t",
     "quantize_1x128_and_128x1_t", "transpose_codes", "swiglu_quantize_1x128", "Fp8Weight", "quantize_weight", "fsdp", "checkpoint",
     "dequantize_1x128", "dequantize_1x128_accumulate", "dequantize_128x128", "gemm_blockwise", "gemm_per_tensor",
-    "gemm_grouped_blockwise", "fp8_linear", "Fp8Linear", "fp8_grouped_linear", "fp8_swiglu_mlp",
+    "gemm_grouped_blockwise", "fp8_linear", "Fp8Linear", "fp8_grouped_linear", "fp8_swiglu_mlp", "Fp8SwiGLUMLP",
     "quantize_bucket", "dequantize_bucket", "Fp8GradBucket",
 ]

@@ -386,3 +386,36 @@ def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True,
         aq, sa = ops.swiglu_quantize_1x128(h, kmajor=True, pow2=dn.pow2, fast=fast)
         y = ops.gemm_blockwise(aq, sa, dn.codes, dn.scale_inv, pow2_scales=dn.pow2)
     return y.reshape(input.shape[:-1] + (dn.codes.shape[0],))
+
+
+class Fp8SwiGLUMLP(nn.Module):
+    """A SwiGLU MLP block with bf16 parameters ``gate_up_proj.weight`` [2 * intermediate, hidden] (gate rows
+    first) and ``down_proj.weight`` [hidden, intermediate], computed by `fp8_swiglu_mlp`.  Like `Fp8Linear` it
+    keeps the FP8 forms of its weights until a parameter is written again, so the micro-batches of one optimizer
+    step and inference calls quantize them once."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, *, fast: bool = True, device=None, dtype=torch.bfloat16):
+        super().__init__()
+        if hidden_size % ops.BLOCK or intermediate_size % ops.BLOCK:
+            raise ValueError("hidden_size and intermediate_size must be multiples of 128")
+        self.hidden_size, self.intermediate_size, self.fast = hidden_size, intermediate_size, fast
+        self.gate_up_proj = nn.Linear(hidden_size, 2 * intermediate_size, bias=False, device=device, dtype=dtype)
+        self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False, device=device, dtype=dtype)
+        self._fp8 = [None, None]
+        self._fp8_key = [None, None]
+
+    def _weight_fp8(self, i: int, w: torch.Tensor) -> Fp8Weight:
+        key = (w._version, w.data_ptr())
+        if self._fp8_key[i] != key:
+            with torch.no_grad():
+                self._fp8[i] = quantize_weight(w.detach(), with_transpose=True)
+            self._fp8_key[i] = key
+        return self._fp8[i]
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        wgu, wd = self.gate_up_proj.weight, self.down_proj.weight
+        return fp8_swiglu_mlp(input, wgu, wd, fast=self.fast, gate_up_fp8=self._weight_fp8(0, wgu),
+                              down_fp8=self._weight_fp8(1, wd))
+
+    def extra_repr(self) -> str:
+        return f"hidden_size={self.hidden_size}, intermediate_size={self.intermediate_size}, fast={self.fast}"

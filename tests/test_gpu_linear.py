@@ -403,3 +403,30 @@ def test_mlp_training_step_replays_from_a_captured_graph(gpu):
         want = step(x.clone().requires_grad_(True))
         for a, b in zip(outs, want):
             assert torch.equal(a, b)
+
+
+def test_swiglu_mlp_module_caches_weights_and_trains(gpu):
+    """The module equals the functional form on its own parameters, quantizes each weight once until the
+    parameter is written, and an SGD step through it lowers a least-squares loss."""
+    import hpfp8
+    torch.manual_seed(0)
+    mlp = hpfp8.Fp8SwiGLUMLP(256, 384, device=gpu)
+    x = torch.randn((128, 256), device=gpu).to(torch.bfloat16)
+    y = mlp(x)
+    want = hpfp8.fp8_swiglu_mlp(x, mlp.gate_up_proj.weight, mlp.down_proj.weight)
+    assert torch.equal(y, want) and y.requires_grad
+    first = mlp._fp8[0]
+    mlp(x)
+    assert mlp._fp8[0] is first                       # same parameter version: no second quantization
+    target = torch.randn((128, 256), device=gpu).to(torch.bfloat16)
+    opt = torch.optim.SGD(mlp.parameters(), lr=0.05)
+    losses = []
+    for _ in range(5):
+        opt.zero_grad()
+        loss = (mlp(x).float() - target.float()).pow(2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert mlp._fp8[0] is not first                   # the optimizer wrote the parameter
+    assert losses[-1] < losses[0]
+    assert set(mlp.state_dict()) == {"gate_up_proj.weight", "down_proj.weight"}
