@@ -430,3 +430,51 @@ def test_swiglu_mlp_module_caches_weights_and_trains(gpu):
     assert mlp._fp8[0] is not first                   # the optimizer wrote the parameter
     assert losses[-1] < losses[0]
     assert set(mlp.state_dict()) == {"gate_up_proj.weight", "down_proj.weight"}
+
+
+def test_two_threads_on_two_streams(gpu):
+    """Calls from two host threads, each on a stream of its own, run concurrently and give the bits of the same
+    calls made one after the other on the default stream (no shared state inside the library besides the
+    per-thread error text)."""
+    import threading
+    import hpfp8
+    xs = [U.randn_bf16((512, 1024), 90 + i).to(gpu) for i in range(2)]
+    ws = [U.randn_bf16((768, 1024), 95 + i, 0.02).to(gpu) for i in range(2)]
+
+    def work(x, w):
+        xq, sx = hpfp8.quantize_1x128(x, kmajor=True)
+        wq, sw = hpfp8.quantize_128x128(w)
+        y = hpfp8.gemm_blockwise(xq, sx, wq, sw)
+        h = hpfp8.gemm_blockwise(xq, sx, wq, sw, out_dtype=torch.float32)
+        aq, sa = hpfp8.swiglu_quantize_1x128(y, kmajor=True, fast=True)
+        return y, h, aq.view(torch.uint8), sa
+
+    want = [work(x, w) for x, w in zip(xs, ws)]
+    torch.cuda.synchronize()
+    got = [None, None]
+    errors = []
+
+    def run(i):
+        try:
+            stream = torch.cuda.Stream()
+            stream.wait_stream(torch.cuda.default_stream())
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    got[i] = work(xs[i], ws[i])
+                try:
+                    hpfp8.quantize_1x128(xs[i][:, :100])          # an error in this thread only
+                except ValueError:
+                    pass
+            stream.synchronize()
+        except Exception as e:                                    # pragma: no cover
+            errors.append(e)
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for g_, w_ in zip(got, want):
+        for a, b in zip(g_, w_):
+            assert torch.equal(a, b)
