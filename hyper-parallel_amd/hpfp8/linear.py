@@ -52,6 +52,22 @@ def _flatten(x: torch.Tensor):
     return x.reshape(-1, x.shape[-1])
 
 
+def _empty_batch_grads(ctx, go):
+    """(dx, dw, db) of a linear whose batch is empty: no token contributes, so the weight and bias gradients are
+    zero (an fp32 main gradient is left as it is, or created as zeros)."""
+    need_dx, need_dw = ctx.need
+    dx = go.new_zeros(ctx.x_shape) if need_dx else None
+    dw = None
+    if need_dw:
+        param = getattr(ctx, "main_grad_of", None)
+        if param is None:
+            dw = go.new_zeros(ctx.w_shape)
+        elif getattr(param, "main_grad", None) is None:
+            param.main_grad = torch.zeros(ctx.w_shape, dtype=torch.float32, device=go.device)
+    db = go.new_zeros(ctx.w_shape[0]) if ctx.has_bias else None
+    return dx, dw, db
+
+
 class _Fp8LinearBlockwise(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, wq=None, sw=None, wqt=None, on_main_grad=False, pow2=False):
@@ -79,6 +95,7 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
         ctx.save_for_backward(x2 if (weight.requires_grad and not fused) else None, xt, sxt,
                               wqt if x.requires_grad else None, sw)
         ctx.x_shape = x.shape
+        ctx.w_shape = weight.shape
         ctx.has_bias = bias is not None
         ctx.need = (x.requires_grad, weight.requires_grad)
         return y.reshape(x.shape[:-1] + (weight.shape[0],))
@@ -93,6 +110,8 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
             go = go.to(torch.bfloat16)
         go = go.contiguous()
         m = go.shape[0]
+        if m == 0:
+            return _empty_batch_grads(ctx, go) + (None, None, None, None, None)
         if need_dw and m % ops.BLOCK:
             raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
         dx = dw = db = None
@@ -145,6 +164,7 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
         else:
             ctx.save_for_backward(x2, weight)
         ctx.x_shape = x.shape
+        ctx.w_shape = weight.shape
         ctx.has_bias = bias is not None
         ctx.need = (x.requires_grad, weight.requires_grad)
         return y.reshape(x.shape[:-1] + (weight.shape[0],))
@@ -156,6 +176,8 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
         if go.dtype != torch.bfloat16:
             go = go.to(torch.bfloat16)
         go = go.contiguous()
+        if go.shape[0] == 0:
+            return _empty_batch_grads(ctx, go)
         dx = dw = db = None
         if ctx.codes_saved:
             xq, sx, wq, sw = ctx.saved_tensors
@@ -313,6 +335,7 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
         ctx.save_for_backward(h2 if h.requires_grad or (weight.requires_grad and not fused) else None, wqt, sw, at, sat)
         ctx.fast = fast
         ctx.h_shape = h.shape
+        ctx.x_shape, ctx.w_shape, ctx.has_bias = h.shape, weight.shape, False
         ctx.need = (h.requires_grad, weight.requires_grad)
         return y.reshape(h.shape[:-1] + (weight.shape[0],))
 
@@ -325,6 +348,8 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
             go = go.to(torch.bfloat16)
         go = go.contiguous()
         m = go.shape[0]
+        if m == 0:
+            return _empty_batch_grads(ctx, go)[:2] + (None, None, None, None)
         if need_dw and m % ops.BLOCK:
             raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
         dh = dw = None

@@ -478,3 +478,28 @@ def test_two_threads_on_two_streams(gpu):
     for g_, w_ in zip(got, want):
         for a, b in zip(g_, w_):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("recipe", ["blockwise", "per_tensor", "blockwise_pow2"])
+def test_empty_batch_and_one_dimensional_input(gpu, recipe):
+    """F.linear's behaviour at the edges of the batch: no rows gives no rows, with zero weight and bias gradients;
+    a 1-D input gives a 1-D output."""
+    import hpfp8
+    w = U.randn_bf16((384, 512), 2, 0.02).to(gpu).requires_grad_(True)
+    b = U.randn_bf16((384,), 3, 0.1).to(gpu).requires_grad_(True)
+    x = torch.empty((0, 512), dtype=torch.bfloat16, device=gpu, requires_grad=True)
+    y = hpfp8.fp8_linear(x, w, b, recipe=recipe)
+    assert y.shape == (0, 384)
+    y.backward(torch.empty_like(y))
+    assert x.grad.shape == (0, 512) and not bool(w.grad.any()) and not bool(b.grad.any()) and w.grad.shape == w.shape
+    v = U.randn_bf16((512,), 5).to(gpu)
+    y1 = hpfp8.fp8_linear(v, w.detach(), b.detach(), recipe=recipe)
+    assert y1.shape == (384,) and torch.equal(y1, hpfp8.fp8_linear(v[None], w.detach(), b.detach(), recipe=recipe)[0])
+    if recipe == "blockwise":
+        x3 = torch.empty((2, 0, 512), dtype=torch.bfloat16, device=gpu, requires_grad=True)
+        wgu = U.randn_bf16((512, 512), 6, 0.02).to(gpu).requires_grad_(True)
+        wd = U.randn_bf16((384, 256), 7, 0.02).to(gpu).requires_grad_(True)
+        y3 = hpfp8.fp8_swiglu_mlp(x3, wgu, wd)
+        assert y3.shape == (2, 0, 384)
+        y3.backward(torch.empty_like(y3))
+        assert x3.grad.shape == x3.shape and not bool(wgu.grad.any()) and not bool(wd.grad.any())
