@@ -52,6 +52,13 @@ def _flatten(x: torch.Tensor):
     return x.reshape(-1, x.shape[-1])
 
 
+def _pad_rows(t: torch.Tensor) -> torch.Tensor:
+    """t[M, C] with zero rows appended up to the next multiple of 128: tokens that contribute nothing to a
+    weight gradient, so that the 128x1 groups along the tokens are whole (the last one holds fewer real values)."""
+    pad = -t.shape[0] % ops.BLOCK
+    return torch.nn.functional.pad(t, (0, 0, 0, pad)) if pad else t
+
+
 def _empty_batch_grads(ctx, go):
     """(dx, dw, db) of a linear whose batch is empty: no token contributes, so the weight and bias gradients are
     zero (an fp32 main gradient is left as it is, or created as zeros)."""
@@ -112,16 +119,16 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
         m = go.shape[0]
         if m == 0:
             return _empty_batch_grads(ctx, go) + (None, None, None, None, None)
-        if need_dw and m % ops.BLOCK:
-            raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
+        ragged = m % ops.BLOCK != 0            # wgrad then runs on zero-padded token rows
         dx = dw = db = None
         goq = sgo = got = sgot = None
-        if need_dx and need_dw:
+        if need_dx and need_dw and not ragged:
             goq, sgo, got, sgot = ops.quantize_1x128_and_128x1_t(go, kmajor=True, pow2=pow2)   # one read of grad_out
-        elif need_dx:
-            goq, sgo = ops.quantize_1x128(go, kmajor=True, pow2=pow2)
-        elif need_dw:
-            got, sgot = ops.quantize_128x1_t(go, kmajor=True, pow2=pow2)
+        else:
+            if need_dx:
+                goq, sgo = ops.quantize_1x128(go, kmajor=True, pow2=pow2)
+            if need_dw:
+                got, sgot = ops.quantize_128x1_t(_pad_rows(go), kmajor=True, pow2=pow2)
         if need_dx:
             # dx[M,K] = go[M,N] . W[N,K]: contraction over N, b operand = W^T codes [K,N] whose
             # 128x128 scales are W's with the two strides swapped.
@@ -129,7 +136,7 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
         if need_dw:
             # dW[N,K] = go^T[N,M] . x[M,K]: contraction over tokens, both operands 1x128 along M
             if xt is None:
-                xt, sxt = ops.quantize_128x1_t(x2, kmajor=True, pow2=pow2)
+                xt, sxt = ops.quantize_128x1_t(_pad_rows(x2), kmajor=True, pow2=pow2)
             param = ctx.main_grad_of
             if param is None:
                 dw = ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, pow2_scales=pow2)
@@ -193,8 +200,8 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
                 wtq, _, swt = ops.quantize_per_tensor(weight.t().contiguous())
                 dx = ops.gemm_per_tensor(goq, sgo, wtq, swt).reshape(ctx.x_shape)
             if need_dw:
-                gotq, _, sgot = ops.quantize_per_tensor(go.t().contiguous())
-                xtq, _, sxt = ops.quantize_per_tensor(x2.t().contiguous())
+                gotq, _, sgot = ops.quantize_per_tensor(_pad_rows(go).t().contiguous())
+                xtq, _, sxt = ops.quantize_per_tensor(_pad_rows(x2).t().contiguous())
                 dw = ops.gemm_per_tensor(gotq, sgot, xtq, sxt)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
@@ -208,7 +215,8 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
 
     input [..., in_features] bf16, weight [out_features, in_features] bf16, bias [out_features] bf16
     or None; returns bf16 [..., out_features].  in_features and out_features must be multiples of
-    128 (ragged tails are rejected, not padded).
+    128 (ragged tails are rejected, not padded); the token count may be anything (for the weight gradient,
+    whose scaling groups run along the tokens, a ragged count is filled up with zero rows).
 
     `weight_fp8` (blockwise recipe) is the weight's FP8 form made earlier -- by `quantize_weight`, or
     from all-gathered FP8 shards (`hpfp8.fsdp`) -- and saves its quantization in this call; `weight`
@@ -350,21 +358,21 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
         m = go.shape[0]
         if m == 0:
             return _empty_batch_grads(ctx, go)[:2] + (None, None, None, None)
-        if need_dw and m % ops.BLOCK:
-            raise ValueError(f"wgrad needs the token count ({m}) to be a multiple of 128")
+        ragged = m % ops.BLOCK != 0            # wgrad then runs on zero-padded token rows
         dh = dw = None
         goq = sgo = got = sgot = None
-        if need_dh and need_dw:
+        if need_dh and need_dw and not ragged:
             goq, sgo, got, sgot = ops.quantize_1x128_and_128x1_t(go, kmajor=True)
-        elif need_dh:
-            goq, sgo = ops.quantize_1x128(go, kmajor=True)
-        elif need_dw:
-            got, sgot = ops.quantize_128x1_t(go, kmajor=True)
+        else:
+            if need_dh:
+                goq, sgo = ops.quantize_1x128(go, kmajor=True)
+            if need_dw:
+                got, sgot = ops.quantize_128x1_t(_pad_rows(go), kmajor=True)
         if need_dw:
             if at is None:
                 # the activation again (bf16 this time), for its 128x1 codes along the tokens
                 _, _, act = ops.swiglu_quantize_1x128(h2, kmajor=True, want_act=True, fast=ctx.fast)
-                at, sat = ops.quantize_128x1_t(act, kmajor=True)
+                at, sat = ops.quantize_128x1_t(_pad_rows(act), kmajor=True)
                 del act
             dw = ops.gemm_blockwise(got, sgot, at, sat, sb_gran=1)
         if need_dh:

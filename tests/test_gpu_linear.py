@@ -503,3 +503,39 @@ def test_empty_batch_and_one_dimensional_input(gpu, recipe):
         assert y3.shape == (2, 0, 384)
         y3.backward(torch.empty_like(y3))
         assert x3.grad.shape == x3.shape and not bool(wgu.grad.any()) and not bool(wd.grad.any())
+
+
+@pytest.mark.parametrize("recipe", ["blockwise", "per_tensor", "blockwise_pow2"])
+def test_token_count_that_is_not_a_multiple_of_128(gpu, recipe):
+    """Any batch size trains: the weight gradient's groups along the tokens are filled up with zero rows, which
+    is exactly the gradient of the batch with those rows appended (bit for bit), and stays within FP8 noise of
+    F.linear's."""
+    import hpfp8
+    x = U.randn_bf16((3, 100, 512), 1).to(gpu).requires_grad_(True)          # 300 tokens
+    w = U.randn_bf16((384, 512), 2, 0.02).to(gpu).requires_grad_(True)
+    b = U.randn_bf16((384,), 3, 0.1).to(gpu).requires_grad_(True)
+    go = U.randn_bf16((3, 100, 384), 4, 1e-3).to(gpu)
+    y = hpfp8.fp8_linear(x, w, b, recipe=recipe)
+    y.backward(go)
+    gx, gw, gb = x.grad.clone(), w.grad.clone(), b.grad.clone()
+    x.grad = w.grad = b.grad = None
+    yr = F.linear(x.float(), w.float(), b.float())
+    yr.backward(go.float())
+    tol = 0.06 if recipe == "blockwise" else 0.08
+    assert rel(y, yr) < tol and rel(gx, x.grad) < tol and rel(gw, w.grad) < tol and rel(gb, b.grad) < 1e-2
+    w.grad = None
+    xp = torch.cat([x.detach().reshape(300, 512), torch.zeros((84, 512), dtype=torch.bfloat16, device=gpu)]).requires_grad_(True)
+    gop = torch.cat([go.reshape(300, 384), torch.zeros((84, 384), dtype=torch.bfloat16, device=gpu)])
+    hpfp8.fp8_linear(xp, w, b, recipe=recipe).backward(gop)
+    if recipe != "per_tensor":                                               # (per tensor: the bias row changes no amax either)
+        assert torch.equal(w.grad, gw)
+    assert rel(w.grad, gw) < 1e-6
+    if recipe == "blockwise":
+        wgu = U.randn_bf16((512, 512), 6, 0.05).to(gpu).requires_grad_(True)
+        wd = U.randn_bf16((384, 256), 7, 0.05).to(gpu).requires_grad_(True)
+        x2 = x.detach().clone().requires_grad_(True)
+        hpfp8.fp8_swiglu_mlp(x2, wgu, wd).backward(go)
+        hr = F.linear(x2.detach().float(), wgu.float())
+        yr = F.linear(F.silu(hr[..., :256]) * hr[..., 256:], wd.float())
+        gr = torch.autograd.grad(yr, (wgu, wd), go.float())
+        assert rel(wgu.grad, gr[0]) < 0.1 and rel(wd.grad, gr[1]) < 0.08 and x2.grad.shape == x2.shape
