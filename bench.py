@@ -288,7 +288,20 @@ def other_configs(dev):
     ms2 = _time(lambda: hpfp8.gemm_grouped_blockwise(xq, sx2, wq.view(e, n, k), sw2.view(e, n // 128, k // 128), offs,
                                                      pow2_scales=True), iters=5)
     res.setdefault("recipe_blockwise_pow2", {})["cfg4_moe_grouped_gemm"] = tf(2.0 * total * n * k, ms2)
-    del xq, sx, wq, sw
+    del xq, sx, wq, sw, sx2, sw2
+    torch.cuda.empty_cache()
+    # the same layer in training: forward + backward of the grouped linear (weights quantized inside the step)
+    xg4 = torch.randn((total, k), generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+    wg4 = (torch.randn((e, n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16).requires_grad_(True)
+    go4 = (torch.randn((total, n), generator=g, device=dev) * 1e-3).to(torch.bfloat16)
+
+    def grouped_train():
+        hpfp8.fp8_grouped_linear(xg4, wg4, offs).backward(go4)
+        xg4.grad = wg4.grad = None
+    ms3 = _time(grouped_train, iters=3, warm=3)
+    res["cfg4_moe_grouped_forward_backward"] = dict(tf(3 * 2.0 * total * n * k, ms3),
+                                                    note="grouped forward and dgrad, per-expert wgrad GEMMs, quantizers")
+    del xg4, wg4, go4
     torch.cuda.empty_cache()
     # cfg 5: gradient bucket, 2^29 elements
     nel = 1 << 29

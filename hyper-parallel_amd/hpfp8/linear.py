@@ -304,15 +304,65 @@ class Fp8Linear(nn.Module):
                 f"bias={self.bias is not None}, recipe={self.recipe}")
 
 
+class _Fp8GroupedLinear(torch.autograd.Function):
+    """Grouped (MoE) linear with the blockwise recipe.  Forward and the input gradient are one grouped GEMM each
+    (the latter on the experts' transposed codes); the weight gradient of expert e contracts over that expert's own
+    token range, one dense wgrad GEMM per expert on its rows filled up with zero rows to a multiple of 128."""
+
+    @staticmethod
+    def forward(ctx, x, weight, offs):
+        e, n, k = weight.shape
+        xq, sx = ops.quantize_1x128(x, kmajor=True)
+        wq, sw = ops.quantize_128x128(weight.reshape(e * n, k))
+        y = ops.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), offs)
+        ctx.save_for_backward(x if weight.requires_grad else None, wq if x.requires_grad else None, sw, offs)
+        ctx.w_shape = weight.shape
+        ctx.need = (x.requires_grad, weight.requires_grad)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, wq, sw, offs = ctx.saved_tensors
+        need_dx, need_dw = ctx.need
+        e, n, k = ctx.w_shape
+        go = grad_out.to(torch.bfloat16).contiguous()
+        ends = [min(max(int(v), 0), go.shape[0]) for v in offs.tolist()]       # (one host read of the row counts)
+        last = ends[-1] if ends else 0
+        dx = dw = None
+        if need_dx:
+            # dx_e = go_e . W_e: the grouped kernel again, b = W_e^T codes [K, N] (128x128 blocks are symmetric,
+            # so W's scales serve with their two block dims swapped)
+            wt = torch.empty((e, k, n), dtype=wq.dtype, device=wq.device)
+            wq3 = wq.view(e, n, k)
+            for i in range(e):
+                wt[i] = ops.transpose_codes(wq3[i])
+            swt = sw.view(e, n // ops.BLOCK, k // ops.BLOCK).transpose(1, 2).contiguous()
+            goq, sgo = ops.quantize_1x128(go, kmajor=True)
+            dx = ops.gemm_grouped_blockwise(goq, sgo, wt, swt, offs)
+            if last < dx.shape[0]:
+                dx[last:] = 0                                                    # rows that belong to no expert
+        if need_dw:
+            dw = torch.zeros(ctx.w_shape, dtype=torch.bfloat16, device=go.device)
+            start = 0
+            for i, end in enumerate(ends):
+                if end > start:
+                    got, sgot = ops.quantize_128x1_t(_pad_rows(go[start:end]), kmajor=True)
+                    xt, sxt = ops.quantize_128x1_t(_pad_rows(x[start:end]), kmajor=True)
+                    ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=dw[i])
+                start = max(start, end)
+        return dx, dw, None
+
+
 def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
-    """MoE grouped linear, forward only: rows of input[total_m, K] are sorted by expert, offs[E] are
-    the inclusive int32 prefix sums of rows per expert, weight[E, N, K] -> bf16 [total_m, N]."""
+    """MoE grouped linear: rows of input[total_m, K] are sorted by expert, offs[E] are the inclusive int32
+    prefix sums of rows per expert (a count may be 0), weight[E, N, K] -> bf16 [total_m, N]; rows past offs[-1]
+    are left uninitialised, as torch's grouped matmul leaves them.  Differentiable in input and weight
+    (blockwise recipe); backward reads offs on the host once."""
     if input.dim() != 2 or weight.dim() != 3 or input.shape[1] != weight.shape[2]:
         raise ValueError("input must be [total_m, K] and weight [E, N, K]")
-    xq, sx = ops.quantize_1x128(input, kmajor=True)
-    e, n, k = weight.shape
-    wq, sw = ops.quantize_128x128(weight.reshape(e * n, k))
-    return ops.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), offs)
+    if input.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("input and weight must be bfloat16")
+    return _Fp8GroupedLinear.apply(input, weight, offs)
 
 
 class _Fp8SwiGLUDown(torch.autograd.Function):

@@ -539,3 +539,35 @@ def test_token_count_that_is_not_a_multiple_of_128(gpu, recipe):
         yr = F.linear(F.silu(hr[..., :256]) * hr[..., 256:], wd.float())
         gr = torch.autograd.grad(yr, (wgu, wd), go.float())
         assert rel(wgu.grad, gr[0]) < 0.1 and rel(wd.grad, gr[1]) < 0.08 and x2.grad.shape == x2.shape
+
+
+def test_grouped_linear_backward(gpu):
+    """Input and weight gradients of the grouped linear against a loop of F.linear over the experts (fp32
+    autograd), experts with no rows and rows that belong to no expert included."""
+    import hpfp8
+    counts = torch.tensor([130, 0, 300, 70])                    # 500 of 512 rows are routed
+    offs = counts.cumsum(0).to(torch.int32).to(gpu)
+    x = U.randn_bf16((512, 256), 31).to(gpu).requires_grad_(True)
+    w = U.randn_bf16((4, 384, 256), 32, 0.05).to(gpu).requires_grad_(True)
+    go = U.randn_bf16((512, 384), 33, 1e-2).to(gpu)
+    y = hpfp8.fp8_grouped_linear(x, w, offs)
+    y.backward(go)
+    gx, gw = x.grad.clone(), w.grad.clone()
+    x.grad = w.grad = None
+    start = 0
+    for e in range(4):
+        c = int(counts[e])
+        if c:
+            F.linear(x[start:start + c].float(), w[e].float()).backward(go[start:start + c].float())
+        start += c
+    assert rel(gx[:500], x.grad[:500]) < 0.06 and not bool(gx[500:].any())
+    assert rel(gw, w.grad) < 0.08 and not bool(gw[1].any())
+    for e in (0, 2, 3):
+        assert rel(gw[e], w.grad[e]) < 0.08
+    # only one of the two gradients
+    x1 = x.detach().clone().requires_grad_(True)
+    hpfp8.fp8_grouped_linear(x1, w.detach(), offs).backward(go)
+    assert torch.equal(x1.grad, gx)
+    w1 = w.detach().clone().requires_grad_(True)
+    hpfp8.fp8_grouped_linear(x.detach(), w1, offs).backward(go)
+    assert torch.equal(w1.grad, gw)
