@@ -29,8 +29,8 @@ PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 # Bytes per GEMM launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 1.9992 calibration + WRITE_SIZE, profiles/bench_cfg2_gemm_blockwise_and_quantizers.md):
-# 1,583,390 KiB fetched + 294,998 KiB written.  Algorithmic operand + output bytes are 582,591 KiB.
-GEMM_TRAFFIC_BYTES = (1583390 + 294998) * 1024   # FETCH_SIZE x 1.9992 + WRITE_SIZE of the GEMM, KiB per dispatch
+# 1,582,999 KiB fetched + 294,946 KiB written.  Algorithmic operand + output bytes are 582,591 KiB.
+GEMM_TRAFFIC_BYTES = (1582999 + 294946) * 1024   # FETCH_SIZE x 1.9992 + WRITE_SIZE of the GEMM, KiB per dispatch
 
 
 def make_inputs(dev):
