@@ -346,8 +346,8 @@ class _Fp8GroupedLinear(torch.autograd.Function):
             start = 0
             for i, end in enumerate(ends):
                 if end > start:
-                    got, sgot = ops.quantize_128x1_t(_pad_rows(go[start:end]), kmajor=True)
-                    xt, sxt = ops.quantize_128x1_t(_pad_rows(x[start:end]), kmajor=True)
+                    got, sgot = ops.quantize_128x1_t_rows(go[start:end])
+                    xt, sxt = ops.quantize_128x1_t_rows(x[start:end])
                     ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=dw[i])
                 start = max(start, end)
         return dx, dw, None

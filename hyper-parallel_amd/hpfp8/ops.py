@@ -287,6 +287,29 @@ def quantize_128x1_t(x: torch.Tensor, want_scale: bool = False, kmajor: bool = F
     return (qt, scale, scale_inv) if want_scale else (qt, scale_inv)
 
 
+def quantize_128x1_t_rows(x: torch.Tensor):
+    """`quantize_128x1_t(..., kmajor=True)` of x[M, K] for any M > 0: the last group of a ragged M is filled up with
+    zero rows.  Only those last rows are copied for the padding; the whole groups are quantized where they lie.
+    Returns (codes_t[K, Mp], scale_inv_t[K, Mp/128]) with Mp = M rounded up to a multiple of 128."""
+    x = _check_bf16(x, "x")
+    if x.dim() != 2 or x.shape[1] % BLOCK or x.shape[0] == 0:
+        raise ValueError("x must be [M, K] with M > 0 and K a multiple of 128")
+    m, k = x.shape
+    main = m // BLOCK * BLOCK
+    mp = main + (BLOCK if m > main else 0)
+    qt = _empty_codes_t(k, mp, x.device)
+    scale_inv = torch.empty((mp // BLOCK, k), dtype=torch.float32, device=x.device)
+    if main:
+        _lib.call("hpfp8_quantize_128x1_t_kmajor_bf16", _ptr(x), main, k, _ptr(qt), qt.stride(0), None, _ptr(scale_inv),
+                  _stream())
+    if m > main:
+        tail = torch.zeros((BLOCK, k), dtype=torch.bfloat16, device=x.device)
+        tail[:m - main] = x[main:]
+        _lib.call("hpfp8_quantize_128x1_t_kmajor_bf16", _ptr(tail), BLOCK, k, qt.data_ptr() + main, qt.stride(0), None,
+                  scale_inv.data_ptr() + main // BLOCK * k * 4, _stream())
+    return qt, scale_inv.t()
+
+
 def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True, pow2: bool = False):
     """Both operand forms of x[M, K] from one read of it.
 

@@ -456,6 +456,23 @@ def test_swiglu_with_both_quantized_forms(gpu, fast):
         hpfp8.ops.swiglu_quantize_1x128_and_128x1_t(hg[:100], fast=fast)
 
 
+@pytest.mark.parametrize("rows", [1, 100, 128, 300, 384])
+def test_transposed_quantizer_on_a_ragged_row_count(gpu, rows):
+    """Whole groups quantized in place and the last, ragged, group from a zero-filled copy: the bits of the
+    transposing quantizer on the zero-padded tensor."""
+    import hpfp8
+    x = U.randn_bf16((rows, 384), 41, 1.0, 0.01, 30.0).to(gpu)
+    big = torch.zeros((640, 384), dtype=torch.bfloat16, device=gpu)
+    big[7:7 + rows] = x                                      # (a row slice that starts at an odd row of its buffer)
+    qt, sit = hpfp8.ops.quantize_128x1_t_rows(big[7:7 + rows])
+    mp = -(-rows // 128) * 128
+    xp = torch.zeros((mp, 384), dtype=torch.bfloat16, device=gpu)
+    xp[:rows] = x
+    wqt, wsit = hpfp8.quantize_128x1_t(xp, kmajor=True)
+    assert qt.shape == (384, mp) and torch.equal(qt.view(torch.uint8), wqt.view(torch.uint8)) and torch.equal(sit, wsit)
+    assert sit.stride(0) == 1
+
+
 def test_dequantize_accumulate_into_fp32_main_grad(gpu):
     import hpfp8
     g = U.randn_bf16((300, 640), 71, 1e-3, 0.002, 100.0)
