@@ -342,13 +342,15 @@ class _Fp8GroupedLinear(torch.autograd.Function):
             if last < dx.shape[0]:
                 dx[last:] = 0                                                    # rows that belong to no expert
         if need_dw:
-            dw = torch.zeros(ctx.w_shape, dtype=torch.bfloat16, device=go.device)
+            dw = torch.empty(ctx.w_shape, dtype=torch.bfloat16, device=go.device)
             start = 0
             for i, end in enumerate(ends):
                 if end > start:
                     got, sgot = ops.quantize_128x1_t_rows(go[start:end])
                     xt, sxt = ops.quantize_128x1_t_rows(x[start:end])
                     ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=dw[i])
+                else:
+                    dw[i].zero_()                                                # an expert without rows
                 start = max(start, end)
         return dx, dw, None
 
