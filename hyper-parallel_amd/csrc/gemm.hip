@@ -17,6 +17,10 @@
 //   * The grid is persistent: one workgroup per CU walks a list of tiles, and the rounds of
 //     consecutive tiles follow each other without a gap.  Each XCD (own L2) owns a contiguous run
 //     of tile numbers.
+//   * Results leave through the wave's own slice of a consumed LDS buffer, regrouped into whole rows of
+//     256 bytes, as streaming stores through a buffer resource that ends with the tile's last valid row
+//     (rows past the end of a ragged tile or of an expert are dropped by its range check); with
+//     accumulate, c's old values are the accumulators' starting values, loaded before the tile's first round.
 //   * One kernel template, by scale form: per tensor, 128x128 blocks of b (forward, dgrad), per-row
 //     scales on both operands (wgrad), and the two blockwise forms again for scales that are powers of
 //     two, which the matrix instruction applies itself (no promotion FMAs); dense or grouped by expert;
