@@ -385,6 +385,8 @@ def test_mlp_training_step_replays_from_a_captured_graph(gpu):
         gx, ggu, gd = torch.autograd.grad(y, (x, wgu, wd), go)
         return y, gx, ggu, gd
 
+    if hasattr(torch.autograd.graph, "set_warn_on_accumulate_grad_stream_mismatch"):
+        torch.autograd.graph.set_warn_on_accumulate_grad_stream_mismatch(False)    # (leaves made on the default stream, used on a side stream)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
