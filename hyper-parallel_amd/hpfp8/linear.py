@@ -39,8 +39,13 @@ class Fp8Weight(NamedTuple):
     pow2: bool = False                  # scales are powers of two ("blockwise_pow2")
 
 
-def quantize_weight(weight: torch.Tensor, with_transpose: bool = True, pow2: bool = False) -> Fp8Weight:
-    """128x128-block quantization of a bf16 weight (and its transposed codes for dgrad)."""
+def quantize_weight(weight: torch.Tensor, with_transpose: bool = True, pow2: bool = False,
+                    per_tensor: bool = False) -> Fp8Weight:
+    """128x128-block quantization of a bf16 weight (and its transposed codes for dgrad); with ``per_tensor`` the
+    weight's form under the "per_tensor" recipe instead: codes and one scale_inv (0-dim)."""
+    if per_tensor:
+        wq, _, sw = ops.quantize_per_tensor(weight)
+        return Fp8Weight(wq, sw, None, False)
     if with_transpose:
         wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True, pow2=pow2)
         return Fp8Weight(wq, sw, wqt, pow2)
@@ -155,10 +160,11 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
 
 class _Fp8LinearPerTensor(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias):
+    def forward(ctx, x, weight, bias, wq=None, sw=None):
         x2 = _flatten(x)
         xq, _, sx = ops.quantize_per_tensor(x2)
-        wq, _, sw = ops.quantize_per_tensor(weight)
+        if wq is None:                          # no prequantized form of the weight was passed in
+            wq, _, sw = ops.quantize_per_tensor(weight)
         y = ops.gemm_per_tensor(xq, sx, wq, sw, bias=bias)
         # With one scale per tensor the codes of a transposed tensor are the transposed codes, so backward
         # needs no second quantization of x and W: it keeps the codes (1 byte per element) where their
@@ -184,7 +190,7 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
             go = go.to(torch.bfloat16)
         go = go.contiguous()
         if go.shape[0] == 0:
-            return _empty_batch_grads(ctx, go)
+            return _empty_batch_grads(ctx, go) + (None, None)
         dx = dw = db = None
         if ctx.codes_saved:
             xq, sx, wq, sw = ctx.saved_tensors
@@ -205,7 +211,7 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
                 dw = ops.gemm_per_tensor(gotq, sgot, xtq, sxt)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
-        return dx, dw, db
+        return dx, dw, db, None, None
 
 
 def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, *,
@@ -218,7 +224,7 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     128 (ragged tails are rejected, not padded); the token count may be anything (for the weight gradient,
     whose scaling groups run along the tokens, a ragged count is filled up with zero rows).
 
-    `weight_fp8` (blockwise recipe) is the weight's FP8 form made earlier -- by `quantize_weight`, or
+    `weight_fp8` is the weight's FP8 form under the same recipe made earlier -- by `quantize_weight`, or
     from all-gathered FP8 shards (`hpfp8.fsdp`) -- and saves its quantization in this call; `weight`
     is still the tensor that receives the gradient.
 
@@ -245,10 +251,14 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
                                not mg.is_contiguous()):
             raise ValueError("weight.main_grad must be a contiguous float32 tensor of the weight's shape")
     if weight_fp8 is not None:
-        if recipe == "per_tensor":
-            raise ValueError("weight_fp8 is only used by the blockwise recipes")
         if tuple(weight_fp8.codes.shape) != tuple(weight.shape):
             raise ValueError("weight_fp8 does not have the weight's shape")
+        if recipe == "per_tensor":
+            if weight_fp8.scale_inv.numel() != 1:
+                raise ValueError("weight_fp8 was not quantized with one scale per tensor")
+            return _Fp8LinearPerTensor.apply(input, weight, bias, weight_fp8.codes, weight_fp8.scale_inv)
+        if weight_fp8.scale_inv.dim() != 2:
+            raise ValueError("weight_fp8 was quantized with one scale per tensor")
         if bool(weight_fp8.pow2) != pow2:
             raise ValueError("weight_fp8 was quantized for the other blockwise recipe")
         return _Fp8LinearBlockwise.apply(input, weight, bias, weight_fp8.codes, weight_fp8.scale_inv,
@@ -286,7 +296,7 @@ class Fp8Linear(nn.Module):
                 self.bias.copy_(ref.bias)
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        if self.recipe == "per_tensor" or not self.cache_weight:
+        if not self.cache_weight:
             return fp8_linear(input, self.weight, self.bias, recipe=self.recipe,
                               apply_grad_on_fp32_main_grad=self.apply_grad_on_fp32_main_grad)
         # The FP8 form of the weight is kept until the parameter is written again (optimizer step,
@@ -294,7 +304,8 @@ class Fp8Linear(nn.Module):
         key = (self.weight._version, self.weight.data_ptr())
         if self._fp8_key != key:
             with torch.no_grad():
-                self._fp8 = quantize_weight(self.weight.detach(), with_transpose=True, pow2=self.recipe == "blockwise_pow2")
+                self._fp8 = quantize_weight(self.weight.detach(), with_transpose=True, pow2=self.recipe == "blockwise_pow2",
+                                            per_tensor=self.recipe == "per_tensor")
             self._fp8_key = key
         return fp8_linear(input, self.weight, self.bias, recipe=self.recipe, weight_fp8=self._fp8,
                           apply_grad_on_fp32_main_grad=self.apply_grad_on_fp32_main_grad)

@@ -116,6 +116,26 @@ def test_prequantized_weight_and_module_cache(gpu):
         mod.weight.mul_(2.0)                  # an in-place update, as an optimizer step is
     b = mod(x.detach())
     assert mod._fp8_key != key and torch.equal(b, hpfp8.fp8_linear(x.detach(), mod.weight.detach()))
+    # the per-tensor recipe: same bits with the weight quantized beforehand, cached by the module, refused under
+    # the other recipe
+    y0 = hpfp8.fp8_linear(x, w, recipe="per_tensor")
+    y0.backward(go)
+    gx0, gw0 = x.grad.clone(), w.grad.clone()
+    x.grad = w.grad = None
+    wf = hpfp8.quantize_weight(w.detach(), per_tensor=True)
+    y1 = hpfp8.fp8_linear(x, w, recipe="per_tensor", weight_fp8=wf)
+    y1.backward(go)
+    assert torch.equal(y1, y0) and torch.equal(x.grad, gx0) and torch.equal(w.grad, gw0)
+    with pytest.raises(ValueError):
+        hpfp8.fp8_linear(x, w, weight_fp8=wf)
+    with pytest.raises(ValueError):
+        hpfp8.fp8_linear(x, w, recipe="per_tensor", weight_fp8=hpfp8.quantize_weight(w.detach()))
+    mod = hpfp8.Fp8Linear(384, 256, bias=False, recipe="per_tensor", device=gpu)
+    with torch.no_grad():
+        mod.weight.copy_(w)
+    a = mod(x.detach())
+    first = mod._fp8
+    assert torch.equal(a, y0.detach()) and torch.equal(mod(x.detach()), a) and mod._fp8 is first
 
 
 def test_weight_gradient_onto_fp32_main_grad(gpu):
