@@ -696,6 +696,53 @@ __global__ __launch_bounds__(256) void dequant_128x128_kernel(const uint8_t* __r
   ov[1] = make_uint4(o[4], o[5], o[6], o[7]);
 }
 
+// codes with one scale for the whole tensor -> bf16 or fp32: out[i] = decode(q[i]) * scale_inv[0], one
+// multiplication and (bf16) one rounding.  16 codes per thread: one 128-bit load, 2 or 4 128-bit stores.
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void dequant_per_tensor_kernel(const uint8_t* __restrict__ q,
+                                                                 const float* __restrict__ scale_inv,
+                                                                 void* __restrict__ out, int64_t n) {
+  const float si = *scale_inv;
+  const int64_t nvec = n >> 4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < nvec) {
+    const uint4 cd = nt_load16(q + i * 16);
+    const uint32_t words[4] = {cd.x, cd.y, cd.z, cd.w};
+    float f[16];
+#pragma unroll
+    for (int wd = 0; wd < 4; ++wd) {
+      const v2f lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], false);
+      const v2f hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)words[wd], true);
+      f[4 * wd] = lo.x * si; f[4 * wd + 1] = lo.y * si; f[4 * wd + 2] = hi.x * si; f[4 * wd + 3] = hi.y * si;
+    }
+    if (OUT_F32) {
+      float* o = reinterpret_cast<float*>(out) + i * 16;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        nt_store16(o + 4 * k, make_uint4(__float_as_uint(f[4 * k]), __float_as_uint(f[4 * k + 1]),
+                                         __float_as_uint(f[4 * k + 2]), __float_as_uint(f[4 * k + 3])));
+    } else {
+      uint32_t w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const __bf16 b0 = (__bf16)f[2 * k], b1 = (__bf16)f[2 * k + 1];
+        w[k] = (uint32_t)__builtin_bit_cast(uint16_t, b0) | ((uint32_t)__builtin_bit_cast(uint16_t, b1) << 16);
+      }
+      uint16_t* o = reinterpret_cast<uint16_t*>(out) + i * 16;
+      nt_store16(o, make_uint4(w[0], w[1], w[2], w[3]));
+      nt_store16(o + 8, make_uint4(w[4], w[5], w[6], w[7]));
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (n & 15)) {       // the last n % 16 codes, one per thread
+    const int64_t j = (nvec << 4) + threadIdx.x;
+    const uint32_t c = q[j];
+    const v2f pair = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, false);
+    const float v = pair.x * si;
+    if (OUT_F32) reinterpret_cast<float*>(out)[j] = v;
+    else reinterpret_cast<uint16_t*>(out)[j] = __builtin_bit_cast(uint16_t, (__bf16)v);
+  }
+}
+
 }  // namespace hpfp8
 
 using namespace hpfp8;
@@ -997,6 +1044,23 @@ int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld,
   transpose_codes_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, (int)rows, (int)cols, ld,
                                                                            (uint8_t*)q_t, ld_t);
   return check_launch("transpose_codes");
+}
+
+int hpfp8_dequantize_per_tensor(const void* q, int64_t n, const float* scale_inv, void* out, int out_type,
+                                hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(n >= 0, HPFP8_ERR_SHAPE, "dequantize_per_tensor: negative element count");
+  HPFP8_REQUIRE(out_type == HPFP8_OUT_BF16 || out_type == HPFP8_OUT_F32, HPFP8_ERR_ARG, "dequantize_per_tensor: bad out_type");
+  if (n == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(q && scale_inv && out, HPFP8_ERR_ARG, "dequantize_per_tensor: null buffer");
+  HPFP8_REQUIRE(aligned16(q) && aligned16(out), HPFP8_ERR_ALIGN, "dequantize_per_tensor: buffers must be 16-byte aligned");
+  int64_t blocks = ((n >> 4) + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "dequantize_per_tensor: tensor too large");
+  if (out_type == HPFP8_OUT_F32)
+    dequant_per_tensor_kernel<true><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, scale_inv, out, n);
+  else
+    dequant_per_tensor_kernel<false><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, scale_inv, out, n);
+  return check_launch("dequantize_per_tensor");
 }
 
 int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols, void* out,

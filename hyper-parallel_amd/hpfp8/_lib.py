@@ -44,6 +44,7 @@ SIGNATURES = {
     "hpfp8_quantize_128x1_t_bf16": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_dequantize_1x128_bf16": [_vp, _vp, _i64, _i64, _vp, _f32, _vp],
     "hpfp8_dequantize_128x128_bf16": [_vp, _vp, _i64, _i64, _vp, _vp],
+    "hpfp8_dequantize_per_tensor": [_vp, _i64, _vp, _vp, _int, _vp],
     "hpfp8_gemm_blockwise": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp,
                              _vp, _i64, _int, _int, _vp],
     "hpfp8_gemm_blockwise_pow2": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp,

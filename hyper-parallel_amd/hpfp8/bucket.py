@@ -78,8 +78,8 @@ class Fp8GradBucket:
     def pack(self, grads: Sequence[torch.Tensor]):
         """_copy_grad_to_unsharded_buffer + cast: gradients (each shard_size * numels[e] elements) ->
         (codes [shard_size, row_elems] e4m3, scale_inv [shard_size, row_elems / 128] fp32)."""
-        ptrs = self._ptr_table(grads, [n * self.shard_size for n in self.numels])
-        dev = grads[0].device if grads else torch.device("cuda")
+        ptrs = self._ptr_table(grads, [n * self.shard_size for n in self.numels])    # (checks: all on the current GPU)
+        dev = torch.device("cuda", torch.cuda.current_device())
         q = torch.empty((self.shard_size, self.row_elems), dtype=ops.FP8, device=dev)
         scale_inv = torch.empty((self.shard_size, self.row_elems // ops.BLOCK), dtype=torch.float32, device=dev)
         _lib.call("hpfp8_bucket_pack_quantize_bf16", ptrs, self._numels_c, self._offsets_c, len(self.numels),
@@ -95,6 +95,8 @@ class Fp8GradBucket:
         if codes_row.dtype != ops.FP8 or scale_inv_row.dtype != torch.float32 or \
                 not codes_row.is_contiguous() or not scale_inv_row.is_contiguous():
             raise TypeError("codes must be contiguous float8_e4m3fn and scale_inv contiguous float32")
+        ops._check_device(codes_row, "codes_row")            # a row reduced on the host must be copied back first
+        ops._check_device(scale_inv_row, "scale_inv_row")
         ptrs = self._ptr_table(outs, self.numels)
         _lib.call("hpfp8_bucket_unpack_dequantize_bf16", ptrs, self._numels_c, self._offsets_c, len(self.numels),
                   self.row_elems, codes_row.data_ptr(), scale_inv_row.data_ptr(), ctypes.c_float(self.grad_scale),

@@ -69,5 +69,4 @@ def load_into(module: torch.nn.Module, state: Mapping[str, torch.Tensor]) -> Non
             pow2 = sub.recipe == "blockwise_pow2"
             if pow2 and bool((scale_inv.view(torch.int32) & 0x007FFFFF).any()):
                 continue        # plain fp32 scales: this module quantizes the dequantized weight itself
-            sub._fp8 = Fp8Weight(codes, scale_inv, ops.transpose_codes(codes), pow2)
-            sub._fp8_key = (sub.weight._version, sub.weight.data_ptr())
+            sub._cache.put(0, sub.weight, Fp8Weight(codes, scale_inv, ops.transpose_codes(codes), pow2))

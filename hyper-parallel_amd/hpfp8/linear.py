@@ -82,34 +82,37 @@ def _empty_batch_grads(ctx, go):
 
 class _Fp8LinearBlockwise(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, wq=None, sw=None, wqt=None, on_main_grad=False, pow2=False):
+    def forward(ctx, x, weight, bias, wq=None, sw=None, wqt=None, on_main_grad=False, pow2=False, grad_mode=True):
         ctx.main_grad_of = weight if on_main_grad else None
         ctx.pow2 = pow2
         x2 = _flatten(x)
         m = x2.shape[0]
+        # grad_mode: whether the caller ran with gradients enabled (inside this function they never are).  A
+        # Parameter has requires_grad set under torch.no_grad() too; without a backward to come nothing is
+        # prepared or kept for it.
+        need_dx, need_dw = grad_mode and x.requires_grad, grad_mode and weight.requires_grad
         # With a weight gradient to come and a token count that allows it, x is read once: its 1x128
         # codes for this GEMM and its transposed 128x1 codes for wgrad, which are what is kept for
         # backward (1 byte per element instead of the bf16 source).
-        fused = weight.requires_grad and m % ops.BLOCK == 0 and m > 0
+        fused = need_dw and m % ops.BLOCK == 0 and m > 0
         if fused:
             xq, sx, xt, sxt = ops.quantize_1x128_and_128x1_t(x2.contiguous(), kmajor=True, pow2=pow2)
         else:
             xq, sx = ops.quantize_1x128(x2, kmajor=True, pow2=pow2)
             xt = sxt = None
         if wq is None:                          # no prequantized form of the weight was passed in
-            if x.requires_grad:
+            if need_dx:
                 wq, sw, wqt = ops.quantize_128x128(weight, with_transpose=True, pow2=pow2)
             else:
                 wq, sw = ops.quantize_128x128(weight, pow2=pow2)
-        elif x.requires_grad and wqt is None:
+        elif need_dx and wqt is None:
             wqt = ops.transpose_codes(wq)
         y = ops.gemm_blockwise(xq, sx, wq, sw, bias=bias, pow2_scales=pow2)
-        ctx.save_for_backward(x2 if (weight.requires_grad and not fused) else None, xt, sxt,
-                              wqt if x.requires_grad else None, sw)
+        ctx.save_for_backward(x2 if (need_dw and not fused) else None, xt, sxt, wqt if need_dx else None, sw)
         ctx.x_shape = x.shape
         ctx.w_shape = weight.shape
         ctx.has_bias = bias is not None
-        ctx.need = (x.requires_grad, weight.requires_grad)
+        ctx.need = (need_dx, need_dw)
         return y.reshape(x.shape[:-1] + (weight.shape[0],))
 
     @staticmethod
@@ -123,7 +126,7 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
         go = go.contiguous()
         m = go.shape[0]
         if m == 0:
-            return _empty_batch_grads(ctx, go) + (None, None, None, None, None)
+            return _empty_batch_grads(ctx, go) + (None, None, None, None, None, None)
         ragged = m % ops.BLOCK != 0            # wgrad then runs on zero-padded token rows
         dx = dw = db = None
         goq = sgo = got = sgot = None
@@ -155,7 +158,7 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
                 ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=param.main_grad, accumulate=True, pow2_scales=pow2)
         if ctx.has_bias:
             db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
-        return dx, dw, db, None, None, None, None, None
+        return dx, dw, db, None, None, None, None, None, None
 
 
 class _Fp8LinearPerTensor(torch.autograd.Function):
@@ -262,14 +265,76 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
         if bool(weight_fp8.pow2) != pow2:
             raise ValueError("weight_fp8 was quantized for the other blockwise recipe")
         return _Fp8LinearBlockwise.apply(input, weight, bias, weight_fp8.codes, weight_fp8.scale_inv,
-                                         weight_fp8.codes_t, apply_grad_on_fp32_main_grad, pow2)
+                                         weight_fp8.codes_t, apply_grad_on_fp32_main_grad, pow2, torch.is_grad_enabled())
     if recipe != "per_tensor":
-        return _Fp8LinearBlockwise.apply(input, weight, bias, None, None, None, apply_grad_on_fp32_main_grad, pow2)
+        return _Fp8LinearBlockwise.apply(input, weight, bias, None, None, None, apply_grad_on_fp32_main_grad, pow2,
+                                         torch.is_grad_enabled())
     return _Fp8LinearPerTensor.apply(input, weight, bias)
 
 
+def _init_like_nn_linear(weight: torch.Tensor, bias: Optional[torch.Tensor]) -> None:
+    """torch.nn.Linear.reset_parameters, in place on the parameters' own device (no fp32 host copy of the layer)."""
+    import math
+    with torch.no_grad():
+        nn.init.kaiming_uniform_(weight, a=math.sqrt(5))
+        if bias is not None:
+            bound = 1.0 / math.sqrt(weight.shape[1]) if weight.shape[1] > 0 else 0.0
+            nn.init.uniform_(bias, -bound, bound)
+
+
+class _Fp8WeightCache:
+    """FP8 forms of a module's bf16 weights, kept between calls.
+
+    Contract.  An entry is refreshed when the parameter's autograd version counter or its data pointer changes:
+    that covers in-place updates under ``torch.no_grad()`` (what torch's optimizers do), ``copy_`` (what
+    ``load_state_dict`` does) and a parameter that was replaced.  It does NOT cover writes the version counter never
+    sees: through ``param.data``, under ``torch.autograd._unsafe_preserve_version_counter``, or by a collective that
+    refills a persistent buffer at the same address (the reference's all-gather into ``_unsharded_param``,
+    hyper_parallel/platform/torch/fully_shard/param.py:627-647).  After such a write call
+    ``module.invalidate_fp8_cache()`` -- `attach_optimizer` registers that as an optimizer step hook, and the
+    modules do it themselves after ``load_state_dict`` -- or construct the module with ``cache_weight=False``."""
+
+    def __init__(self, n: int = 1):
+        self._fp8 = [None] * n
+        self._key = [None] * n
+
+    def get(self, i: int, w: torch.Tensor, make) -> Fp8Weight:
+        key = (w._version, w.data_ptr())
+        if self._key[i] != key:
+            with torch.no_grad():
+                self._fp8[i] = make(w.detach())
+            self._key[i] = key
+        return self._fp8[i]
+
+    def put(self, i: int, w: torch.Tensor, fp8: Fp8Weight) -> None:
+        """Install an FP8 form made elsewhere (stored codes read from a checkpoint) as the cached form of w as it is now."""
+        self._fp8[i] = fp8
+        self._key[i] = (w._version, w.data_ptr())
+
+    def clear(self) -> None:
+        self._fp8 = [None] * len(self._fp8)
+        self._key = [None] * len(self._key)
+
+
+def invalidate_fp8_caches(module: nn.Module) -> None:
+    """`invalidate_fp8_cache()` on every submodule that has one."""
+    for m in module.modules():
+        f = getattr(m, "invalidate_fp8_cache", None)
+        if callable(f):
+            f()
+
+
+def attach_optimizer(optimizer: torch.optim.Optimizer, module: nn.Module):
+    """Drop the cached FP8 weights of `module` after every `optimizer.step()`, however that step writes the
+    parameters.  Returns the hook handle."""
+    return optimizer.register_step_post_hook(lambda *_: invalidate_fp8_caches(module))
+
+
 class Fp8Linear(nn.Module):
-    """Drop-in for torch.nn.Linear (bf16 parameters) whose matmuls run through fp8_linear."""
+    """Drop-in for torch.nn.Linear (bf16 parameters) whose matmuls run through fp8_linear.
+
+    With ``cache_weight`` (the default) the weight's FP8 form is kept between calls; see `_Fp8WeightCache` for when
+    it is refreshed by itself and when `invalidate_fp8_cache()` must be called."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, *, recipe: str = "blockwise",
                  cache_weight: bool = True, apply_grad_on_fp32_main_grad: bool = False, device=None,
@@ -277,8 +342,7 @@ class Fp8Linear(nn.Module):
         super().__init__()
         self.cache_weight = cache_weight
         self.apply_grad_on_fp32_main_grad = apply_grad_on_fp32_main_grad
-        self._fp8: Optional[Fp8Weight] = None
-        self._fp8_key = None
+        self._cache = _Fp8WeightCache(1)
         if recipe not in RECIPES:
             raise ValueError(f"recipe must be one of {RECIPES}, got {recipe!r}")
         if in_features % ops.BLOCK or out_features % ops.BLOCK:
@@ -287,13 +351,23 @@ class Fp8Linear(nn.Module):
         self.weight = nn.Parameter(torch.empty((out_features, in_features), device=device, dtype=dtype))
         self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=dtype)) if bias else None
         self.reset_parameters()
+        self.register_load_state_dict_post_hook(lambda module, _keys: module.invalidate_fp8_cache())
 
     def reset_parameters(self) -> None:
-        ref = nn.Linear(self.in_features, self.out_features, bias=self.bias is not None)
-        with torch.no_grad():
-            self.weight.copy_(ref.weight)
-            if self.bias is not None:
-                self.bias.copy_(ref.bias)
+        _init_like_nn_linear(self.weight, self.bias)
+        self.invalidate_fp8_cache()
+
+    def invalidate_fp8_cache(self) -> None:
+        """Forget the cached FP8 form of the weight: the next forward quantizes it again."""
+        self._cache.clear()
+
+    @property
+    def _fp8(self):
+        return self._cache._fp8[0]
+
+    @property
+    def _fp8_key(self):
+        return self._cache._key[0]
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         if not self.cache_weight:
@@ -301,13 +375,9 @@ class Fp8Linear(nn.Module):
                               apply_grad_on_fp32_main_grad=self.apply_grad_on_fp32_main_grad)
         # The FP8 form of the weight is kept until the parameter is written again (optimizer step,
         # load_state_dict, ...): micro-batches of one step and inference calls quantize it once.
-        key = (self.weight._version, self.weight.data_ptr())
-        if self._fp8_key != key:
-            with torch.no_grad():
-                self._fp8 = quantize_weight(self.weight.detach(), with_transpose=True, pow2=self.recipe == "blockwise_pow2",
-                                            per_tensor=self.recipe == "per_tensor")
-            self._fp8_key = key
-        return fp8_linear(input, self.weight, self.bias, recipe=self.recipe, weight_fp8=self._fp8,
+        f8 = self._cache.get(0, self.weight, lambda w: quantize_weight(
+            w, with_transpose=True, pow2=self.recipe == "blockwise_pow2", per_tensor=self.recipe == "per_tensor"))
+        return fp8_linear(input, self.weight, self.bias, recipe=self.recipe, weight_fp8=f8,
                           apply_grad_on_fp32_main_grad=self.apply_grad_on_fp32_main_grad)
 
     def extra_repr(self) -> str:
@@ -497,16 +567,19 @@ class Fp8SwiGLUMLP(nn.Module):
         self.hidden_size, self.intermediate_size, self.fast = hidden_size, intermediate_size, fast
         self.gate_up_proj = nn.Linear(hidden_size, 2 * intermediate_size, bias=False, device=device, dtype=dtype)
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False, device=device, dtype=dtype)
-        self._fp8 = [None, None]
-        self._fp8_key = [None, None]
+        self._cache = _Fp8WeightCache(2)
+        self.register_load_state_dict_post_hook(lambda module, _keys: module.invalidate_fp8_cache())
+
+    def invalidate_fp8_cache(self) -> None:
+        """Forget the cached FP8 forms of both weights (see `_Fp8WeightCache` for when this is needed)."""
+        self._cache.clear()
+
+    @property
+    def _fp8(self):
+        return self._cache._fp8
 
     def _weight_fp8(self, i: int, w: torch.Tensor) -> Fp8Weight:
-        key = (w._version, w.data_ptr())
-        if self._fp8_key[i] != key:
-            with torch.no_grad():
-                self._fp8[i] = quantize_weight(w.detach(), with_transpose=True)
-            self._fp8_key[i] = key
-        return self._fp8[i]
+        return self._cache.get(i, w, lambda t: quantize_weight(t, with_transpose=True))
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         wgu, wd = self.gate_up_proj.weight, self.down_proj.weight

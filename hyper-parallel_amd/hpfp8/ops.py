@@ -83,6 +83,13 @@ def _empty_codes_t(rows: int, cols: int, device) -> torch.Tensor:
     return torch.empty((rows, ld), dtype=FP8, device=device)[:, :cols]
 
 
+def _check_offs(offs: torch.Tensor) -> torch.Tensor:
+    if not isinstance(offs, torch.Tensor) or offs.dtype != torch.int32 or offs.dim() != 1 or not offs.is_contiguous():
+        raise TypeError("offs must be a contiguous 1-D int32 GPU tensor")
+    _check_device(offs, "offs")
+    return offs
+
+
 def _check_f32(x: torch.Tensor, name: str) -> torch.Tensor:
     if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32:
         raise TypeError(f"{name} must be a float32 GPU tensor")
@@ -360,12 +367,24 @@ def dequantize_1x128_accumulate(q: torch.Tensor, scale_inv: torch.Tensor, main_g
     rows = q.numel() // cols if cols else 0
     if scale_inv.numel() != rows * (cols // BLOCK) or not scale_inv.is_contiguous() or not q.is_contiguous():
         raise ValueError("q must be contiguous and scale_inv contiguous with one entry per 128 codes")
-    if main_grad.dtype != torch.float32 or not main_grad.is_cuda or not main_grad.is_contiguous() or \
-            main_grad.numel() != q.numel():
+    _check_f32(main_grad, "main_grad")
+    if not main_grad.is_contiguous() or main_grad.numel() != q.numel():
         raise ValueError("main_grad must be a contiguous float32 GPU tensor with as many elements as q")
     _lib.call("hpfp8_dequantize_1x128_accumulate_f32", _ptr(q), _ptr(scale_inv), rows, cols, _ptr(main_grad),
               ctypes.c_float(grad_scale), _stream())
     return main_grad
+
+
+def dequantize_per_tensor(q: torch.Tensor, scale_inv: torch.Tensor, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """codes (any shape) with one scale_inv (0-dim or 1-element fp32) -> decode * scale_inv as bf16 or fp32: the cast
+    back of a tensor that `quantize_per_tensor` cast in."""
+    q = _check_fp8(q, "q")
+    scale_inv = _check_f32(scale_inv, "scale_inv")
+    if scale_inv.numel() != 1:
+        raise ValueError("a per-tensor scale has exactly one element")
+    out = torch.empty(q.shape, dtype=dtype, device=q.device)
+    _lib.call("hpfp8_dequantize_per_tensor", _ptr(q), q.numel(), _ptr(scale_inv), _ptr(out), _out_code(dtype), _stream())
+    return out
 
 
 def dequantize_128x128(q: torch.Tensor, scale_inv: torch.Tensor) -> torch.Tensor:
@@ -428,7 +447,8 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
             raise ValueError("accumulate needs an existing `out`")
         out = torch.empty((m, n), dtype=out_dtype, device=a.device)
     else:
-        if tuple(out.shape) != (m, n) or out.stride(1) != 1 or not out.is_cuda:
+        _check_device(out, "out")
+        if tuple(out.shape) != (m, n) or out.stride(1) != 1:
             raise ValueError("out must be a GPU tensor [M, N] with unit inner stride")
         out_dtype = out.dtype
     if accumulate and out_dtype != torch.float32:
@@ -476,8 +496,7 @@ def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, s
     sb = _check_f32(sb, "sb")
     if a.dim() != 2 or b.dim() != 3 or a.shape[1] != b.shape[2]:
         raise ValueError(f"a {tuple(a.shape)} must be [total_m, K] and b {tuple(b.shape)} [E, N, K]")
-    if not offs.is_cuda or offs.dtype != torch.int32 or offs.dim() != 1 or not offs.is_contiguous():
-        raise TypeError("offs must be a contiguous 1-D int32 GPU tensor")
+    _check_offs(offs)
     total_m, k = a.shape
     e, n, _ = b.shape
     if offs.numel() != e:

@@ -8,16 +8,29 @@ weight dims and along the contraction dim must be multiples of 128, so that no 1
 128x128 block straddles two ranks (the kernels reject other shapes).
 
 This module imports hyper_parallel and is only loaded by hyper_parallel's own dispatcher; the hpfp8
-package never imports it.
+package never imports it.  The dispatcher finds it either as a top-level module (`distributed_op_file`, with
+HYPER_PARALLEL_OPS_PYTHON_PATH naming this directory, which the dispatcher itself puts on sys.path:
+hyper_parallel/core/shard/_op_dispatch.py:140-146, :176-186) or as `hpfp8.plugin.parallel_fp8_linear`
+(`distributed_op_module`); the sibling module with the rule is imported accordingly.
 """
-import os
-import sys
-
 from hyper_parallel.core.layout import Layout
 from hyper_parallel.core.shard.ops.parallel_ops import DistributedOp
 
-sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from layout_rule import bias_divisor, infer_fp8_linear_map  # noqa: E402  (same directory, loaded by file path)
+if __package__:
+    from .layout_rule import BLOCK, bias_divisor, infer_fp8_linear_map
+else:
+    from layout_rule import BLOCK, bias_divisor, infer_fp8_linear_map
+
+
+def check_local_shapes(x, w) -> None:
+    """The FP8 constraint on what one rank holds: the local contraction dim and the local output dim are whole
+    multiples of 128, so that no 1x128 group or 128x128 block straddles two ranks."""
+    k, n = int(w.shape[-1]), int(w.shape[0])
+    if int(x.shape[-1]) != k:
+        raise ValueError(f"fp8_linear: local contraction dims differ: input {int(x.shape[-1])}, weight {k}")
+    if k % BLOCK or n % BLOCK:
+        raise ValueError(f"fp8_linear: the local weight shard [{n}, {k}] does not hold whole 128x128 blocks; "
+                         f"shard boundaries must be multiples of {BLOCK}")
 
 
 class Fp8LinearDistributedOp(DistributedOp):
@@ -43,12 +56,15 @@ class Fp8LinearDistributedOp(DistributedOp):
         return out
 
     def get_expand_impl(self, func, output_layout, layouts, extra_args):
+        """Always a wrapper (the reference's linear returns None when there is nothing to rescale): the local
+        shards are checked against the 128 alignment before the kernels see them, and with a sharded contraction
+        the bias is pre-divided so that the all-reduce(sum) of the partial outputs adds it once."""
         x_layout = layouts[0]
         factor = bias_divisor(x_layout.alias_tensor_map, x_layout.mesh_shape, x_layout.alias_name)
-        if factor == 1 or not layouts[2]:
-            return None
+        rescale = factor != 1 and bool(layouts[2])
 
-        def expand_impl(x, w, bias):
-            return func(x, w, bias / factor)
+        def expand_impl(x, w, bias=None):
+            check_local_shapes(x, w)
+            return func(x, w, bias / factor if rescale and bias is not None else bias)
 
         return expand_impl

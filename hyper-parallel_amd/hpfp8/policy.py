@@ -25,7 +25,11 @@ class Fp8Tensor(NamedTuple):
     scale_inv: torch.Tensor      # 0-dim float32
 
     def dequantize(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-        return (self.codes.float() * self.scale_inv).to(dtype)
+        """The cast back (`.to(origin_dtype)` of hyper_parallel/core/hsdp/hsdp_grad_hook.py:32-40): decode * scale_inv
+        rounded once to bf16, or in fp32; any other dtype is a cast of the fp32 result."""
+        if dtype in (torch.bfloat16, torch.float32):
+            return ops.dequantize_per_tensor(self.codes, self.scale_inv, dtype)
+        return ops.dequantize_per_tensor(self.codes, self.scale_inv, torch.float32).to(dtype)
 
 
 @dataclass

@@ -182,6 +182,13 @@ int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld,
  * * scale_inv); when grad_scale != 1 the bf16 result is multiplied by it and rounded again. */
 int hpfp8_dequantize_1x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
                                 void* out, float grad_scale, hpfp8_stream_t stream);
+/* The cast back of the per-parameter cast hooks, HSDPGradHook._cast_hook
+ * (hyper_parallel/core/hsdp/hsdp_grad_hook.py:32-40: `.to(origin_dtype)` after the reduction) and
+ * HSDPAsyncGradHook._post_process (hyper_parallel/core/hsdp/hsdp_async_grad_hook.py:23-39), for a tensor that
+ * hpfp8_quantize_per_tensor_bf16 cast in: out[i] = decode(q[i]) * scale_inv[0] for n codes, one multiplication
+ * in fp32, rounded once to bf16 (HPFP8_OUT_BF16) or left in fp32 (HPFP8_OUT_F32). */
+int hpfp8_dequantize_per_tensor(const void* q, int64_t n, const float* scale_inv, void* out, int out_type,
+                                hpfp8_stream_t stream);
 int hpfp8_dequantize_128x128_bf16(const void* q, const float* scale_inv, int64_t rows, int64_t cols,
                                   void* out, hpfp8_stream_t stream);
 /* main_grad[i] += (decode(q[i]) * scale_inv) * grad_scale, all in fp32 (two multiplications, then the

@@ -73,7 +73,7 @@ __all__ = [
     "quantize_128x128", "quantize_128x1_t", "dequantize_per_tensor", "dequantize_1x128",
     "dequantize_128x128", "quantize_bucket", "dequantize_bucket",
     "gemm_per_tensor", "gemm_blockwise", "gemm_rowwise_both", "gemm_grouped_blockwise",
-    "gemm_dequant_f64",
+    "gemm_dequant_f64", "dequantize_per_tensor_f32", "swiglu_backward",
 ]
 
 
@@ -241,6 +241,13 @@ def dequantize_per_tensor(codes: np.ndarray, scale_inv) -> np.ndarray:
     return _to_bf16_bits_product(e4m3_decode(codes), np.float32(scale_inv)).reshape(codes.shape)
 
 
+def dequantize_per_tensor_f32(codes: np.ndarray, scale_inv) -> np.ndarray:
+    """decode(codes) * scale_inv as fp32 values (one multiplication, no second rounding): the cast back of the
+    per-parameter cast hook (hyper_parallel/core/hsdp/hsdp_grad_hook.py:32-40) when the original dtype is fp32."""
+    with np.errstate(invalid="ignore"):
+        return (e4m3_decode(codes) * np.float32(scale_inv)).astype(np.float32).reshape(np.shape(codes))
+
+
 def dequantize_1x128(codes: np.ndarray, scale_inv: np.ndarray) -> np.ndarray:
     r, c = codes.shape
     v = e4m3_decode(codes).reshape(r, c // BLOCK, BLOCK)
@@ -311,6 +318,39 @@ def swiglu_quantize_1x128(h_bits: np.ndarray, pow2: bool = False):
     act = swiglu(h_bits)
     codes, scale, scale_inv = quantize_1x128(act, pow2)
     return codes, scale, scale_inv, act
+
+
+def swiglu_backward(h_bits: np.ndarray, dact_bits: np.ndarray) -> np.ndarray:
+    """bf16 bits of d gate | d up for act = bf16(silu(gate)) * up, h = [gate | up] ([M, 2I] bf16 bits), dact [M, I]:
+        sig    = 1 / (1 + exp(-g))                     (fp32)
+        silu   = g * sig                               (fp32)
+        d up   = bf16( dact * bf16(silu) )             (the rounded silu is what forward multiplied up with)
+        d gate = bf16( (dact * up) * (sig + silu * (1 - sig)) )
+    every operation a separate fp32 rounding, in this order -- the order of the device kernel.
+
+    TOLERANCE CONTRACT.  The device kernel takes sig from the hardware's base-2 exponential and reciprocal
+    approximations (each within one unit in the last place of fp32), which no CPU reproduces bit for bit; here sig
+    is the correctly rounded fp32 value of the exact sigmoid.  The two therefore agree to a few fp32 units in the last
+    place before the final bf16 rounding: a device result is either the same bf16 value, or one bf16 step away
+    where the fp32 value sits next to a rounding boundary (d up: two steps where the bf16 rounding of silu itself
+    was such a near-tie), or -- for d gate near gate = -1.278, where sig + silu (1 - sig) passes through zero and its
+    terms cancel -- within 1e-3 * |dact * up| absolutely.  tests/test_gpu_linear.py holds the kernel to exactly
+    this, with the fraction of differing elements bounded."""
+    f = np.float32
+    h_bits = np.asarray(h_bits, dtype=np.uint16)
+    inter = h_bits.shape[-1] // 2
+    g = bf16_bits_to_f32(h_bits[..., :inter])
+    u = bf16_bits_to_f32(h_bits[..., inter:])
+    d = bf16_bits_to_f32(np.asarray(dact_bits, dtype=np.uint16))
+    with np.errstate(over="ignore"):
+        sig = (1.0 / (1.0 + np.exp(-g.astype(np.float64)))).astype(f)
+    silu = (g * sig).astype(f)
+    silu_b = bf16_bits_to_f32(f32_to_bf16_bits(silu))
+    du = (d * silu_b).astype(f)
+    one_minus = (f(1.0) - sig).astype(f)
+    deriv = (sig + (silu * one_minus).astype(f)).astype(f)
+    dg = ((d * u).astype(f) * deriv).astype(f)
+    return np.concatenate([f32_to_bf16_bits(dg), f32_to_bf16_bits(du)], axis=-1)
 
 
 def dequantize_1x128_accumulate(codes: np.ndarray, scale_inv: np.ndarray, main_grad: np.ndarray,

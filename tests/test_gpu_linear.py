@@ -229,6 +229,95 @@ def test_fp8_all_gather_hooks_rebuild_the_full_weight(gpu):
     assert torch.equal(hpfp8.fp8_linear(x, w, weight_fp8=wf), hpfp8.fp8_linear(x, w))
 
 
+def test_fsdp_extension_methods_on_the_sharded_tensor(gpu):
+    """The tensor type that carries the all-gather extension as methods: detected the way the reference detects it
+    (`hasattr(inner_tensor, ...)`, hyper_parallel/platform/torch/fully_shard/param.py:299-310), an ordinary bf16
+    parameter otherwise, and its two hooks -- called as methods with the protocol's argument lists -- rebuild the
+    whole weight's FP8 form from the per-shard pieces without a second quantization."""
+    import hpfp8
+    from hpfp8.fsdp import Fp8ShardedWeight, Fp8GatheredWeight
+    w = U.randn_bf16((512, 384), 43, 0.02).to(gpu)
+    shards = [torch.nn.Parameter(Fp8ShardedWeight(s.contiguous())) for s in w.chunk(4, dim=0)]
+    inner = shards[0]
+    assert hasattr(inner, "fsdp_pre_all_gather") and hasattr(inner, "fsdp_post_all_gather")
+    assert isinstance(inner, torch.nn.Parameter) and inner.dtype == torch.bfloat16 and inner.requires_grad
+    assert type(inner * 2) is torch.Tensor                      # arithmetic sees a plain tensor
+    with pytest.raises(ValueError):
+        Fp8ShardedWeight(w[:100])
+    outs, metas = zip(*(s.fsdp_pre_all_gather(None, s.shape, s.stride(), None, None) for s in shards))
+    assert outs[0][0].dtype == torch.uint8 and outs[0][1].dtype == torch.float32
+    bufs = (torch.cat([o[0].reshape(-1) for o in outs]), torch.cat([o[1].reshape(-1) for o in outs]))   # the all-gather
+    unsharded, inner_tensors = inner.fsdp_post_all_gather(bufs, metas[0], torch.bfloat16)
+    assert isinstance(unsharded, Fp8GatheredWeight) and unsharded.shape == (512, 384)
+    assert unsharded.data_ptr() == bufs[0].data_ptr() and inner_tensors[0] is bufs[0]      # a view, no copy
+    ref = hpfp8.quantize_weight(w, with_transpose=True)
+    wf = unsharded.as_fp8_weight()
+    assert torch.equal(wf.codes.view(torch.uint8), ref.codes.view(torch.uint8)) and torch.equal(wf.scale_inv, ref.scale_inv)
+    assert torch.equal(wf.codes_t.view(torch.uint8), ref.codes_t.view(torch.uint8))
+    x = U.randn_bf16((128, 384), 44).to(gpu).requires_grad_(True)
+    wp = w.clone().requires_grad_(True)
+    y = hpfp8.fp8_linear(x, wp, weight_fp8=wf)
+    y.backward(U.randn_bf16((128, 512), 45, 1e-3).to(gpu))
+    assert torch.equal(y, hpfp8.fp8_linear(x.detach(), w)) and x.grad is not None and wp.grad is not None
+    # a later all-gather refills the same buffers; with out= nothing is rebuilt but what was derived is dropped
+    w2 = (w.float() * 1.5).to(torch.bfloat16)
+    outs2 = [Fp8ShardedWeight(s.contiguous()).fsdp_pre_all_gather()[0] for s in w2.chunk(4, dim=0)]
+    bufs[0].copy_(torch.cat([o[0].reshape(-1) for o in outs2]))
+    bufs[1].copy_(torch.cat([o[1].reshape(-1) for o in outs2]))
+    assert inner.fsdp_post_all_gather(bufs, metas[0], torch.bfloat16, out=unsharded) is None
+    ref2 = hpfp8.quantize_weight(w2, with_transpose=True)
+    wf2 = unsharded.as_fp8_weight()
+    assert torch.equal(wf2.codes.view(torch.uint8), ref2.codes.view(torch.uint8))
+    assert torch.equal(wf2.codes_t.view(torch.uint8), ref2.codes_t.view(torch.uint8)) and torch.equal(wf2.scale_inv, ref2.scale_inv)
+
+
+def test_weight_cache_contract_and_inference_mode(gpu, monkeypatch):
+    """Writes the version counter never sees (`.data`) leave the cache stale until `invalidate_fp8_cache()` (or the
+    optimizer hook) drops it; `load_state_dict` drops it by itself.  Under `torch.no_grad()` a Parameter's
+    `requires_grad` does not make forward prepare anything for a backward."""
+    import hpfp8
+    from hpfp8 import ops
+    mod = hpfp8.Fp8Linear(384, 256, bias=False, device=gpu)
+    x = U.randn_bf16((128, 384), 51).to(gpu)
+    a = mod(x).detach().clone()
+    mod.weight.data.mul_(2.0)                                   # _version does not move
+    stale = mod(x).detach()
+    assert torch.equal(stale, a)
+    mod.invalidate_fp8_cache()
+    b = mod(x).detach()
+    assert not torch.equal(b, a) and torch.equal(b, hpfp8.fp8_linear(x, mod.weight.detach()))
+    opt = torch.optim.SGD(mod.parameters(), lr=0.5)
+    handle = hpfp8.attach_optimizer(opt, mod)
+    mod(x).float().square().mean().backward()
+    cached = mod._fp8
+    opt.step()
+    assert mod._fp8 is None and cached is not None              # the step hook dropped it
+    handle.remove()
+    c = mod(x).detach().clone()
+    sd = {k: v.clone() * 0.5 for k, v in mod.state_dict().items()}
+    mod.load_state_dict(sd)
+    assert mod._fp8 is None
+    assert not torch.equal(mod(x).detach(), c)
+    mlp = hpfp8.Fp8SwiGLUMLP(256, 384, device=gpu)
+    y0 = mlp(U.randn_bf16((128, 256), 52).to(gpu)).detach().clone()
+    mlp.down_proj.weight.data.mul_(0.5)
+    hpfp8.invalidate_fp8_caches(mlp)
+    assert not torch.equal(mlp(U.randn_bf16((128, 256), 52).to(gpu)).detach(), y0)
+    # inference: no dual quantization of x, no transposed weight codes
+    calls = []
+    real_dual, real_w = ops.quantize_1x128_and_128x1_t, ops.quantize_128x128
+    monkeypatch.setattr(ops, "quantize_1x128_and_128x1_t", lambda *a_, **k: calls.append("dual") or real_dual(*a_, **k))
+    monkeypatch.setattr(ops, "quantize_128x128", lambda *a_, **k: calls.append(("w", k.get("with_transpose", False))) or real_w(*a_, **k))
+    w = torch.nn.Parameter(U.randn_bf16((256, 384), 53, 0.02).to(gpu))
+    xr = x.clone().requires_grad_(True)
+    with torch.no_grad():
+        y_inf = hpfp8.fp8_linear(xr, w)
+    assert calls == [("w", False)] and not y_inf.requires_grad
+    calls.clear()
+    y_tr = hpfp8.fp8_linear(xr, w)
+    assert calls == ["dual", ("w", True)] and torch.equal(y_tr.detach(), y_inf)
+
+
 def test_fp8_checkpoint_round_trip(gpu, tmp_path):
     """Weights written as `weight` (float8_e4m3fn) + `weight_scale_inv` (the DeepSeek-V3 convention)
     and read back: the loaded module computes with the stored codes, so its output equals the
@@ -278,6 +367,14 @@ def test_policy_record_and_fp8_cast_hook(gpu):
     rq, _, rsi = O.quantize_per_tensor(U.bits(x))
     assert np.array_equal(U.codes(t.codes), rq) and np.array_equal(U.f32_bits(U.f32(t.scale_inv)), U.f32_bits(rsi))
     assert rel(t.dequantize(torch.float32), x.float()) < 0.05
+    # the cast back is the library's kernel, bit for bit the oracle's decode * scale_inv (bf16: rounded once)
+    assert np.array_equal(U.bits(t.dequantize()), O.dequantize_per_tensor(rq, rsi))
+    assert np.array_equal(U.f32_bits(U.f32(t.dequantize(torch.float32))), U.f32_bits(O.dequantize_per_tensor_f32(rq, rsi)))
+    assert t.dequantize(torch.float16).dtype == torch.float16
+    odd = hpfp8.cast_fp_tensor(torch.float8_e4m3fn, x.reshape(-1)[:1000 * 3 + 7].contiguous())       # n % 16 != 0
+    oq, _, osi = O.quantize_per_tensor(U.bits(x.reshape(-1)[:3007]))
+    assert np.array_equal(U.bits(odd.dequantize()), O.dequantize_per_tensor(oq, osi))
+    assert np.array_equal(U.f32_bits(U.f32(odd.dequantize(torch.float32))), U.f32_bits(O.dequantize_per_tensor_f32(oq, osi)))
     pol = hpfp8.Fp8MixedPrecisionPolicy(apply_grad_on_fp32_main_grad=True, fp8_recipe="blockwise_pow2")
     w = U.randn_bf16((256, 384), 92, 0.02).to(gpu).requires_grad_(True)
     hpfp8.fp8_linear(x, w, **pol.linear_kwargs()).backward(U.randn_bf16((256, 256), 93, 1e-3).to(gpu))
@@ -344,6 +441,16 @@ def test_swiglu_backward_kernel_vs_torch_autograd(gpu):
         assert bool(((d <= 2) | small).all()) and float(((d > 1) & ~small).float().mean()) < 1e-4
         assert float(((d != 0) & ~small).float().mean()) < 0.02
     assert rel(dh[:, :inter], g.grad) < 5e-3 and rel(dh[:, inter:], du_f32) < 5e-3
+    # against the oracle's restatement of the same operation order (oracle/fp8_oracle.py swiglu_backward), to the
+    # tolerance contract stated there: same bf16 value, or one step (d up: two) where a last-place difference of the
+    # hardware's sigmoid crosses a rounding boundary, or inside the cancellation slack of silu'
+    want = U.from_bits(O.swiglu_backward(U.bits(h), U.bits(da))).to(gpu)
+    for lo, hi, steps, slack in ((0, inter, 1, 1e-3 * scale), (inter, 2 * inter, 2, 0 * scale)):
+        got_h, want_h = dh[:, lo:hi], want[:, lo:hi]
+        d = (got_h.view(torch.int16).int() - want_h.view(torch.int16).int()).abs()
+        small = (got_h.float() - want_h.float()).abs() <= slack + 1e-30
+        assert bool(((d <= steps) | small).all())
+        assert float(((d != 0) & ~small).float().mean()) < 5e-3
     wide = torch.zeros((m, 2 * inter + 64), dtype=torch.bfloat16, device=gpu)
     wide[:, :2 * inter] = h
     assert torch.equal(hpfp8.ops.swiglu_backward(wide[:, :2 * inter], da), dh)

@@ -355,6 +355,24 @@ def test_bucket_argument_checks(gpu):
         b.pack([good[0], torch.zeros(200, dtype=torch.float32, device=gpu)])
     q, si = b.pack(good)
     assert q.shape == (2, 384) and si.shape == (2, 3) and not bool(q.view(torch.uint8).any())
+    # tensors that do not live on the current GPU never reach a kernel: a row reduced on the host, a host gradient
+    outs = [torch.empty(256, dtype=torch.bfloat16, device=gpu), torch.empty(100, dtype=torch.bfloat16, device=gpu)]
+    with pytest.raises(ValueError, match="must live on the GPU"):
+        b.unpack(q[0].cpu(), si[0], outs)
+    with pytest.raises(ValueError, match="must live on the GPU"):
+        b.unpack(q[0], si[0].cpu(), outs)
+    with pytest.raises(TypeError):
+        b.unpack(q[0], si[0], [outs[0].cpu(), outs[1]])
+    with pytest.raises(TypeError):
+        b.pack([good[0].cpu(), good[1]])
+    xq, sx = hpfp8.quantize_1x128(torch.zeros((128, 128), dtype=torch.bfloat16, device=gpu), kmajor=True)
+    wq, sw = hpfp8.quantize_128x128(torch.zeros((128, 128), dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(ValueError, match="must live on the GPU"):
+        hpfp8.gemm_blockwise(xq, sx, wq, sw, out=torch.empty((128, 128), dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="must live on the GPU"):
+        hpfp8.gemm_grouped_blockwise(xq, sx, wq.view(1, 128, 128), sw.view(1, 1, 1), torch.tensor([128], dtype=torch.int32))
+    with pytest.raises((TypeError, ValueError)):
+        hpfp8.dequantize_1x128_accumulate(xq, sx.contiguous(), torch.zeros((128, 128)))
 
 
 @pytest.mark.parametrize("shape,kmajor", [((256, 768), True), ((100, 256), False), ((512, 36864), True)])

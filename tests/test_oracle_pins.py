@@ -496,3 +496,73 @@ def test_c_restatement_of_pow2_scales_and_swiglu_bit_exact():
     h = U.randn_bf16((64, 512), 5, 2.0, 0.01, 30.0)
     h[0, :6] = torch.tensor([0.0, -0.0, 88.5, -88.5, -200.0, 200.0], dtype=torch.bfloat16)
     assert np.array_equal(O.swiglu(U.bits(h)), C.swiglu(U.bits(h)))
+
+
+def test_dequantize_accumulate_against_torch_casts_and_a_scalar_loop():
+    """`dequantize_1x128_accumulate`: with a zero main gradient and grad_scale 1 it is torch's float8 decode times
+    the group's scale_inv, exactly; in general it equals a scalar loop over elements written with torch's fp32
+    arithmetic (decode, times scale_inv, times grad_scale, plus main_grad: four roundings in that order); a
+    different association ((scale_inv * grad_scale) first) gives other bits on this data, so the order is pinned."""
+    rng = np.random.default_rng(11)
+    rows, cols = 6, 256
+    codes = rng.integers(0, 256, (rows, cols)).astype(np.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x3C                                  # (no NaN codes: compared as numbers)
+    si = (rng.uniform(0.3, 3.0, (rows, cols // 128)) * 2.0 ** rng.integers(-12, 3, (rows, cols // 128))).astype(np.float32)
+    dec = torch.from_numpy(codes).view(torch.float8_e4m3fn).float()      # torch's decode, not the oracle's
+    zero = np.zeros((rows, cols), np.float32)
+    got0 = O.dequantize_1x128_accumulate(codes, si, zero, 1.0)
+    want0 = (dec * torch.from_numpy(np.repeat(si, 128, axis=1))).numpy() + np.float32(0.0)   # (+0 + -0 = +0)
+    assert np.array_equal(got0.view(np.uint32), want0.view(np.uint32))
+    main = (rng.normal(0, 1e-2, (rows, cols))).astype(np.float32)
+    gs = 0.3
+    got = O.dequantize_1x128_accumulate(codes, si, main, gs)
+    want = np.empty_like(main)
+    tgs = torch.tensor(gs, dtype=torch.float32)
+    for r in range(rows):
+        for c in range(cols):
+            v = dec[r, c] * torch.tensor(si[r, c // 128])                 # fp32 scalar arithmetic, one rounding each
+            v = v * tgs
+            want[r, c] = float(torch.tensor(main[r, c]) + v)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    other = (main + dec.numpy() * (np.repeat(si, 128, axis=1) * np.float32(gs)).astype(np.float32)).astype(np.float32)
+    assert not np.array_equal(other.view(np.uint32), want.view(np.uint32))
+    # shape of main_grad is kept, 1-D buckets included
+    flat = O.dequantize_1x128_accumulate(codes.reshape(-1), si.reshape(-1), main.reshape(-1), gs)
+    assert flat.shape == (rows * cols,) and np.array_equal(flat.reshape(rows, cols).view(np.uint32), want.view(np.uint32))
+
+
+def test_dequantize_per_tensor_f32_is_torch_decode_times_scale():
+    codes = np.arange(256, dtype=np.uint8)
+    codes = codes[(codes & 0x7F) != 0x7F]
+    dec = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fn).float().numpy()
+    for si in (np.float32(1.0), np.float32(0.0123), np.float32(3.1e-9)):
+        got = O.dequantize_per_tensor_f32(codes, si)
+        assert np.array_equal(got.view(np.uint32), (dec * si).astype(np.float32).view(np.uint32))
+        assert np.array_equal(O.dequantize_per_tensor(codes, si), O.f32_to_bf16_bits(got))
+
+
+def test_swiglu_backward_against_float64_autograd():
+    """`swiglu_backward` against torch's float64 autograd of act = bf16(silu(gate)) * up (d up) and of
+    silu(gate) * up (d gate): within bf16 rounding of the exact derivative, and exactly zero / exactly the factor
+    at the closed-form points gate = 0 (silu' = 1/2) and large |gate| (silu' -> 1 or 0)."""
+    m, inter = 48, 256
+    h = U.randn_bf16((m, 2 * inter), 21, 2.0, 0.002, 15.0)
+    h[0, :4] = torch.tensor([0.0, -0.0, 40.0, -40.0], dtype=torch.bfloat16)
+    da = U.randn_bf16((m, inter), 22, 1e-2)
+    da[0, :4] = torch.tensor([0.5, 0.5, 0.25, 0.25], dtype=torch.bfloat16)
+    h[0, inter:inter + 4] = torch.tensor([2.0, 2.0, 4.0, 4.0], dtype=torch.bfloat16)
+    dh = U.from_bits(O.swiglu_backward(U.bits(h), U.bits(da)))
+    g = h[:, :inter].double().requires_grad_(True)
+    u = h[:, inter:].double()
+    (torch.nn.functional.silu(g) * u * da.double()).sum().backward()
+    dg_ref = g.grad
+    silu_b = torch.nn.functional.silu(h[:, :inter].double()).to(torch.bfloat16).double()
+    du_ref = da.double() * silu_b
+    for got, want in ((dh[:, :inter], dg_ref), (dh[:, inter:], du_ref)):
+        err = (got.double() - want).abs()
+        # half a bf16 step of the result, plus a few fp32 steps of the factor for the cancelling region of silu'
+        assert bool((err <= want.abs() * 2.0 ** -8 + (da.double() * u).abs() * 1e-6 + 1e-40).all())
+    # closed-form points: silu'(0) = 1/2 -> d gate = dact * up / 2 = 0.5; silu'(40) = 1 -> 1.0; silu'(-40) = 0 (to fp32)
+    assert [float(v) for v in dh[0, :3]] == [0.5, 0.5, 1.0] and abs(float(dh[0, 3])) < 1e-14
+    # d up at those points: dact * bf16(silu): silu(0) = 0, silu(40) = 40, silu(-40) = -0 (to bf16)
+    assert [float(v) for v in dh[0, inter:inter + 3]] == [0.0, 0.0, 10.0] and abs(float(dh[0, inter + 3])) < 1e-14
