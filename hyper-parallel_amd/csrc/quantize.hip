@@ -80,6 +80,147 @@ __global__ __launch_bounds__(256) void cast_per_tensor_kernel(const uint16_t* __
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// per-tensor amax + cast in one launch, for tensors small enough that the grid holds them in registers
+// ---------------------------------------------------------------------------------------------
+// Each workgroup loads its slice once (VEC 128-bit vectors per thread), the grid agrees on the maximum through
+// ONE 32-bit word, and every workgroup then casts the slice it still holds: 3 bytes per element instead of the
+// 5 of the two-pass form, one launch instead of two.
+//
+// The word is the caller's amax word itself.  bf16 magnitudes are 16-bit, so while the kernel runs its upper
+// half holds the running maximum (the fp32 bit pattern of max |x| has a zero lower half) and its lower half the
+// grid's book-keeping: bits 0..14 count the workgroups that have arrived and not yet left, bit 15 is set once the
+// maximum is final.  The word must be zero at launch; it is a clean fp32 amax when the last workgroup has left.
+//   arrive : raise the upper half to the workgroup's maximum (compare-and-swap, needed by the few workgroups
+//            that raise it), then count + 1; the workgroup that makes the count reach the grid size sets bit 15
+//   wait   : poll bit 15, at most spin_limit times
+//   leave  : count - 1; the workgroup that brings it to zero clears bit 15
+// Every wait is bounded.  A workgroup whose wait runs out (the grid was not resident together for that long)
+// computes the maximum of the whole tensor by itself, publishes it and sets bit 15 for everyone, so the result
+// does not depend on how the wait ended; a workgroup that arrives after the others have left waits out its own
+// limit and does the same.  The grid is at most 256 workgroups of 256 threads (one per CU fits always).
+constexpr int kFusedMaxBlocks = 256;
+constexpr int kFusedMaxVec = 8;
+constexpr int64_t kFusedMaxElems = (int64_t)kFusedMaxBlocks * 256 * kFusedMaxVec * 8;   // 4 Mi elements
+
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* part) {
+  m = row16_max_u32(m);
+  if ((threadIdx.x & 15) == 0) part[threadIdx.x >> 4] = m;
+  __syncthreads();
+  m = row16_max_u32(part[threadIdx.x & 15]);
+  __syncthreads();
+  return m;                       // the same in every thread
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void quant_per_tensor_fused_kernel(const uint16_t* __restrict__ x, int64_t n,
+                                                                     uint32_t* __restrict__ word,
+                                                                     uint8_t* __restrict__ q,
+                                                                     float* __restrict__ scale_out,
+                                                                     float* __restrict__ scale_inv_out,
+                                                                     uint32_t spin_limit) {
+  __shared__ uint32_t part[16];
+  __shared__ uint32_t s_amax, s_alone;
+  const uint4* xv = reinterpret_cast<const uint4*>(x);
+  const int64_t nvec = n >> 3;
+  const int64_t base = (int64_t)blockIdx.x * (256 * VEC) + threadIdx.x;
+  uint4 v[VEC];
+  uint32_t m = 0;
+#pragma unroll
+  for (int u = 0; u < VEC; ++u) {
+    const int64_t i = base + u * 256;
+    v[u] = i < nvec ? nt_load16(&xv[i]) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int u = 0; u < VEC; ++u) m = umax(m, mag8(v[u]));
+  uint32_t tail = 0;              // the last n % 8 elements, one per thread of workgroup 0
+  const bool has_tail = blockIdx.x == 0 && threadIdx.x < (n & 7);
+  if (has_tail) {
+    tail = x[(nvec << 3) + threadIdx.x];
+    m = umax(m, tail & 0x7FFFu);
+  }
+  m = block_max_u32(m, part);
+  const uint32_t grid = gridDim.x;
+  if (threadIdx.x == 0) {
+    uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while ((old >> 16) < m) {
+      const uint32_t want = (m << 16) | (old & 0xFFFFu);
+      if (__hip_atomic_compare_exchange_strong(word, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+        break;
+    }
+    const uint32_t before = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((before & 0x7FFFu) + 1u == grid) __hip_atomic_fetch_or(word, 0x8000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t now = 0, spins = 0;
+    bool done = false;
+    while (true) {
+      now = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (now & 0x8000u) { done = true; break; }
+      if (spins++ >= spin_limit) break;
+      __builtin_amdgcn_s_sleep(2);
+    }
+    s_amax = now >> 16;
+    s_alone = done ? 0u : 1u;
+  }
+  __syncthreads();
+  uint32_t amax16 = s_amax;
+  if (s_alone) {                  // (uniform over the workgroup) the wait ran out: the whole tensor's maximum, alone
+    uint32_t mm = m;
+    for (int64_t i = threadIdx.x; i < nvec; i += 256) mm = umax(mm, mag8(xv[i]));
+    if (threadIdx.x < (n & 7)) mm = umax(mm, x[(nvec << 3) + threadIdx.x] & 0x7FFFu);
+    amax16 = block_max_u32(mm, part);
+    if (threadIdx.x == 0) {
+      uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      while ((old >> 16) < amax16) {
+        const uint32_t want = (amax16 << 16) | (old & 0xFFFFu);
+        if (__hip_atomic_compare_exchange_strong(word, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+          break;
+      }
+      __hip_atomic_fetch_or(word, 0x8000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  float scale, scale_inv;
+  scales_from_amax(__uint_as_float(amax16 << 16), scale, scale_inv);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (scale_out) *scale_out = scale;
+    if (scale_inv_out) *scale_inv_out = scale_inv;
+  }
+  uint2* qv = reinterpret_cast<uint2*>(q);
+#pragma unroll
+  for (int u = 0; u < VEC; ++u) {
+    const int64_t i = base + u * 256;
+    if (i < nvec) nt_store8(&qv[i], cvt8<true>(v[u], scale));
+  }
+  if (has_tail) q[(nvec << 3) + threadIdx.x] = (uint8_t)(cvt2<false, true>(0u, tail, scale) & 0xFFu);
+  if (threadIdx.x == 0) {
+    const uint32_t before = __hip_atomic_fetch_sub(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((before & 0x7FFFu) == 1u) __hip_atomic_fetch_and(word, 0xFFFF0000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// Polls a waiting workgroup makes before it stops relying on the others (about a microsecond each).
+static uint32_t g_spin_limit = 1u << 22;
+
+// Launches fill + fused kernel; `word` (device, 4 bytes) is zeroed first by a kernel (not a memset node, so the
+// sequence can be captured in a graph).  n in (0, kFusedMaxElems].
+static int launch_per_tensor_fused(const void* x, int64_t n, void* q, uint32_t* word, float* scale, float* scale_inv,
+                                   hipStream_t s) {
+  fill_u32_kernel<<<1, 64, 0, s>>>(word, 0u, 1);
+  const int64_t nvec = (n >> 3) > 0 ? (n >> 3) : 1;
+  const int64_t per_thread = (nvec + (int64_t)kFusedMaxBlocks * 256 - 1) / ((int64_t)kFusedMaxBlocks * 256);
+  const int vec = per_thread <= 1 ? 1 : (per_thread <= 2 ? 2 : (per_thread <= 4 ? 4 : 8));
+  const unsigned grid = (unsigned)((nvec + 256 * vec - 1) / (256 * vec));
+  const uint16_t* xs = (const uint16_t*)x;
+  uint8_t* q8 = (uint8_t*)q;
+  switch (vec) {
+    case 1: quant_per_tensor_fused_kernel<1><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
+    case 2: quant_per_tensor_fused_kernel<2><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
+    case 4: quant_per_tensor_fused_kernel<4><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
+    default: quant_per_tensor_fused_kernel<8><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
+  }
+  return check_launch("quantize_per_tensor");
+}
+
 // ---------------------------------------------------------------------------------------------
 // 1x128 groups along the contiguous dim (activations, gradient buckets)
 // ---------------------------------------------------------------------------------------------
@@ -785,10 +926,15 @@ int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void
 
 int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
                                    float* scale_inv, hpfp8_stream_t stream) {
-  int rc = hpfp8_amax_bf16(x, n, amax, stream);
+  if (n > 0 && n <= kFusedMaxElems && amax && x && q && aligned16(x) && aligned16(q))
+    return launch_per_tensor_fused(x, n, q, reinterpret_cast<uint32_t*>(amax), scale, scale_inv, (hipStream_t)stream);
+  int rc = hpfp8_amax_bf16(x, n, amax, stream);      // (also reports the argument errors)
   if (rc != HPFP8_OK) return rc;
   return hpfp8_cast_per_tensor_bf16(x, n, amax, q, scale, scale_inv, stream);
 }
+
+void hpfp8_debug_set_spin_limit(uint32_t polls) { g_spin_limit = polls; }
+
 
 int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
                               float* scale_inv, hpfp8_stream_t stream) {

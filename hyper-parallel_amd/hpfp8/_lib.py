@@ -80,6 +80,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = _int
+    lib.hpfp8_debug_set_spin_limit.argtypes = [ctypes.c_uint32]
+    lib.hpfp8_debug_set_spin_limit.restype = None
     lib.hpfp8_last_error.argtypes = []
     lib.hpfp8_last_error.restype = ctypes.c_char_p
     _lib = lib

@@ -67,9 +67,17 @@ int hpfp8_amax_bf16(const void* x, int64_t n, float* amax_out, hpfp8_stream_t st
 int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void* q, float* scale,
                                float* scale_inv, hpfp8_stream_t stream);
 
-/* amax followed by cast: amax (fp32[1], required) is written then consumed. */
+/* amax followed by cast: amax (fp32[1], required) is written then consumed.  Up to 4 Mi elements this is one
+ * pass over x (3 bytes per element): the grid keeps x in registers and agrees on the maximum through the amax
+ * word itself, whose lower half serves as its counter while the kernel runs; larger tensors take the two passes
+ * above.  Either way amax holds max |x| as a clean fp32 when the call's kernels have finished. */
 int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
                                    float* scale_inv, hpfp8_stream_t stream);
+
+/* Test hook, not part of the path: how many times a workgroup of the one-pass per-tensor quantizer polls for the
+ * rest of its grid before it computes the tensor's maximum alone (default 2^22, about seconds).  0 forces that
+ * path, which must give the same results. */
+void hpfp8_debug_set_spin_limit(uint32_t polls);
 
 /* ---- blockwise quantizers --------------------------------------------------------------------
  * Operand preparation for the linear of hyper_parallel/core/shard/_op_dispatch.py:277-283. */

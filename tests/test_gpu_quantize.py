@@ -505,6 +505,37 @@ def test_dequantize_accumulate_into_fp32_main_grad(gpu):
     assert np.array_equal(U.f32_bits(U.f32(again)), U.f32_bits(want2))
 
 
+@pytest.mark.parametrize("n", [5, 8, 3007, 2048 * 1024, 4 * 1024 * 1024, 4 * 1024 * 1024 + 8])
+def test_per_tensor_one_pass_form_and_its_bounded_wait(gpu, n):
+    """Per-tensor quantization on both sides of the size where one pass over x (the grid keeps it in registers and
+    agrees on the maximum through the amax word) gives way to two passes: codes, both scales and the amax word equal
+    the oracle's bit for bit -- also when every workgroup's wait for the others is cut to nothing from the host, so
+    that each computes the maximum alone (the kernel's exit path for a grid that is not resident together)."""
+    import hpfp8
+    from hpfp8 import _lib
+    x = (U.randn_bf16((n,), 100 + n % 7, 1.0, 0.0005, 30.0)).to(gpu)
+    rq, rs, rsi = O.quantize_per_tensor(U.bits(x))
+    ram = np.float32(np.abs(x.float().cpu().numpy()).max())
+    lib = _lib.load()
+    try:
+        for limit in (1 << 22, 0):
+            lib.hpfp8_debug_set_spin_limit(limit)
+            for _ in range(2):
+                q = torch.empty((n,), dtype=torch.float8_e4m3fn, device=gpu)
+                am = torch.full((1,), float("nan"), dtype=torch.float32, device=gpu)      # (garbage in the word before the call)
+                sc = torch.empty((2,), dtype=torch.float32, device=gpu)
+                _lib.call("hpfp8_quantize_per_tensor_bf16", x.data_ptr(), n, q.data_ptr(), am.data_ptr(), sc.data_ptr(),
+                          sc.data_ptr() + 4, torch.cuda.current_stream().cuda_stream)
+                torch.cuda.synchronize()
+                assert np.array_equal(U.codes(q), rq)
+                assert U.f32_bits(U.f32(sc))[0] == U.f32_bits(rs) and U.f32_bits(U.f32(sc))[1] == U.f32_bits(rsi)
+                assert U.f32_bits(U.f32(am))[0] == U.f32_bits(ram), "the amax word is not a clean fp32 maximum"
+    finally:
+        lib.hpfp8_debug_set_spin_limit(1 << 22)
+    q2, s2, si2 = hpfp8.quantize_per_tensor(x)
+    assert np.array_equal(U.codes(q2), rq) and U.f32_bits(U.f32(si2)) == U.f32_bits(rsi)
+
+
 def test_tensors_beyond_2_31_elements(gpu):
     """4.3 GB of bf16 (2.15e9 elements): element offsets no longer fit 32 bits.  Every quantizer gives, on
     row blocks at the start, across the 2^31-element mark and at the end, the bits it gives for those rows
