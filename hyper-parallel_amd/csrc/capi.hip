@@ -26,7 +26,9 @@ int hpfp8_check_device(void) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return hpfp8::fail(HPFP8_ERR_DEVICE, "device %d is %s; this library is built for gfx950 only", dev,
                        prop.gcnArchName);
-  return HPFP8_OK;
+  // set-up work for this device: the address of the library's own device memory (used by
+  // hpfp8_quantize_per_tensor_noalloc_bf16), so that the first such call needs no set-up of its own
+  return hpfp8::prepare_scratch();
 }
 
 }  // extern "C"

@@ -10,6 +10,7 @@
 namespace hpfp8 {
 
 char* error_buffer();  // thread-local, defined in capi.hip
+int prepare_scratch();  // quantize.hip: resolves the no-allocation entry point's device memory on the current device
 
 inline int fail(int code, const char* fmt, ...) {
   va_list ap;

@@ -4,10 +4,50 @@
 // 16-bit integers (exact for bf16), amax reduced across lanes with DPP, scale = 448/amax by a
 // full IEEE division, E4M3 conversion with the hardware packed converter after an explicit
 // clamp to +-448, 64/128-bit stores.
+#include <mutex>
+
 #include "hpfp8_device.h"
 #include "hpfp8_host.h"
 
 namespace hpfp8 {
+
+// ---------------------------------------------------------------------------------------------
+// device memory for the entry point that allocates nothing
+// ---------------------------------------------------------------------------------------------
+// hpfp8_quantize_per_tensor_noalloc_bf16 keeps its amax word here instead of taking it from the caller.  Every
+// GPU holds its own copy of this array for the life of the process.  In host code the array's name is only a
+// handle: the address kernels can use is asked for once per device (scratch_for_current_device) and that pointer is
+// what is passed on; the array keeps the previous call's contents, so a call clears the word it uses first.
+constexpr int kScratchWords = 64;
+static __device__ __align__(256) uint32_t scratch[kScratchWords];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static uint32_t* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// The scratch array's device address on the current device (resolved on the first call per device); nullptr
+// with the error text set if HIP refuses.
+static uint32_t* scratch_for_current_device() {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(HPFP8_ERR_DEVICE, "scratch: no usable current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index beyond 63");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    uint32_t* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      fail(HPFP8_ERR_DEVICE, "scratch: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  return g_scratch_ptr[dev];
+}
+
+int prepare_scratch() { return scratch_for_current_device() ? HPFP8_OK : HPFP8_ERR_DEVICE; }
 
 // ---------------------------------------------------------------------------------------------
 // per-tensor amax
@@ -935,6 +975,20 @@ int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* ama
 
 void hpfp8_debug_set_spin_limit(uint32_t polls) { g_spin_limit = polls; }
 
+int hpfp8_quantize_per_tensor_noalloc_bf16(const void* x, int64_t n, void* q, float* scale, float* scale_inv,
+                                           hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(n >= 0, HPFP8_ERR_SHAPE, "quantize_per_tensor_noalloc: negative element count");
+  HPFP8_REQUIRE(n <= kFusedMaxElems, HPFP8_ERR_SHAPE,
+                "quantize_per_tensor_noalloc: %lld elements exceed the maximum of %lld this entry point serves; use "
+                "hpfp8_quantize_per_tensor_bf16 with an amax word of your own",
+                (long long)n, (long long)kFusedMaxElems);
+  if (n == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(x && q && aligned16(x) && aligned16(q), HPFP8_ERR_ALIGN,
+                "quantize_per_tensor_noalloc: buffers must be non-null and 16-byte aligned");
+  uint32_t* word = scratch_for_current_device();     // (a pointer asked for once per device; never the array's name)
+  if (!word) return HPFP8_ERR_DEVICE;
+  return launch_per_tensor_fused(x, n, q, word, scale, scale_inv, (hipStream_t)stream);
+}
 
 int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
                               float* scale_inv, hpfp8_stream_t stream) {

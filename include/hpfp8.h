@@ -74,6 +74,18 @@ int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void
 int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
                                    float* scale_inv, hpfp8_stream_t stream);
 
+/* hpfp8_quantize_per_tensor_bf16 for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the amax word is not supplied by the caller but lives in
+ * 256 bytes of device memory the library holds on every GPU it runs on until the process ends, so the call
+ * needs no workspace and allocates nothing.  No counterpart in the reference.  Same codes, scale and scale_inv
+ * as hpfp8_quantize_per_tensor_bf16.  At most 4,194,304 elements (the one-pass form; more is HPFP8_ERR_SHAPE).
+ * All calls on one GPU share that memory: calls that overlap on one GPU (different streams without ordering)
+ * race and may produce wrong scales; calls ordered on a stream, or separated by events, are safe.  The
+ * memory's address is resolved on the first call per device, or by hpfp8_check_device() made with that device
+ * current (do one of the two before capturing a graph). */
+int hpfp8_quantize_per_tensor_noalloc_bf16(const void* x, int64_t n, void* q, float* scale, float* scale_inv,
+                                           hpfp8_stream_t stream);
+
 /* Test hook, not part of the path: how many times a workgroup of the one-pass per-tensor quantizer polls for the
  * rest of its grid before it computes the tensor's maximum alone (default 2^22, about seconds).  0 forces that
  * path, which must give the same results. */
