@@ -300,7 +300,7 @@ def other_configs(dev):
         xg4.grad = wg4.grad = None
     ms3 = _time(grouped_train, iters=3, warm=3)
     res["cfg4_moe_grouped_forward_backward"] = dict(tf(3 * 2.0 * total * n * k, ms3),
-                                                    note="grouped forward and dgrad, per-expert wgrad GEMMs, quantizers")
+                                                    note="quantizers (weights included), grouped forward, dgrad and wgrad GEMMs: no host read of offs")
     del xg4, wg4, go4
     torch.cuda.empty_cache()
     # cfg 5: gradient bucket, 2^29 elements

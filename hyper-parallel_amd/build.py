@@ -11,7 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "hpfp8", "libhpfp8.so")
-SOURCES = ["capi.hip", "quantize.hip", "bucket.hip", "gemm.hip"]
+SOURCES = ["capi.hip", "quantize.hip", "bucket.hip", "grouped.hip", "gemm.hip"]
 HEADERS = ["hpfp8_device.h", "hpfp8_host.h", os.path.join("..", "..", "include", "hpfp8.h")]
 
 

@@ -23,8 +23,10 @@
 //     accumulate, c's old values are the accumulators' starting values, loaded before the tile's first round.
 //   * One kernel template, by scale form: per tensor, 128x128 blocks of b (forward, dgrad), per-row
 //     scales on both operands (wgrad), and the two blockwise forms again for scales that are powers of
-//     two, which the matrix instruction applies itself (no promotion FMAs); dense or grouped by expert;
-//     bf16 or fp32 output, optionally added onto what c holds.
+//     two, which the matrix instruction applies itself (no promotion FMAs); dense, grouped by expert
+//     along the rows (MoE forward and dgrad: an expert owns a range of rows of a and c and its own b), or
+//     grouped along the contraction (MoE wgrad: an expert owns a range of k-blocks of both operands and
+//     its own c); bf16 or fp32 output, optionally added onto what c holds.
 #include <type_traits>
 
 #include "hpfp8_device.h"
@@ -48,6 +50,8 @@ constexpr int kRectTiles = 32;              // tiles of the rectangle one XCD (3
 // kScalePow2Row: the same with the scales laid out as for kScaleRow.
 enum ScaleMode { kScaleTensor = 0, kScaleBlock = 1, kScaleRow = 2, kScalePow2 = 3, kScalePow2Row = 4 };
 
+enum Grouping { kDense = 0, kGroupedRows = 1, kGroupedK = 2 };
+
 struct GemmParams {
   const uint8_t* a;
   const uint8_t* b;
@@ -55,16 +59,19 @@ struct GemmParams {
   const float* sb;
   int64_t sa_sm, sa_sk;   // element strides of sa over (row, k-block)
   int64_t sb_sn, sb_sk;   // element strides of sb over (row or 128-row block, k-block)
-  int64_t sb_se;          // grouped: stride of sb between experts
+  int64_t sb_se;          // grouped by rows: stride of sb between experts
+  int64_t b_se;           // grouped by rows: bytes from one expert's b to the next
+  int64_t c_se;           // grouped along the contraction: elements from one expert's c to the next
   int sb_bytes;           // size of the sb array in bytes (block form)
   void* c;
   int64_t ldc;
   const uint16_t* bias;
-  const int32_t* offs;    // grouped: inclusive prefix sums of rows per expert
+  const int32_t* offs;    // grouped by rows: inclusive prefix sums of rows per expert
+  const int32_t* layout;  // grouped along the contraction: the table of grouped.hip
   int experts;
   int64_t lda, ldb;       // row strides of a and b in bytes (>= K)
-  int M, N, K;            // M = total rows of a
-  int tiles;              // dense: number of output tiles
+  int M, N, K;            // M = total rows of a; grouped along the contraction: K = the padded token axis
+  int tiles;              // dense: number of output tiles; grouped along the contraction: per expert
   int accumulate;
 };
 
@@ -124,14 +131,18 @@ struct TileInfo {
   int row0, row_end;   // rows [row0, row_end) of a and c that exist (row_end - row0 may be < BM)
   int n0;              // first row of b / column of c
   int expert;
+  int kb0, kbn;        // grouped along the contraction: first k-block of the tile's expert and how many (>= 1)
 };
 
-// Position `d` k-blocks after k-block kb of the current tile: how many tiles further (0..2, d <= 2)
-// and which k-block there.
-__device__ __forceinline__ int tiles_ahead(int kb, int d, int kblocks, int& kb_out) {
+// Position `d` k-blocks after k-block kb of the current tile (which has k0 k-blocks, the next one k1, every
+// tile at least one): how many tiles further (0..2, d <= 2) and which k-block there.
+__device__ __forceinline__ int tiles_ahead(int kb, int d, int k0, int k1, int& kb_out) {
   int pos = kb + d, q = 0;
-  if (pos >= kblocks) { pos -= kblocks; q = 1; }
-  if (pos >= kblocks) { pos -= kblocks; q = 2; }
+  if (pos >= k0) {
+    pos -= k0;
+    q = 1;
+    if (pos >= k1) { pos -= k1; q = 2; }
+  }
   kb_out = pos;
   return q;
 }
@@ -142,6 +153,8 @@ __device__ __forceinline__ TileInfo pick_tile(int q, TileInfo t0, TileInfo t1, T
   r.row_end = q == 2 ? t2.row_end : (q == 1 ? t1.row_end : t0.row_end);
   r.n0 = q == 2 ? t2.n0 : (q == 1 ? t1.n0 : t0.n0);
   r.expert = q == 2 ? t2.expert : (q == 1 ? t1.expert : t0.expert);
+  r.kb0 = q == 2 ? t2.kb0 : (q == 1 ? t1.kb0 : t0.kb0);
+  r.kbn = q == 2 ? t2.kbn : (q == 1 ? t1.kbn : t0.kbn);
   return r;
 }
 
@@ -154,9 +167,11 @@ __device__ __forceinline__ int expert_end(int off, int prev, int total_rows) {
 
 // SA4: the activation scales have unit stride over rows (the k-block-major layout), so a lane's four
 // of them are one 16-byte load.
-template <int MODE, bool GROUPED, bool OUT_F32, bool ACC, bool SA4>
+template <int MODE, int GROUPED, bool OUT_F32, bool ACC, bool SA4>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
   static_assert(!ACC || (OUT_F32 && MODE != kScaleTensor), "accumulating onto c: fp32 output, sums that start from c's values");
+  static_assert(GROUPED != kGroupedK || (!ACC && (MODE == kScaleRow || MODE == kScalePow2Row)),
+                "grouped along the contraction: the wgrad form");
   constexpr int kBStages = b_stages(MODE);
   constexpr bool kRowScales = MODE == kScaleRow || MODE == kScalePow2Row;   // per-row b scales, staged in LDS
   constexpr bool kPromote = MODE == kScaleBlock || MODE == kScaleRow;       // partial sums scaled by FMAs
@@ -181,7 +196,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // congruent mod 8, own L2) owns a contiguous run of numbers, and the workgroups of an XCD walk
   // through that run side by side, so at any moment they work on one rectangle.
   int total_tiles = p.tiles;
-  if (GROUPED) {
+  if (GROUPED == kGroupedK) total_tiles = p.experts * p.tiles;
+  if (GROUPED == kGroupedRows) {
     // tiles are numbered expert by expert; an expert with no rows has none
     int prev = 0, mt = 0;
     for (int e = 0; e < p.experts; ++e) {
@@ -201,17 +217,35 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     const int cnt = base + (xcd < big ? 1 : 0);
     t_first = xcd * base + (xcd < big ? xcd : big) + slot;
     my_tiles = slot < cnt ? (cnt - slot + t_step - 1) / t_step : 0;
+    if (GROUPED == kGroupedK) {
+      // Tiles differ in length (an expert's contraction is its own token count) and are numbered longest expert
+      // first.  They are dealt out in rounds of one tile per workgroup -- the XCD with index x takes positions
+      // [x * t_step, (x + 1) * t_step) of every round, consecutive tiles as before -- so that every workgroup
+      // gets the same mix of lengths and only the shortest tiles are left for the last, incomplete round.
+      t_first = xcd * t_step + slot;
+      t_step = nwg;
+      my_tiles = t_first < total_tiles ? (total_tiles - t_first + nwg - 1) / nwg : 0;
+    }
   }
   if (my_tiles == 0) return;
   const int n_pad = tiles_n * BN;
   // grouped: forward-only search state (tile numbers are asked for in increasing order)
   int g_e = 0, g_prev = 0, g_first = 0;
   auto lookup = [&](int k, TileInfo& ti) {
-    int row0 = p.M, row_end = p.M, n0 = n_pad, expert = 0;
+    int row0 = p.M, row_end = p.M, n0 = n_pad, expert = 0, kb0 = 0, kbn = GROUPED == kGroupedK ? 1 : kblocks;
     if (k < my_tiles) {
       const int t = t_first + k * t_step;
       int tm, tn;
-      if (GROUPED) {
+      if (GROUPED == kGroupedK) {
+        const int i = t / p.tiles;
+        expert = p.layout[4 * p.experts + i];
+        kb0 = p.layout[4 * expert + 2];
+        kbn = p.layout[4 * expert + 3];
+        rect_map(t - i * p.tiles, (p.M + BM - 1) / BM, tiles_n, tm, tn);
+        row0 = tm * BM;
+        row_end = row0 + BM < p.M ? row0 + BM : p.M;
+        n0 = tn * BN;
+      } else if (GROUPED == kGroupedRows) {
         int end = 0, cnt = 0;
         while (g_e < p.experts) {
           end = expert_end(p.offs[g_e], g_prev, p.M);
@@ -242,6 +276,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     ti.row_end = __builtin_amdgcn_readfirstlane(row_end);
     ti.n0 = __builtin_amdgcn_readfirstlane(n0);
     ti.expert = __builtin_amdgcn_readfirstlane(expert);
+    ti.kb0 = __builtin_amdgcn_readfirstlane(kb0);
+    ti.kbn = __builtin_amdgcn_readfirstlane(kbn);
   };
   // T0 is the tile being accumulated; transfers and scale loads run up to two k-blocks ahead and
   // so reach into T1 (and into T2 when K is a single k-block).
@@ -256,8 +292,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // (The resource runs on to the end of the tensor rather than to the end of the tile: transfers
   // through a resource that only just covers the rows they touch were measured markedly slower.  Rows
   // of a between the end of a ragged tile and the end of the tensor are read but never stored.)
-  auto span_bytes = [](int64_t rows, int64_t ld) {
-    const int64_t bytes = rows * ld;
+  auto span_bytes = [&](int64_t rows, int64_t ld) {     // up to the end of the last row's K codes
+    const int64_t bytes = rows > 0 ? (rows - 1) * ld + K : 0;
     return (int)(bytes < (int64_t)0x7FFFF000 ? bytes : (int64_t)0x7FFFF000);   // 256 rows always fit (host check)
   };
   auto rsrc_a_of = [&](const TileInfo& ti) {
@@ -267,7 +303,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   };
   auto rsrc_b_of = [&](const TileInfo& ti) {
     const int rows = N - ti.n0 > 0 ? N - ti.n0 : 0;
-    const uint8_t* base = p.b + (GROUPED ? (int64_t)ti.expert * N * p.ldb : 0) + (int64_t)(rows ? ti.n0 : 0) * p.ldb;
+    const uint8_t* base = p.b + (GROUPED == kGroupedRows ? (int64_t)ti.expert * p.b_se : 0) + (int64_t)(rows ? ti.n0 : 0) * p.ldb;
     return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, span_bytes(rows, p.ldb), 0x00020000);
   };
   uint32_t a_off[4], b_off[4];
@@ -288,10 +324,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // (wave 0), possible because that scale array is k-block-major (unit stride over rows).
   const __amdgpu_buffer_rsrc_t rsrc_sb = __builtin_amdgcn_make_buffer_rsrc(
       (void*)p.sb, 0, kRowScales ? (int)((((int64_t)kblocks - 1) * p.sb_sk + N) * 4) : 0, 0x00020000);
-  auto issue_sb_load = [&](const TileInfo& ti, int kb, int stage) {
+  auto issue_sb_load = [&](const TileInfo& ti, int kb, int stage) {      // kb counted inside the tile's own contraction
     if (kRowScales && wave == 0)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sb, (lds_ptr_t)(sb_lds + stage * BN), 16,
-                                               (uint32_t)(ti.n0 + lane * 4) * 4u, (int)(kb * p.sb_sk * 4), 0, 0);
+                                               (uint32_t)(ti.n0 + lane * 4) * 4u,
+                                               (int)(((GROUPED == kGroupedK ? ti.kb0 : 0) + kb) * p.sb_sk * 4), 0, 0);
   };
   // One transfer = 8 rows x 128 B per wave; `sub` (0..3) selects which of the wave's four 8-row groups
   // of the 256-row tile.  The four transfers of one operand tile share one LDS base (M0) and differ
@@ -336,7 +373,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     }
     int nblk_idx = (ti.n0 + wn * 128) >> 7;
     if (nblk_idx > (N >> 7) - 1) nblk_idx = (N >> 7) - 1;
-    sb_soff = ((GROUPED ? ti.expert * (int)p.sb_se : 0) + nblk_idx * (int)p.sb_sn) * 4;
+    sb_soff = ((GROUPED == kGroupedRows ? ti.expert * (int)p.sb_se : 0) + nblk_idx * (int)p.sb_sn) * 4;
   };
   auto load_scales = [&](int kb, float raw[5]) {
     if (MODE == kScaleBlock || MODE == kScalePow2)
@@ -404,17 +441,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // ---- prologue: k-block 0 of both operands, k-block 1 of b where it has three buffers, and the
   // first half of k-block 1 of a (and of b where it has two buffers)
   float s_cur[4] = {1.f, 1.f, 1.f, 1.f}, s_raw[5] = {1.f, 1.f, 1.f, 1.f, 1.f};
+  // (k-block numbers passed to transfers and scale loads are absolute: grouped along the contraction, a tile's
+  // own k-blocks start at its expert's first block kb0; otherwise kb0 is 0)
+  auto kfirst = [](const TileInfo& ti) { return GROUPED == kGroupedK ? ti.kb0 : 0; };
+  auto kcount = [&](const TileInfo& ti) { return GROUPED == kGroupedK ? ti.kbn : kblocks; };
   scale_target(T0);
-  load_scales(0, s_raw);
+  load_scales(kfirst(T0), s_raw);
   combine_scales(s_raw, s_cur);
   {
     const __amdgpu_buffer_rsrc_t ra = rsrc_a_of(T0), rb = rsrc_b_of(T0);
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) issue_tile(ra, a_off, 0, 0, sub);
+    for (int sub = 0; sub < 4; ++sub) issue_tile(ra, a_off, 0, kfirst(T0), sub);
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) issue_tile(rb, b_off, 2, 0, sub);
+    for (int sub = 0; sub < 4; ++sub) issue_tile(rb, b_off, 2, kfirst(T0), sub);
     int kb1;
-    const TileInfo t1 = pick_tile(tiles_ahead(0, 1, kblocks, kb1), T0, T1, T2);
+    const TileInfo t1 = pick_tile(tiles_ahead(0, 1, kcount(T0), kcount(T1), kb1), T0, T1, T2);
+    kb1 += kfirst(t1);
     if (kBAhead == 2) {
       const __amdgpu_buffer_rsrc_t rb1 = rsrc_b_of(t1);
 #pragma unroll
@@ -455,6 +497,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   // transfer targets (ordinal in the tile list) and their buffer resources
   int ord_1 = 0, ord_2 = 0;
   TileInfo tile_1 = T0;
+  int kofs_2 = kfirst(T0);             // first k-block of the tile the transfers two ahead go to
   __amdgpu_buffer_rsrc_t rs_a1 = rsrc_a_of(T0), rs_a2 = rs_a1, rs_b1 = rsrc_b_of(T0), rs_b2 = rs_b1;
 
   // per-tensor form: the one multiplier of the store phase, read once (inside the tile loop the loads
@@ -464,16 +507,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 
   for (int tile = 0; tile < my_tiles; ++tile) {
   if (ACC) load_old_values(T0);
-  for (int kb = 0; kb < kblocks; ++kb) {
+  const int kbn0 = kcount(T0);         // k-blocks of this tile
+  for (int kb = 0; kb < kbn0; ++kb) {
     // Where this round's transfers and scale loads go: one k-block ahead (scales, second half of
     // those tiles), two ahead (first half of those tiles, or the whole b tile when it has three
     // buffers).  Only in the last
     // two rounds of a tile does a target move on to the next tile of the list; its resource is
     // rebuilt then and stays valid when that tile becomes the current one.
     int kb1 = kb + 1, kb2 = kb + 2;
-    if (kb2 >= kblocks) {
-      const int o1 = tile + tiles_ahead(kb, 1, kblocks, kb1);
-      const int o2 = tile + tiles_ahead(kb, 2, kblocks, kb2);
+    if (kb2 >= kbn0) {
+      const int o1 = tile + tiles_ahead(kb, 1, kbn0, kcount(T1), kb1);
+      const int o2 = tile + tiles_ahead(kb, 2, kbn0, kcount(T1), kb2);
       if (o1 != ord_1) {
         ord_1 = o1;
         tile_1 = pick_tile(o1 - tile, T0, T1, T2);
@@ -486,8 +530,12 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
         const TileInfo t2 = pick_tile(o2 - tile, T0, T1, T2);
         rs_a2 = rsrc_a_of(t2);
         rs_b2 = rsrc_b_of(t2);
+        kofs_2 = kfirst(t2);
       }
     }
+    const int kb1_rel = kb1;             // inside tile_1's own contraction (what issue_sb_load counts in)
+    kb1 += kfirst(tile_1);
+    kb2 += kofs_2;
     load_scales(kb1, s_raw);
     const uint8_t* bcur = lds + (2 + bbuf) * kTileBytes;
     int bnext = bbuf + 1 == kBStages ? 0 : bbuf + 1;           // holds the next k-block
@@ -542,7 +590,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       const float* sb_row = sb_lds + sbuf * BN + wn * 128 + g * 4;
       v4f sbv[2];
       if (MODE == kScaleRow) sbv[0] = *reinterpret_cast<const v4f*>(sb_row);
-      if (MODE == kScaleRow) issue_sb_load(tile_1, kb1, snext);
+      if (MODE == kScaleRow) issue_sb_load(tile_1, kb1_rel, snext);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -590,7 +638,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       const float* sb_lane = sb_lds + sbuf * BN + wn * 128 + l16;
       int e_bi[2] = {127, 127};
       if (MODE == kScalePow2Row) e_bi[0] = (int)(__builtin_bit_cast(uint32_t, sb_lane[0]) >> 23);
-      if (MODE == kScalePow2Row) issue_sb_load(tile_1, kb1, snext);
+      if (MODE == kScalePow2Row) issue_sb_load(tile_1, kb1_rel, snext);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if (i == 6) round_sync();
@@ -661,7 +709,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   constexpr int kEsize = OUT_F32 ? 4 : 2;
   const int rows_valid = row_end - row0 < BM ? row_end - row0 : BM;
   const __amdgpu_buffer_rsrc_t rsrc_st = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(reinterpret_cast<uint8_t*>(p.c) + ((int64_t)row0 * p.ldc + ncol) * kEsize), 0,
+      (void*)(reinterpret_cast<uint8_t*>(p.c) +
+              ((int64_t)row0 * p.ldc + ncol + (GROUPED == kGroupedK ? (int64_t)T0.expert * p.c_se : 0)) * kEsize), 0,
       cols_ok && rows_valid > 0 ? (int)((((int64_t)rows_valid - 1) * p.ldc + 128) * kEsize) : 0, 0x00020000);
   const uint32_t st_lane = (uint32_t)(((wm * 64 + ge * 4) * (int)p.ldc) * kEsize + l16e * 16);
   const int st_row = (int)p.ldc * kEsize;        // bytes from one row of c to the next
@@ -752,11 +801,11 @@ static int persistent_grid(int64_t tiles) {
   return (int)g;
 }
 
-template <int MODE, bool GROUPED, bool SA4>
+template <int MODE, int GROUPED, bool SA4>
 static int launch_sa(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
   dim3 grid((unsigned)persistent_grid(tiles)), block(kGemmThreads);
   if (out_type == HPFP8_OUT_F32) {
-    if constexpr (MODE != kScaleTensor && !GROUPED) {   // (the per-tensor and grouped entry points have no accumulate)
+    if constexpr (MODE != kScaleTensor && GROUPED == kDense) {   // (the per-tensor and grouped entry points have no accumulate)
       if (p.accumulate) {
         gemm_kernel<MODE, GROUPED, true, true, SA4><<<grid, block, 0, stream>>>(p);
         return check_launch("gemm");
@@ -769,7 +818,7 @@ static int launch_sa(const GemmParams& p, int out_type, int64_t tiles, hipStream
   return check_launch("gemm");
 }
 
-template <int MODE, bool GROUPED>
+template <int MODE, int GROUPED>
 static int launch(const GemmParams& p, int out_type, int64_t tiles, hipStream_t stream) {
   if constexpr (MODE != kScaleTensor) {
     if (p.sa_sm == 1) return launch_sa<MODE, GROUPED, true>(p, out_type, tiles, stream);
@@ -843,8 +892,8 @@ static int gemm_blockwise_impl(const void* a, int64_t lda, const float* sa, int6
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   p.tiles = (int)tiles;
   if (sb_gran == 128) {
-    if (pow2) return launch<kScalePow2, false>(p, out_type, tiles, (hipStream_t)stream);
-    return launch<kScaleBlock, false>(p, out_type, tiles, (hipStream_t)stream);
+    if (pow2) return launch<kScalePow2, kDense>(p, out_type, tiles, (hipStream_t)stream);
+    return launch<kScaleBlock, kDense>(p, out_type, tiles, (hipStream_t)stream);
   }
   // per-row b scales travel to LDS as one contiguous 1 KB piece per k-block
   if (K == BK) sb_stride_k = N;     // a single k-block: the stride between k-blocks is never used
@@ -854,8 +903,8 @@ static int gemm_blockwise_impl(const void* a, int64_t lda, const float* sa, int6
                 "16-byte aligned rows)");
   HPFP8_REQUIRE(((K / BK - 1) * sb_stride_k + N) * 4 < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE,
                 "gemm_blockwise: b scale array too large");
-  if (pow2) return launch<kScalePow2Row, false>(p, out_type, tiles, (hipStream_t)stream);
-  return launch<kScaleRow, false>(p, out_type, tiles, (hipStream_t)stream);
+  if (pow2) return launch<kScalePow2Row, kDense>(p, out_type, tiles, (hipStream_t)stream);
+  return launch<kScaleRow, kDense>(p, out_type, tiles, (hipStream_t)stream);
 }
 
 int hpfp8_gemm_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
@@ -885,48 +934,91 @@ int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const
   p.M = (int)M; p.N = (int)N; p.K = (int)K;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   p.tiles = (int)tiles;
-  return launch<kScaleTensor, false>(p, out_type, tiles, (hipStream_t)stream);
+  return launch<kScaleTensor, kDense>(p, out_type, tiles, (hipStream_t)stream);
 }
 
 static int gemm_grouped_impl(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
-                             const void* b, const float* sb, const int32_t* offs, int experts,
+                             const void* b, int64_t ldb, int64_t b_stride_e, const float* sb, int64_t sb_stride_e,
+                             int64_t sb_stride_n, int64_t sb_stride_k, const int32_t* offs, int experts,
                              int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type, bool pow2,
                              hpfp8_stream_t stream) {
   HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "gemm_grouped: bad expert count %d", experts);
-  int rc = check_common("gemm_grouped", a, lda, b, K, sa, sb, total_m, N, K, nullptr, c, ldc, out_type, 0);
+  int rc = check_common("gemm_grouped", a, lda, b, ldb, sa, sb, total_m, N, K, nullptr, c, ldc, out_type, 0);
   if (rc <= 0) return rc;
   if (experts == 0) return HPFP8_OK;
   HPFP8_REQUIRE(offs != nullptr, HPFP8_ERR_ARG, "gemm_grouped: null offs");
+  HPFP8_REQUIRE(b_stride_e >= 0 && b_stride_e % 16 == 0, HPFP8_ERR_SHAPE,
+                "gemm_grouped: the stride between experts' b matrices must be a non-negative multiple of 16 bytes");
+  HPFP8_REQUIRE(sb_stride_e >= 0 && sb_stride_n >= 0 && sb_stride_k >= 0, HPFP8_ERR_SHAPE, "gemm_grouped: negative sb stride");
   GemmParams p{};
-  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = K;
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = ldb; p.b_se = b_stride_e;
   p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k;
-  p.sb_sn = K / BK; p.sb_sk = 1; p.sb_se = (N / kBlock) * (K / BK);
+  p.sb_sn = sb_stride_n; p.sb_sk = sb_stride_k; p.sb_se = sb_stride_e;
   rc = check_scale_span("gemm_grouped", total_m, K / BK, sa_stride_m, sa_stride_k, "sa");
   if (rc <= 0) return rc;
-  HPFP8_REQUIRE((int64_t)experts * p.sb_se * 4 < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE, "gemm_grouped: b scale array exceeds 2 GiB");
-  p.sb_bytes = (int)((int64_t)experts * p.sb_se * 4);
+  const int64_t sb_span = ((int64_t)(experts - 1) * sb_stride_e + (N / kBlock - 1) * sb_stride_n + (K / BK - 1) * sb_stride_k + 1) * 4;
+  HPFP8_REQUIRE(sb_span < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE, "gemm_grouped: b scale array exceeds 2 GiB");
+  p.sb_bytes = (int)sb_span;
   p.c = c; p.ldc = ldc; p.offs = offs; p.experts = experts;
   p.M = (int)total_m; p.N = (int)N; p.K = (int)K;
   // upper bound on row tiles: every expert may add one partial tile
   const int64_t tiles = (total_m / BM + experts) * ((N + BN - 1) / BN);
-  if (pow2) return launch<kScalePow2, true>(p, out_type, tiles, (hipStream_t)stream);
-  return launch<kScaleBlock, true>(p, out_type, tiles, (hipStream_t)stream);
+  if (pow2) return launch<kScalePow2, kGroupedRows>(p, out_type, tiles, (hipStream_t)stream);
+  return launch<kScaleBlock, kGroupedRows>(p, out_type, tiles, (hipStream_t)stream);
 }
 
 int hpfp8_gemm_grouped_blockwise(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
                                  const void* b, const float* sb, const int32_t* offs, int experts,
                                  int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc, int out_type,
                                  hpfp8_stream_t stream) {
-  return gemm_grouped_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, sb, offs, experts, total_m, N, K, c, ldc, out_type,
-                           false, stream);
+  return gemm_grouped_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, K, N * K, sb, (N / kBlock) * (K / BK), K / BK, 1, offs,
+                           experts, total_m, N, K, c, ldc, out_type, false, stream);
 }
 
 int hpfp8_gemm_grouped_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m,
                                       int64_t sa_stride_k, const void* b, const float* sb, const int32_t* offs,
                                       int experts, int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc,
                                       int out_type, hpfp8_stream_t stream) {
-  return gemm_grouped_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, sb, offs, experts, total_m, N, K, c, ldc, out_type,
-                           true, stream);
+  return gemm_grouped_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, K, N * K, sb, (N / kBlock) * (K / BK), K / BK, 1, offs,
+                           experts, total_m, N, K, c, ldc, out_type, true, stream);
+}
+
+int hpfp8_gemm_grouped_blockwise_strided(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m,
+                                         int64_t sa_stride_k, const void* b, int64_t ldb, int64_t b_stride_e,
+                                         const float* sb, int64_t sb_stride_e, int64_t sb_stride_n, int64_t sb_stride_k,
+                                         const int32_t* offs, int experts, int64_t total_m, int64_t N, int64_t K,
+                                         void* c, int64_t ldc, int out_type, int pow2, hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(pow2 == 0 || pow2 == 1, HPFP8_ERR_ARG, "gemm_grouped: pow2 must be 0 or 1");
+  return gemm_grouped_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, ldb, b_stride_e, sb, sb_stride_e, sb_stride_n,
+                           sb_stride_k, offs, experts, total_m, N, K, c, ldc, out_type, pow2 != 0, stream);
+}
+
+int hpfp8_gemm_grouped_wgrad(const void* a, int64_t lda, const float* sa, const void* b, int64_t ldb, const float* sb,
+                             const int32_t* layout, int experts, int64_t total_m, int64_t N, int64_t K, void* c,
+                             int out_type, hpfp8_stream_t stream) {
+  const char* what = "gemm_grouped_wgrad";
+  HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "%s: bad expert count %d", what, experts);
+  HPFP8_REQUIRE(total_m >= 0 && total_m < (int64_t)0x7FFFFF00, HPFP8_ERR_SHAPE, "%s: bad row count", what);
+  HPFP8_REQUIRE(N >= 0 && K >= 0 && N % kBlock == 0 && K % kBlock == 0, HPFP8_ERR_SHAPE,
+                "%s: N=%lld and K=%lld must be multiples of 128", what, (long long)N, (long long)K);
+  if (experts == 0 || N == 0 || K == 0) return HPFP8_OK;
+  // the GEMM behind it: rows = N (rows of grad_out^T), columns = K (rows of x^T), contraction = the padded token axis
+  const int64_t padded = (total_m / kBlock + experts) * kBlock;
+  int rc = check_common(what, a, lda, b, ldb, sa, sb, N, K, padded, nullptr, c, K, out_type, 0);
+  if (rc <= 0) return rc;
+  HPFP8_REQUIRE(layout != nullptr, HPFP8_ERR_ARG, "%s: null layout", what);
+  HPFP8_REQUIRE(aligned16(sa) && aligned16(sb), HPFP8_ERR_ALIGN, "%s: scale arrays must be 16-byte aligned", what);
+  HPFP8_REQUIRE((padded / BK) * (N > K ? N : K) * 4 < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: a scale array spans 2 GiB or more", what);
+  HPFP8_REQUIRE((int64_t)experts * (((N + BM - 1) / BM) * ((K + BN - 1) / BN)) < (int64_t)0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: too many tiles", what);
+  GemmParams p{};
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = ldb;
+  p.sa_sm = 1; p.sa_sk = N;          // [padded / 128, N]: block-major, as the grouped transposed quantizer writes them
+  p.sb_sn = 1; p.sb_sk = K;          // [padded / 128, K]
+  p.c = c; p.ldc = K; p.c_se = N * K; p.layout = layout; p.experts = experts;
+  p.M = (int)N; p.N = (int)K; p.K = (int)padded;
+  const int64_t per_expert = ((N + BM - 1) / BM) * ((K + BN - 1) / BN);
+  p.tiles = (int)per_expert;
+  return launch<kScaleRow, kGroupedK>(p, out_type, per_expert * experts, (hipStream_t)stream);
 }
 
 }  // extern "C"

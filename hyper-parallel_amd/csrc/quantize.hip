@@ -56,6 +56,10 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
 }
+__global__ void fill2_u32_kernel(uint32_t* a, uint32_t* b) {
+  if (threadIdx.x == 0) *a = 0u;
+  if (threadIdx.x == 1) *b = 0u;
+}
 
 // amax_bits receives the fp32 bit pattern of max|x| (non-negative floats order like integers).
 __global__ __launch_bounds__(256) void amax_bf16_kernel(const uint16_t* __restrict__ x, int64_t n,
@@ -125,28 +129,34 @@ __global__ __launch_bounds__(256) void cast_per_tensor_kernel(const uint16_t* __
 // per-tensor amax + cast in one launch, for tensors small enough that the grid holds them in registers
 // ---------------------------------------------------------------------------------------------
 // Each workgroup loads its slice once (VEC 128-bit vectors per thread), the grid agrees on the maximum through
-// ONE 32-bit word, and every workgroup then casts the slice it still holds: 3 bytes per element instead of the
-// 5 of the two-pass form, one launch instead of two.
-//
-// The word is the caller's amax word itself.  bf16 magnitudes are 16-bit, so while the kernel runs its upper
-// half holds the running maximum (the fp32 bit pattern of max |x| has a zero lower half) and its lower half the
-// grid's book-keeping: bits 0..14 count the workgroups that have arrived and not yet left, bit 15 is set once the
-// maximum is final.  The word must be zero at launch; it is a clean fp32 amax when the last workgroup has left.
-//   arrive : raise the upper half to the workgroup's maximum (compare-and-swap, needed by the few workgroups
-//            that raise it), then count + 1; the workgroup that makes the count reach the grid size sets bit 15
-//   wait   : poll bit 15, at most spin_limit times
-//   leave  : count - 1; the workgroup that brings it to zero clears bit 15
-// Every wait is bounded.  A workgroup whose wait runs out (the grid was not resident together for that long)
-// computes the maximum of the whole tensor by itself, publishes it and sets bit 15 for everyone, so the result
-// does not depend on how the wait ended; a workgroup that arrives after the others have left waits out its own
-// limit and does the same.  The grid is at most 256 workgroups of 256 threads (one per CU fits always).
-constexpr int kFusedMaxBlocks = 256;
+// two 32-bit words, and every workgroup then casts the slice it still holds: 3 bytes per element instead of the
+// 5 of the two-pass form, one pass instead of two.
+//   amax word : raised with an atomic maximum by the workgroups whose own maximum exceeds a (possibly stale)
+//               reading of it -- a handful of atomics, as in amax_bf16_kernel; a clean fp32 value at all times
+//   count word: every workgroup adds 1 once its maximum is published (release), then polls it (acquire) until it
+//               has reached the grid size; it is never decremented.  Both words must be zero at launch.
+// The count word is the caller's scale_inv output: when the first workgroup finally stores scale_inv there, every
+// value it can take (amax_c / 448 >= 2e-15, Inf, NaN) reads as an integer far above the grid size, so a
+// workgroup still polling sees "everyone has arrived" either way.
+// Every wait is bounded: a workgroup whose polls run out (the grid was not resident together for that long)
+// computes the maximum of the whole tensor by itself and publishes it, so the result does not depend on how the
+// wait ended.  A workgroup that arrives only after scale_inv has been stored (possible only after such a
+// time-out) finds a count above the grid size: its own + 1 has disturbed the stored value, and it stores the value
+// again at its end (the amax word is final by then: the store is ordered after the maximum that justified it).
+// The grid is at most 64 workgroups of 1024 threads (they are always resident together on a chip of 256 CUs):
+// few and large, because every arrival is an atomic on one word, and those serialise across the chip at tens of
+// nanoseconds each (256 arrivals cost more than the second pass they save).
+constexpr int kFusedMaxBlocks = 64;
+constexpr int kFusedThreads = 1024;
 constexpr int kFusedMaxVec = 8;
-constexpr int64_t kFusedMaxElems = (int64_t)kFusedMaxBlocks * 256 * kFusedMaxVec * 8;   // 4 Mi elements
+constexpr int64_t kFusedMaxElems = (int64_t)kFusedMaxBlocks * kFusedThreads * kFusedMaxVec * 8;   // 4 Mi elements
 
+// maximum over a workgroup of 1024 threads; part: 16 words of LDS
 __device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* part) {
   m = row16_max_u32(m);
-  if ((threadIdx.x & 15) == 0) part[threadIdx.x >> 4] = m;
+  m = umax(m, (uint32_t)__shfl_xor((int)m, 16));
+  m = umax(m, (uint32_t)__shfl_xor((int)m, 32));
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
   __syncthreads();
   m = row16_max_u32(part[threadIdx.x & 15]);
   __syncthreads();
@@ -154,22 +164,22 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* part) {
 }
 
 template <int VEC>
-__global__ __launch_bounds__(256) void quant_per_tensor_fused_kernel(const uint16_t* __restrict__ x, int64_t n,
-                                                                     uint32_t* __restrict__ word,
+__global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(const uint16_t* __restrict__ x, int64_t n,
+                                                                     uint32_t* __restrict__ amax_word,
+                                                                     uint32_t* __restrict__ count_word,
                                                                      uint8_t* __restrict__ q,
                                                                      float* __restrict__ scale_out,
-                                                                     float* __restrict__ scale_inv_out,
                                                                      uint32_t spin_limit) {
   __shared__ uint32_t part[16];
-  __shared__ uint32_t s_amax, s_alone;
+  __shared__ uint32_t s_amax, s_alone, s_repair;
   const uint4* xv = reinterpret_cast<const uint4*>(x);
   const int64_t nvec = n >> 3;
-  const int64_t base = (int64_t)blockIdx.x * (256 * VEC) + threadIdx.x;
+  const int64_t base = (int64_t)blockIdx.x * (kFusedThreads * VEC) + threadIdx.x;
   uint4 v[VEC];
   uint32_t m = 0;
 #pragma unroll
   for (int u = 0; u < VEC; ++u) {
-    const int64_t i = base + u * 256;
+    const int64_t i = base + u * kFusedThreads;
     v[u] = i < nvec ? nt_load16(&xv[i]) : make_uint4(0, 0, 0, 0);
   }
 #pragma unroll
@@ -183,80 +193,63 @@ __global__ __launch_bounds__(256) void quant_per_tensor_fused_kernel(const uint1
   m = block_max_u32(m, part);
   const uint32_t grid = gridDim.x;
   if (threadIdx.x == 0) {
-    uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    while ((old >> 16) < m) {
-      const uint32_t want = (m << 16) | (old & 0xFFFFu);
-      if (__hip_atomic_compare_exchange_strong(word, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-        break;
+    if ((m << 16) > __hip_atomic_load(amax_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+      __hip_atomic_fetch_max(amax_word, m << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t seen = __hip_atomic_fetch_add(count_word, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+    s_repair = seen > grid ? 1u : 0u;
+    uint32_t spins = 0;
+    while (seen < grid && spins++ < spin_limit) {
+      __builtin_amdgcn_s_sleep(1);
+      seen = __hip_atomic_load(count_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    const uint32_t before = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((before & 0x7FFFu) + 1u == grid) __hip_atomic_fetch_or(word, 0x8000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    uint32_t now = 0, spins = 0;
-    bool done = false;
-    while (true) {
-      now = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (now & 0x8000u) { done = true; break; }
-      if (spins++ >= spin_limit) break;
-      __builtin_amdgcn_s_sleep(2);
-    }
-    s_amax = now >> 16;
-    s_alone = done ? 0u : 1u;
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);          // (agent scope and wider)
+    s_amax = __hip_atomic_load(amax_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 16;
+    s_alone = seen < grid ? 1u : 0u;
   }
   __syncthreads();
   uint32_t amax16 = s_amax;
   if (s_alone) {                  // (uniform over the workgroup) the wait ran out: the whole tensor's maximum, alone
     uint32_t mm = m;
-    for (int64_t i = threadIdx.x; i < nvec; i += 256) mm = umax(mm, mag8(xv[i]));
+    for (int64_t i = threadIdx.x; i < nvec; i += kFusedThreads) mm = umax(mm, mag8(xv[i]));
     if (threadIdx.x < (n & 7)) mm = umax(mm, x[(nvec << 3) + threadIdx.x] & 0x7FFFu);
     amax16 = block_max_u32(mm, part);
-    if (threadIdx.x == 0) {
-      uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      while ((old >> 16) < amax16) {
-        const uint32_t want = (amax16 << 16) | (old & 0xFFFFu);
-        if (__hip_atomic_compare_exchange_strong(word, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-          break;
-      }
-      __hip_atomic_fetch_or(word, 0x8000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    if (threadIdx.x == 0) __hip_atomic_fetch_max(amax_word, amax16 << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   float scale, scale_inv;
   scales_from_amax(__uint_as_float(amax16 << 16), scale, scale_inv);
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    if (scale_out) *scale_out = scale;
-    if (scale_inv_out) *scale_inv_out = scale_inv;
-  }
   uint2* qv = reinterpret_cast<uint2*>(q);
 #pragma unroll
   for (int u = 0; u < VEC; ++u) {
-    const int64_t i = base + u * 256;
+    const int64_t i = base + u * kFusedThreads;
     if (i < nvec) nt_store8(&qv[i], cvt8<true>(v[u], scale));
   }
   if (has_tail) q[(nvec << 3) + threadIdx.x] = (uint8_t)(cvt2<false, true>(0u, tail, scale) & 0xFFu);
-  if (threadIdx.x == 0) {
-    const uint32_t before = __hip_atomic_fetch_sub(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((before & 0x7FFFu) == 1u) __hip_atomic_fetch_and(word, 0xFFFF0000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0 && (blockIdx.x == 0 || s_repair)) {
+    if (scale_out) *scale_out = scale;
+    // scale_inv takes the place of the count (ordered after the maximum this workgroup may have published)
+    __hip_atomic_store(count_word, __float_as_uint(scale_inv), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
 // Polls a waiting workgroup makes before it stops relying on the others (about a microsecond each).
 static uint32_t g_spin_limit = 1u << 22;
 
-// Launches fill + fused kernel; `word` (device, 4 bytes) is zeroed first by a kernel (not a memset node, so the
-// sequence can be captured in a graph).  n in (0, kFusedMaxElems].
+// Launches fill + fused kernel; the two words (device, 4 bytes each: amax, and scale_inv as the count) are zeroed
+// first by a kernel (not a memset node, so the sequence can be captured in a graph).  n in (0, kFusedMaxElems].
 static int launch_per_tensor_fused(const void* x, int64_t n, void* q, uint32_t* word, float* scale, float* scale_inv,
                                    hipStream_t s) {
-  fill_u32_kernel<<<1, 64, 0, s>>>(word, 0u, 1);
+  fill2_u32_kernel<<<1, 64, 0, s>>>(word, reinterpret_cast<uint32_t*>(scale_inv));
   const int64_t nvec = (n >> 3) > 0 ? (n >> 3) : 1;
-  const int64_t per_thread = (nvec + (int64_t)kFusedMaxBlocks * 256 - 1) / ((int64_t)kFusedMaxBlocks * 256);
+  const int64_t per_thread = (nvec + (int64_t)kFusedMaxBlocks * kFusedThreads - 1) / ((int64_t)kFusedMaxBlocks * kFusedThreads);
   const int vec = per_thread <= 1 ? 1 : (per_thread <= 2 ? 2 : (per_thread <= 4 ? 4 : 8));
-  const unsigned grid = (unsigned)((nvec + 256 * vec - 1) / (256 * vec));
+  const unsigned grid = (unsigned)((nvec + kFusedThreads * vec - 1) / (kFusedThreads * vec));
   const uint16_t* xs = (const uint16_t*)x;
   uint8_t* q8 = (uint8_t*)q;
   switch (vec) {
-    case 1: quant_per_tensor_fused_kernel<1><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
-    case 2: quant_per_tensor_fused_kernel<2><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
-    case 4: quant_per_tensor_fused_kernel<4><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
-    default: quant_per_tensor_fused_kernel<8><<<grid, 256, 0, s>>>(xs, n, word, q8, scale, scale_inv, g_spin_limit); break;
+    case 1: quant_per_tensor_fused_kernel<1><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
+    case 2: quant_per_tensor_fused_kernel<2><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
+    case 4: quant_per_tensor_fused_kernel<4><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
+    default: quant_per_tensor_fused_kernel<8><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
   }
   return check_launch("quantize_per_tensor");
 }
@@ -636,14 +629,23 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // and what is quantized is act = silu(gate) * up, computed as the tile is loaded: both operand forms of the
 // down projection's input from one read of the gate/up output, the bf16 activation never written.
 // ld_src: row stride of the source in elements (K, or at least 2K with SW).
-template <bool KMAJOR, bool DUAL, int SW = 0>
+// With GROUPED (MoE: rows of x sorted by expert) the 128-row groups restart at every expert's first row and the
+// transposed output lives on the padded token axis of `layout` (grouped.hip): output block tr belongs to expert
+// layout[5E + 1 + tr], holds that expert's rows [128 j, 128 j + 128) (j = tr - the expert's first block) and is
+// filled up with zero codes past the expert's last row; m is then the number of source rows (any count), mb the
+// number of padded blocks the grid covers, and blocks beyond those in use are left untouched.  The 1x128 form
+// (DUAL) is written for the rows that exist, at their own positions.
+template <bool KMAJOR, bool DUAL, int SW = 0, bool GROUPED = false>
 __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int m, int k,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale_t,
                                                             float* __restrict__ scale_inv_t,
                                                             uint8_t* __restrict__ q, float* __restrict__ scale_r,
-                                                            float* __restrict__ scale_inv_r, int pow2) {
-  const int kb = k >> 7, mb = m >> 7;
+                                                            float* __restrict__ scale_inv_r, int pow2,
+                                                            const int32_t* __restrict__ layout = nullptr, int experts = 0,
+                                                            int padded_blocks = 0) {
+  static_assert(!GROUPED || (SW == 0 && kTilesPerBlock == 1), "grouped form: plain source, one tile per workgroup");
+  const int kb = k >> 7, mb = GROUPED ? padded_blocks : m >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   const int wave = threadIdx.x >> 6;
   __shared__ uint32_t part[4][64];  // [wave][cg*4 + word]
@@ -655,11 +657,24 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
   const int total = kb * mb;
   const int t0 = blockIdx.x * kTilesPerBlock;
   const int t1 = t0 + kTilesPerBlock < total ? t0 + kTilesPerBlock : total;
+  // first source row of the tile and how many of its 128 rows exist (dense: tr * 128 and all of them)
+  int g_row0 = 0, g_valid = 128;
+  if (GROUPED) {
+    const int tr = t0 % mb;
+    const int e = layout[5 * experts + 1 + tr];
+    if (e < 0) return;                                   // (uniform over the workgroup) a block no expert owns
+    const int j = tr - layout[4 * e + 2];
+    g_row0 = layout[4 * e + 0] + j * 128;
+    g_valid = layout[4 * e + 1] - j * 128;
+    g_valid = g_valid < 0 ? 0 : (g_valid > 128 ? 128 : g_valid);
+  }
   auto load_tile = [&](int t, uint4 v[8]) {
     const int tc = t / mb, tr = t % mb;
-    const int64_t off = (int64_t)tr * 128 * ld_src + tc * 128 + cg * 8;
+    const int64_t off = (int64_t)(GROUPED ? g_row0 : tr * 128) * ld_src + tc * 128 + cg * 8;
 #pragma unroll
-    for (int p = 0; p < 8; ++p) v[p] = nt_load16(x + off + (int64_t)tile_row(rq, p) * ld_src);
+    for (int p = 0; p < 8; ++p)
+      v[p] = (!GROUPED || tile_row(rq, p) < g_valid) ? nt_load16(x + off + (int64_t)tile_row(rq, p) * ld_src)
+                                                     : make_uint4(0, 0, 0, 0);
     if (SW) {
 #pragma unroll
       for (int p = 0; p < 8; ++p) {
@@ -707,7 +722,9 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
           const int row = tile_row(rq, 4 * half + p);
-          *reinterpret_cast<uint2*>(q + ((int64_t)tr * 128 + row) * k + tc * 128 + cg * 8) = cvt8<false>(v[4 * half + p], s[p]);
+          if (!GROUPED || row < g_valid)
+            *reinterpret_cast<uint2*>(q + ((int64_t)(GROUPED ? g_row0 : tr * 128) + row) * k + tc * 128 + cg * 8) =
+                cvt8<false>(v[4 * half + p], s[p]);
         }
         if (cg < 4) {
           const int row = tile_row(rq, 4 * half + cg);
@@ -719,9 +736,12 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
     __syncthreads();
     if (DUAL && threadIdx.x >= 128) {
       const int row = threadIdx.x - 128;
-      const int64_t o = KMAJOR ? (int64_t)tc * m + tr * 128 + row : ((int64_t)tr * 128 + row) * kb + tc;
-      if (scale_r) scale_r[o] = s_row[row];
-      scale_inv_r[o] = s_row[128 + row];
+      const int64_t r_abs = (int64_t)(GROUPED ? g_row0 : tr * 128) + row;
+      const int64_t o = KMAJOR ? (int64_t)tc * m + r_abs : r_abs * kb + tc;
+      if (!GROUPED || row < g_valid) {
+        if (scale_r) scale_r[o] = s_row[row];
+        scale_inv_r[o] = s_row[128 + row];
+      }
     }
     if (threadIdx.x < 128) {
       const int col = threadIdx.x, word = col >> 1;
@@ -966,7 +986,7 @@ int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void
 
 int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
                                    float* scale_inv, hpfp8_stream_t stream) {
-  if (n > 0 && n <= kFusedMaxElems && amax && x && q && aligned16(x) && aligned16(q))
+  if (n > 0 && n <= kFusedMaxElems && amax && scale_inv && x && q && aligned16(x) && aligned16(q))
     return launch_per_tensor_fused(x, n, q, reinterpret_cast<uint32_t*>(amax), scale, scale_inv, (hipStream_t)stream);
   int rc = hpfp8_amax_bf16(x, n, amax, stream);      // (also reports the argument errors)
   if (rc != HPFP8_OK) return rc;
@@ -987,7 +1007,10 @@ int hpfp8_quantize_per_tensor_noalloc_bf16(const void* x, int64_t n, void* q, fl
                 "quantize_per_tensor_noalloc: buffers must be non-null and 16-byte aligned");
   uint32_t* word = scratch_for_current_device();     // (a pointer asked for once per device; never the array's name)
   if (!word) return HPFP8_ERR_DEVICE;
-  return launch_per_tensor_fused(x, n, q, word, scale, scale_inv, (hipStream_t)stream);
+  // word[0]: the amax word; word[1]: stands in for scale_inv (which doubles as the grid's arrival count) when the
+  // caller does not want that output
+  return launch_per_tensor_fused(x, n, q, word, scale, scale_inv ? scale_inv : reinterpret_cast<float*>(word + 1),
+                                 (hipStream_t)stream);
 }
 
 int hpfp8_quantize_1x128_bf16(const void* x, int64_t rows, int64_t cols, void* q, float* scale,
@@ -1129,6 +1152,36 @@ int hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, in
   else
     quant_128x1_t_kernel<true, true, 1><<<grid, 256, 0, s>>>((const uint16_t*)h, ld_h, (int)rows, (int)inter, (uint8_t*)q_t, ld_t,
                                                             scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0);
+  return check_launch(what);
+}
+
+int hpfp8_quantize_128x1_t_grouped_bf16(const void* x, int64_t total_m, int64_t k, const int32_t* layout, int experts,
+                                        void* q_t, int64_t ld_t, float* scale_inv_t, void* q, float* scale_inv,
+                                        hpfp8_stream_t stream) {
+  const char* what = "quantize_128x1_t_grouped";
+  HPFP8_REQUIRE(total_m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
+  HPFP8_REQUIRE(k % kBlock == 0, HPFP8_ERR_SHAPE, "%s: width %lld is not a multiple of 128", what, (long long)k);
+  HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "%s: bad expert count %d", what, experts);
+  HPFP8_REQUIRE(total_m < (1 << 30) && k < (1 << 30), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
+  const int64_t padded_blocks = total_m / kBlock + experts;
+  const int64_t blocks = padded_blocks * (k / kBlock);
+  if (blocks == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
+  HPFP8_REQUIRE((x || total_m == 0) && layout && q_t && scale_inv_t, HPFP8_ERR_ARG, "%s: null buffer", what);
+  HPFP8_REQUIRE(aligned16(x) && aligned16(q_t), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
+  HPFP8_REQUIRE(ld_t >= padded_blocks * kBlock && ld_t % 16 == 0, HPFP8_ERR_SHAPE,
+                "%s: ld_t=%lld must be a multiple of 16 and at least the padded row count %lld", what, (long long)ld_t,
+                (long long)(padded_blocks * kBlock));
+  HPFP8_REQUIRE(!q || (scale_inv && aligned16(q)), HPFP8_ERR_ARG, "%s: q needs scale_inv and 16-byte alignment", what);
+  hipStream_t s = (hipStream_t)stream;
+  if (q)
+    quant_128x1_t_kernel<true, true, 0, true><<<(unsigned)blocks, 256, 0, s>>>(
+        (const uint16_t*)x, k, (int)total_m, (int)k, (uint8_t*)q_t, ld_t, nullptr, scale_inv_t, (uint8_t*)q, nullptr, scale_inv, 0,
+        layout, experts, (int)padded_blocks);
+  else
+    quant_128x1_t_kernel<true, false, 0, true><<<(unsigned)blocks, 256, 0, s>>>(
+        (const uint16_t*)x, k, (int)total_m, (int)k, (uint8_t*)q_t, ld_t, nullptr, scale_inv_t, nullptr, nullptr, nullptr, 0,
+        layout, experts, (int)padded_blocks);
   return check_launch(what);
 }
 

@@ -55,6 +55,17 @@ SIGNATURES = {
                                      _int, _vp],
     "hpfp8_gemm_grouped_blockwise_pow2": [_vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _i64,
                                           _int, _vp],
+    "hpfp8_gemm_grouped_blockwise_strided": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _int,
+                                             _i64, _i64, _i64, _vp, _i64, _int, _int, _vp],
+    "hpfp8_grouped_layout": [_vp, _int, _i64, _vp, _vp],
+    "hpfp8_quantize_128x1_t_grouped_bf16": [_vp, _i64, _i64, _vp, _int, _vp, _i64, _vp, _vp, _vp, _vp],
+    "hpfp8_gemm_grouped_wgrad": [_vp, _i64, _vp, _vp, _i64, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _vp],
+    "hpfp8_grouped_zero_unrouted_rows_bf16": [_vp, _i64, _vp, _int, _i64, _i64, _vp],
+}
+# functions that return a size, not a status
+SIZE_FUNCTIONS = {
+    "hpfp8_grouped_padded_rows": [_int, _i64],
+    "hpfp8_grouped_layout_words": [_int, _i64],
 }
 
 OUT_BF16, OUT_F32 = 0, 1
@@ -81,6 +92,10 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = _int
+    for name, argtypes in SIZE_FUNCTIONS.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = _i64
     lib.hpfp8_debug_set_spin_limit.argtypes = [ctypes.c_uint32]
     lib.hpfp8_debug_set_spin_limit.restype = None
     lib.hpfp8_last_error.argtypes = []

@@ -385,67 +385,91 @@ class Fp8Linear(nn.Module):
                 f"bias={self.bias is not None}, recipe={self.recipe}")
 
 
+def quantize_grouped_weight(weight: torch.Tensor, with_transpose: bool = True) -> Fp8Weight:
+    """The blockwise FP8 form of the experts' stacked weight [E, N, K]: codes [E, N, K], scale_inv [E, N/128, K/128]
+    and (for the input gradient) the transposed codes of the stacked matrix, [K, E * N]."""
+    if weight.dim() != 3:
+        raise ValueError("weight must be [E, N, K]")
+    e, n, k = weight.shape
+    flat = weight.reshape(e * n, k)
+    if with_transpose:
+        wq, sw, wqt = ops.quantize_128x128(flat, with_transpose=True)
+    else:
+        (wq, sw), wqt = ops.quantize_128x128(flat), None
+    return Fp8Weight(wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), wqt, False)
+
+
 class _Fp8GroupedLinear(torch.autograd.Function):
-    """Grouped (MoE) linear with the blockwise recipe.  Forward and the input gradient are one grouped GEMM each
-    (the latter on the experts' transposed codes); the weight gradient of expert e contracts over that expert's own
-    token range, one dense wgrad GEMM per expert on its rows filled up with zero rows to a multiple of 128."""
+    """Grouped (MoE) linear with the blockwise recipe: forward, the input gradient and the weight gradient are one
+    grouped GEMM each.  Everything that depends on the rows per expert is derived from `offs` on the device (the
+    layout table of the padded token axis the wgrad operands live on), so nothing here reads `offs` on the host and
+    forward + backward can be captured in a HIP graph."""
 
     @staticmethod
-    def forward(ctx, x, weight, offs):
+    def forward(ctx, x, weight, offs, wq=None, sw=None, wqt=None, grad_mode=True):
         e, n, k = weight.shape
-        xq, sx = ops.quantize_1x128(x, kmajor=True)
-        wq, sw = ops.quantize_128x128(weight.reshape(e * n, k))
-        y = ops.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // ops.BLOCK, k // ops.BLOCK), offs)
-        ctx.save_for_backward(x if weight.requires_grad else None, wq if x.requires_grad else None, sw, offs)
+        total_m = x.shape[0]
+        need_dx, need_dw = grad_mode and x.requires_grad, grad_mode and weight.requires_grad
+        layout = xt = sxt = None
+        if need_dw:
+            # one read of x: its 1x128 codes for this GEMM and its transposed codes, grouped by expert, for wgrad
+            layout = ops.grouped_layout(offs, total_m)
+            xq, sx, xt, sxt = ops.quantize_128x1_t_grouped(x.contiguous(), layout, e, with_1x128=True)
+        else:
+            xq, sx = ops.quantize_1x128(x, kmajor=True)
+        if wq is None:                          # no prequantized form of the weight was passed in
+            f8 = quantize_grouped_weight(weight, with_transpose=need_dx)
+            wq, sw, wqt = f8.codes, f8.scale_inv, f8.codes_t
+        elif need_dx and wqt is None:
+            wqt = ops.transpose_codes(wq.view(e * n, k))
+        y = ops.gemm_grouped_blockwise(xq, sx, wq, sw, offs)
+        ctx.save_for_backward(xt, sxt, layout, wqt if need_dx else None, sw, offs)
         ctx.w_shape = weight.shape
-        ctx.need = (x.requires_grad, weight.requires_grad)
+        ctx.total_m = total_m
+        ctx.need = (need_dx, need_dw)
         return y
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, wq, sw, offs = ctx.saved_tensors
+        xt, sxt, layout, wqt, sw, offs = ctx.saved_tensors
         need_dx, need_dw = ctx.need
         e, n, k = ctx.w_shape
         go = grad_out.to(torch.bfloat16).contiguous()
-        ends = [min(max(int(v), 0), go.shape[0]) for v in offs.tolist()]       # (one host read of the row counts)
-        last = ends[-1] if ends else 0
         dx = dw = None
-        if need_dx:
-            # dx_e = go_e . W_e: the grouped kernel again, b = W_e^T codes [K, N] (128x128 blocks are symmetric,
-            # so W's scales serve with their two block dims swapped)
-            wt = torch.empty((e, k, n), dtype=wq.dtype, device=wq.device)
-            wq3 = wq.view(e, n, k)
-            for i in range(e):
-                wt[i] = ops.transpose_codes(wq3[i])
-            swt = sw.view(e, n // ops.BLOCK, k // ops.BLOCK).transpose(1, 2).contiguous()
+        goq = sgo = got = sgot = None
+        if need_dw:                              # one read of grad_out for both of its operand forms
+            out = ops.quantize_128x1_t_grouped(go, layout, e, with_1x128=need_dx)
+            (goq, sgo, got, sgot) = out if need_dx else (None, None) + out
+        elif need_dx:
             goq, sgo = ops.quantize_1x128(go, kmajor=True)
-            dx = ops.gemm_grouped_blockwise(goq, sgo, wt, swt, offs)
-            if last < dx.shape[0]:
-                dx[last:] = 0                                                    # rows that belong to no expert
+        if need_dx:
+            # dx_e = go_e . W_e: the grouped kernel on the stacked weight's transposed codes (128x128 blocks are
+            # symmetric, so W's scales serve with their two block strides swapped); rows of no expert are zeroed
+            dx = ops.gemm_grouped_blockwise_t(goq, sgo, wqt, sw, offs)
         if need_dw:
-            dw = torch.empty(ctx.w_shape, dtype=torch.bfloat16, device=go.device)
-            start = 0
-            for i, end in enumerate(ends):
-                if end > start:
-                    got, sgot = ops.quantize_128x1_t_rows(go[start:end])
-                    xt, sxt = ops.quantize_128x1_t_rows(x[start:end])
-                    ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=dw[i])
-                else:
-                    dw[i].zero_()                                                # an expert without rows
-                start = max(start, end)
-        return dx, dw, None
+            dw = ops.gemm_grouped_wgrad(got, sgot, xt, sxt, layout, e, ctx.total_m)
+        return dx, dw, None, None, None, None, None
 
 
-def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
+def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Tensor, *,
+                       weight_fp8: Optional[Fp8Weight] = None) -> torch.Tensor:
     """MoE grouped linear: rows of input[total_m, K] are sorted by expert, offs[E] are the inclusive int32
     prefix sums of rows per expert (a count may be 0), weight[E, N, K] -> bf16 [total_m, N]; rows past offs[-1]
-    are left uninitialised, as torch's grouped matmul leaves them.  Differentiable in input and weight
-    (blockwise recipe); backward reads offs on the host once."""
+    are left uninitialised, as torch's grouped matmul leaves them (their input gradient is zero).  Differentiable in
+    input and weight (blockwise recipe); neither forward nor backward reads offs on the host.  ``weight_fp8`` is the
+    weight's FP8 form made earlier by `quantize_grouped_weight` (e.g. once per optimizer step)."""
     if input.dim() != 2 or weight.dim() != 3 or input.shape[1] != weight.shape[2]:
         raise ValueError("input must be [total_m, K] and weight [E, N, K]")
     if input.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("input and weight must be bfloat16")
-    return _Fp8GroupedLinear.apply(input, weight, offs)
+    if offs.numel() != weight.shape[0]:
+        raise ValueError(f"offs must have {weight.shape[0]} entries")
+    if weight_fp8 is not None:
+        if tuple(weight_fp8.codes.shape) != tuple(weight.shape) or weight_fp8.scale_inv.dim() != 3 or weight_fp8.pow2:
+            raise ValueError("weight_fp8 must be the blockwise form of this weight (quantize_grouped_weight)")
+        return _Fp8GroupedLinear.apply(input, weight, offs, weight_fp8.codes, weight_fp8.scale_inv, weight_fp8.codes_t,
+                                       torch.is_grad_enabled())
+    return _Fp8GroupedLinear.apply(input, weight, offs, None, None, None, torch.is_grad_enabled())
 
 
 class _Fp8SwiGLUDown(torch.autograd.Function):

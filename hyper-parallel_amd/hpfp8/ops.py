@@ -512,3 +512,106 @@ def gemm_grouped_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, s
     _lib.call("hpfp8_gemm_grouped_blockwise_pow2" if pow2_scales else "hpfp8_gemm_grouped_blockwise", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b), _ptr(sb),
               _ptr(offs), e, total_m, n, k, _ptr(out), n, _out_code(out_dtype), _stream())
     return out
+
+
+def gemm_grouped_blockwise_t(a: torch.Tensor, sa: torch.Tensor, b_t: torch.Tensor, sb: torch.Tensor, offs: torch.Tensor,
+                             out_dtype: torch.dtype = torch.bfloat16, pow2_scales: bool = False,
+                             zero_unrouted: bool = True) -> torch.Tensor:
+    """The input gradient of the grouped linear: rows of a[total_m, N] (grad_out codes, 1x128 along N) sorted by
+    expert, b_t[K, E * N] the transposed codes of the stacked weight [E * N, K] (what
+    ``quantize_128x128(w.view(E * N, K), with_transpose=True)`` or ``transpose_codes`` gives; any row stride),
+    sb[E, N/128, K/128] the weight's block scales -> c[total_m, K]: rows of expert e = a_e . W_e.  With
+    ``zero_unrouted`` the rows past offs[-1] are set to zero (on the device, no host read of offs)."""
+    a = _check_codes_2d(a, "a")
+    b_t = _check_codes_2d(b_t, "b_t")
+    sa = _check_f32(sa, "sa")
+    sb = _check_f32(sb, "sb")
+    _check_offs(offs)
+    total_m, n = a.shape
+    e = offs.numel()
+    k = b_t.shape[0]
+    if sb.dim() != 3 or e == 0 or b_t.shape[1] != e * n or tuple(sb.shape) != (e, n // BLOCK, k // BLOCK) or not sb.is_contiguous():
+        raise ValueError(f"b_t must be [K, E * N] = [{k}, {e * n}] and sb contiguous [E, N/128, K/128]")
+    if k % BLOCK or n % BLOCK or n == 0:
+        raise ValueError(f"K={k} and N={n} must be multiples of 128, N positive")
+    if tuple(sa.shape) != (total_m, n // BLOCK):
+        raise ValueError(f"sa must be [{total_m}, {n // BLOCK}]")
+    out = torch.empty((total_m, k), dtype=out_dtype, device=a.device)
+    # the GEMM behind it: rows of b = K, contraction = N; expert e's operand starts N bytes after its predecessor's
+    _lib.call("hpfp8_gemm_grouped_blockwise_strided", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b_t), _ld(b_t),
+              n, _ptr(sb), sb.stride(0), 1, k // BLOCK, _ptr(offs), e, total_m, k, n, _ptr(out), k, _out_code(out_dtype),
+              int(pow2_scales), _stream())
+    if zero_unrouted and out_dtype == torch.bfloat16:
+        _lib.call("hpfp8_grouped_zero_unrouted_rows_bf16", _ptr(out), k, _ptr(offs), e, total_m, k, _stream())
+    elif zero_unrouted:
+        raise ValueError("zero_unrouted is implemented for bfloat16 output")
+    return out
+
+
+def grouped_padded_rows(experts: int, total_m: int) -> int:
+    """Columns of the padded token axis the grouped wgrad operands live on: (total_m // 128 + experts) * 128."""
+    return (total_m // BLOCK + experts) * BLOCK
+
+
+def grouped_layout(offs: torch.Tensor, total_m: int) -> torch.Tensor:
+    """The device-side table (int32) that places every expert's 128-token blocks on the padded token axis, made
+    from offs[E] (inclusive prefix sums of rows per expert) without a host read: per expert {first row, rows, first
+    padded block, blocks}, the experts ordered by block count, the number of blocks in use, each block's owner."""
+    _check_offs(offs)
+    e = offs.numel()
+    words = 5 * e + 1 + (total_m // BLOCK + e)
+    layout = torch.empty((words,), dtype=torch.int32, device=offs.device)
+    _lib.call("hpfp8_grouped_layout", _ptr(offs), e, total_m, _ptr(layout), _stream())
+    return layout
+
+
+def quantize_128x1_t_grouped(x: torch.Tensor, layout: torch.Tensor, experts: int, with_1x128: bool = False):
+    """The wgrad operand of x[total_m, K] (rows sorted by expert) for the grouped weight gradient: transposed 128x1
+    codes on the padded token axis of ``layout`` -- (codes_t[K, P], scale_inv_t[K, P/128]) with P =
+    ``grouped_padded_rows``, every expert's groups counted from its own first row, its last group filled up with
+    zero codes; blocks beyond those in use are left uninitialised.  With ``with_1x128`` also the 1x128 form of the
+    same read, (codes[total_m, K], scale_inv[total_m, K/128]) first; rows that belong to no expert stay
+    uninitialised there."""
+    x = _check_bf16(x, "x")
+    if x.dim() != 2 or x.shape[1] % BLOCK:
+        raise ValueError("x must be [total_m, K] with K a multiple of 128")
+    _check_device(layout, "layout")
+    total_m, k = x.shape
+    if layout.dtype != torch.int32 or layout.numel() != 5 * experts + 1 + (total_m // BLOCK + experts) or not layout.is_contiguous():
+        raise ValueError("layout does not belong to this expert count and row count")
+    p = grouped_padded_rows(experts, total_m)
+    qt = _empty_codes_t(k, p, x.device)
+    st_inv = torch.empty((p // BLOCK, k), dtype=torch.float32, device=x.device)
+    q = s_inv = None
+    if with_1x128:
+        q = torch.empty((total_m, k), dtype=FP8, device=x.device)
+        s_inv = torch.empty((k // BLOCK, total_m), dtype=torch.float32, device=x.device)
+    _lib.call("hpfp8_quantize_128x1_t_grouped_bf16", _ptr(x), total_m, k, _ptr(layout), experts, _ptr(qt), _ld(qt),
+              _ptr(st_inv), _ptr(q), _ptr(s_inv), _stream())
+    if with_1x128:
+        return q, s_inv.t(), qt, st_inv.t()
+    return qt, st_inv.t()
+
+
+def gemm_grouped_wgrad(got: torch.Tensor, sgot: torch.Tensor, xt: torch.Tensor, sxt: torch.Tensor, layout: torch.Tensor,
+                       experts: int, total_m: int, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """dW[E, N, K]: dW[e] = grad_out_e^T . x_e over expert e's own tokens.  got[N, P] / xt[K, P] and their scales
+    [N, P/128] / [K, P/128] are what ``quantize_128x1_t_grouped`` returns for grad_out and x with the same layout."""
+    got = _check_codes_2d(got, "got")
+    xt = _check_codes_2d(xt, "xt")
+    sgot = _check_f32(sgot, "sgot")
+    sxt = _check_f32(sxt, "sxt")
+    _check_device(layout, "layout")
+    p = grouped_padded_rows(experts, total_m)
+    n, k = got.shape[0], xt.shape[0]
+    if got.shape[1] != p or xt.shape[1] != p or n % BLOCK or k % BLOCK:
+        raise ValueError(f"operands must be [N, {p}] and [K, {p}] with N and K multiples of 128")
+    for name, s_, rows in (("sgot", sgot, n), ("sxt", sxt, k)):
+        if tuple(s_.shape) != (rows, p // BLOCK) or s_.stride(0) != 1 or (p > BLOCK and s_.stride(1) != rows):
+            raise ValueError(f"{name} must be the block-major [{rows}, {p // BLOCK}] scales the grouped quantizer returns")
+    if layout.dtype != torch.int32 or layout.numel() != 5 * experts + 1 + (total_m // BLOCK + experts):
+        raise ValueError("layout does not belong to this expert count and row count")
+    out = torch.empty((experts, n, k), dtype=out_dtype, device=got.device)
+    _lib.call("hpfp8_gemm_grouped_wgrad", _ptr(got), _ld(got), _ptr(sgot), _ptr(xt), _ld(xt), _ptr(sxt), _ptr(layout),
+              experts, total_m, n, k, _ptr(out), _out_code(out_dtype), _stream())
+    return out

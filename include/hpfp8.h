@@ -67,10 +67,11 @@ int hpfp8_amax_bf16(const void* x, int64_t n, float* amax_out, hpfp8_stream_t st
 int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void* q, float* scale,
                                float* scale_inv, hpfp8_stream_t stream);
 
-/* amax followed by cast: amax (fp32[1], required) is written then consumed.  Up to 4 Mi elements this is one
- * pass over x (3 bytes per element): the grid keeps x in registers and agrees on the maximum through the amax
- * word itself, whose lower half serves as its counter while the kernel runs; larger tensors take the two passes
- * above.  Either way amax holds max |x| as a clean fp32 when the call's kernels have finished. */
+/* amax followed by cast: amax (fp32[1], required) is written then consumed.  Up to 4 Mi elements, and when
+ * scale_inv is asked for, this is one pass over x (3 bytes per element): the grid keeps x in registers and agrees
+ * on the maximum through the amax word, using the scale_inv word as its arrival count until the value is stored
+ * there; larger tensors take the two passes above.  Either way amax holds max |x| as a clean fp32 and scale_inv
+ * its value when the call's kernels have finished. */
 int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
                                    float* scale_inv, hpfp8_stream_t stream);
 
@@ -301,6 +302,62 @@ int hpfp8_gemm_grouped_blockwise_pow2(const void* a, int64_t lda, const float* s
                                       int64_t sa_stride_k, const void* b, const float* sb, const int32_t* offs,
                                       int experts, int64_t total_m, int64_t N, int64_t K, void* c, int64_t ldc,
                                       int out_type, hpfp8_stream_t stream);
+
+/* hpfp8_gemm_grouped_blockwise[_pow2] with the experts' b matrices and scales addressed through strides: expert e's
+ * b[N, K] starts b_stride_e bytes after expert e - 1's and has row stride ldb;
+ *   sb(e, n, kb) = sb[e * sb_stride_e + (n / 128) * sb_stride_n + kb * sb_stride_k].
+ * This is the input gradient of the grouped linear (the dgrad of the same autograd the plain form stands for):
+ * with W^T held as the transposed codes [K_w, experts * N_w] that hpfp8_quantize_128x128_bf16 writes for the stacked
+ * weight [experts * N_w, K_w] (row stride ld_t), expert e's operand is b + e * N_w with ldb = ld_t, and the
+ * weight's scales [experts, N_w / 128, K_w / 128] serve with their two block strides swapped. */
+int hpfp8_gemm_grouped_blockwise_strided(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m,
+                                         int64_t sa_stride_k, const void* b, int64_t ldb, int64_t b_stride_e,
+                                         const float* sb, int64_t sb_stride_e, int64_t sb_stride_n, int64_t sb_stride_k,
+                                         const int32_t* offs, int experts, int64_t total_m, int64_t N, int64_t K,
+                                         void* c, int64_t ldc, int out_type, int pow2, hpfp8_stream_t stream);
+
+/* ---- MoE grouped weight gradient ----------------------------------------------------------------
+ * dW[e] = grad_out_e^T . x_e for every expert e, the contraction running over that expert's own rows
+ * [offs[e-1], offs[e]) -- the wgrad of the autograd that hpfp8_gemm_grouped_blockwise stands in for
+ * (hyper_parallel/core/shard/_op_dispatch.py:277-283; no grouped counterpart in the reference).  Nothing in this
+ * group of calls reads offs on the host, so a grouped backward can be captured in a HIP graph.
+ *
+ * The 128x1 scaling groups of the two operands run along the tokens and restart at each expert's first row.  The
+ * operands therefore live on a padded token axis of hpfp8_grouped_padded_rows(experts, total_m) =
+ * (total_m / 128 + experts) * 128 columns: expert e owns max(1, ceil(rows_e / 128)) blocks of 128, the rest of its
+ * last block (an empty expert's whole block) holding zero codes.
+ *
+ *   hpfp8_grouped_layout       offs[experts] (int32, device; read clamped like the grouped GEMM reads it) ->
+ *                              layout, hpfp8_grouped_layout_words(experts, total_m) int32 words on the device:
+ *                              per expert {first row, rows, first padded block, blocks}, the experts ordered by
+ *                              block count, the blocks in use, and the owner of every padded block.
+ *   hpfp8_quantize_128x1_t_grouped_bf16
+ *                              x[total_m, k] bf16 -> q_t[k, padded] (row stride ld_t bytes >= padded, multiple of 16)
+ *                              and scale_inv_t[padded / 128, k] (block-major), expert e's 128-row groups counted
+ *                              from its own first row; per expert the same codes and scales as
+ *                              hpfp8_quantize_128x1_t_kmajor_bf16 on that expert's rows filled up with zero rows.
+ *                              Padded blocks beyond those in use are left untouched.  With q != NULL also the 1x128
+ *                              form of the rows that belong to an expert: q[total_m, k], scale_inv[k / 128, total_m]
+ *                              (k-block-major), as hpfp8_quantize_1x128_kmajor_bf16 writes them.
+ *   hpfp8_gemm_grouped_wgrad   a = grad_out^T codes [N, padded] (row stride lda), sa [padded / 128, N];
+ *                              b = x^T codes [K, padded] (row stride ldb), sb [padded / 128, K]; both scale arrays
+ *                              contiguous and 16-byte aligned -> c[experts, N, K] contiguous, bf16 or fp32; an
+ *                              expert without rows gets zeros.  Per expert the result of hpfp8_gemm_blockwise with
+ *                              sb_gran = 1 on that expert's blocks.
+ *   hpfp8_grouped_zero_unrouted_rows_bf16
+ *                              out[total_m, cols] (row stride ld elements): rows from the last offset on := 0, the rows
+ *                              of an input gradient that belong to no expert. */
+int64_t hpfp8_grouped_padded_rows(int experts, int64_t total_m);
+int64_t hpfp8_grouped_layout_words(int experts, int64_t total_m);
+int hpfp8_grouped_layout(const int32_t* offs, int experts, int64_t total_m, int32_t* layout, hpfp8_stream_t stream);
+int hpfp8_quantize_128x1_t_grouped_bf16(const void* x, int64_t total_m, int64_t k, const int32_t* layout, int experts,
+                                        void* q_t, int64_t ld_t, float* scale_inv_t, void* q, float* scale_inv,
+                                        hpfp8_stream_t stream);
+int hpfp8_gemm_grouped_wgrad(const void* a, int64_t lda, const float* sa, const void* b, int64_t ldb, const float* sb,
+                             const int32_t* layout, int experts, int64_t total_m, int64_t N, int64_t K, void* c,
+                             int out_type, hpfp8_stream_t stream);
+int hpfp8_grouped_zero_unrouted_rows_bf16(void* out, int64_t ld, const int32_t* offs, int experts, int64_t total_m,
+                                          int64_t cols, hpfp8_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -55,6 +55,14 @@ How each function is pinned (tests/test_oracle_pins.py)
   gemm_*                    : torch._scaled_mm on CPU for per-tensor scales (library routine);
       exact integer-valued inputs with unit scales reduce to an exact integer matmul; the
       grouped variant equals a loop of dense calls; float64 dequant matmul bounds the rest.
+  dequantize_1x128_accumulate, dequantize_per_tensor_f32 : torch's float8 decode and a scalar loop in torch's fp32
+      arithmetic; the association of the two multiplications is pinned by a case where the other one differs.
+  swiglu_backward           : torch's float64 autograd of the same graph and closed-form points; its docstring
+      states the tolerance contract the device kernel is held to (it uses hardware approximations).
+  grouped_layout, quantize_128x1_t_grouped, gemm_grouped_wgrad : hand-computed block tables for ragged, empty and
+      malformed offsets; every expert's piece equals quantize_1x128 of that expert's zero-padded rows transposed;
+      the weight gradient equals the float64 product of the dequantized per-expert operands and is unchanged by
+      the zero padding.
 No function here is "parity unpinned" in the mathematical sense; what IS unpinned is parity
 with the reference, because the reference has no FP8 code to compare with.
 """
@@ -74,6 +82,7 @@ __all__ = [
     "dequantize_128x128", "quantize_bucket", "dequantize_bucket",
     "gemm_per_tensor", "gemm_blockwise", "gemm_rowwise_both", "gemm_grouped_blockwise",
     "gemm_dequant_f64", "dequantize_per_tensor_f32", "swiglu_backward",
+    "grouped_layout", "quantize_128x1_t_grouped", "gemm_grouped_wgrad",
 ]
 
 
@@ -459,6 +468,58 @@ def gemm_grouped_blockwise(a, sa_inv, b, sb_inv, offs):
         if end > start:
             out[start:end], _ = gemm_blockwise(a[start:end], sa_inv[start:end], b[e], sb_inv[e])
         start = end
+    return out, f32_to_bf16_bits(out)
+
+
+def grouped_layout(offs, total_m: int):
+    """Where every expert's 128-token blocks lie on the padded token axis of the grouped weight gradient:
+    ([(first row, rows, first block, blocks) per expert], blocks in use).  offs are inclusive prefix sums of rows per
+    expert, read clamped to [previous end, total_m] as the grouped GEMM reads them; an expert owns
+    max(1, ceil(rows / 128)) blocks (an empty expert one block of zeros, which adds nothing to any sum).  The axis is
+    allocated with (total_m // 128 + E) blocks, which always suffices."""
+    table, prev, blk = [], 0, 0
+    for off in np.asarray(offs).reshape(-1):
+        end = min(max(int(off), prev), int(total_m))
+        rows = end - prev
+        nb = -(-rows // BLOCK) if rows > 0 else 1
+        table.append((prev, rows, blk, nb))
+        blk += nb
+        prev = end
+    return table, blk
+
+
+def quantize_128x1_t_grouped(x_bits: np.ndarray, offs):
+    """The wgrad operand of the MoE grouped linear: x[total_m, K] (rows sorted by expert) -> codes_t[K, P],
+    scale_t / scale_inv_t[K, P/128] on the padded token axis (P = (total_m // 128 + E) * 128): expert e's rows,
+    filled up with zero rows to whole blocks of 128, quantized like `quantize_128x1_t`, at that expert's blocks.
+    Blocks no expert owns are returned as zeros (the device leaves them untouched)."""
+    x_bits = np.asarray(x_bits, dtype=np.uint16)
+    total_m, k = x_bits.shape
+    table, _ = grouped_layout(offs, total_m)
+    p = (total_m // BLOCK + len(table)) * BLOCK
+    codes_t = np.zeros((k, p), np.uint8)
+    scale_t = np.zeros((k, p // BLOCK), np.float32)
+    scale_inv_t = np.zeros((k, p // BLOCK), np.float32)
+    for start, rows, b0, nb in table:
+        padded = np.zeros((nb * BLOCK, k), np.uint16)
+        padded[:rows] = x_bits[start:start + rows]
+        c, s_, si = quantize_128x1_t(padded)
+        codes_t[:, b0 * BLOCK:(b0 + nb) * BLOCK] = c
+        scale_t[:, b0:b0 + nb] = s_
+        scale_inv_t[:, b0:b0 + nb] = si
+    return codes_t, scale_t, scale_inv_t
+
+
+def gemm_grouped_wgrad(got, sgot_inv, xt, sxt_inv, offs, total_m: int):
+    """dW[E, N, K]: dW[e] = go_e^T . x_e, the contraction over expert e's own blocks of the padded token axis;
+    got[N, P], xt[K, P] codes with scales [N, P/128], [K, P/128] (`quantize_128x1_t_grouped` of grad_out and x).
+    Per expert this is `gemm_rowwise_both` on that expert's columns.  Returns (fp32, bf16 bits)."""
+    table, _ = grouped_layout(offs, total_m)
+    n, k = got.shape[0], xt.shape[0]
+    out = np.zeros((len(table), n, k), np.float32)
+    for e, (_, _, b0, nb) in enumerate(table):
+        cols = slice(b0 * BLOCK, (b0 + nb) * BLOCK)
+        out[e], _ = gemm_rowwise_both(got[:, cols], sgot_inv[:, b0:b0 + nb], xt[:, cols], sxt_inv[:, b0:b0 + nb])
     return out, f32_to_bf16_bits(out)
 
 

@@ -700,3 +700,29 @@ def test_grouped_linear_backward(gpu):
     w1 = w.detach().clone().requires_grad_(True)
     hpfp8.fp8_grouped_linear(x.detach(), w1, offs).backward(go)
     assert torch.equal(w1.grad, gw)
+
+
+def test_grouped_linear_prequantized_weight_and_inference(gpu):
+    """`weight_fp8` for the grouped linear gives the same outputs and gradients bit for bit; under no_grad nothing is
+    prepared for a backward."""
+    import hpfp8
+    counts = torch.tensor([130, 0, 300, 70])
+    offs = counts.cumsum(0).to(torch.int32).to(gpu)
+    x = U.randn_bf16((512, 256), 31).to(gpu).requires_grad_(True)
+    w = U.randn_bf16((4, 384, 256), 32, 0.05).to(gpu).requires_grad_(True)
+    go = U.randn_bf16((512, 384), 33, 1e-2).to(gpu)
+    y0 = hpfp8.fp8_grouped_linear(x, w, offs)
+    y0.backward(go)
+    gx, gw = x.grad.clone(), w.grad.clone()
+    x.grad = w.grad = None
+    for with_t in (True, False):
+        f8 = hpfp8.quantize_grouped_weight(w.detach(), with_transpose=with_t)
+        y1 = hpfp8.fp8_grouped_linear(x, w, offs, weight_fp8=f8)
+        y1.backward(go)
+        assert torch.equal(y1[:500], y0[:500]) and torch.equal(x.grad, gx) and torch.equal(w.grad, gw)
+        x.grad = w.grad = None
+    with torch.no_grad():
+        y2 = hpfp8.fp8_grouped_linear(x, w, offs)
+    assert torch.equal(y2[:500], y0.detach()[:500]) and not y2.requires_grad
+    with pytest.raises(ValueError):
+        hpfp8.fp8_grouped_linear(x, w, offs[:3])

@@ -566,3 +566,59 @@ def test_swiglu_backward_against_float64_autograd():
     assert [float(v) for v in dh[0, :3]] == [0.5, 0.5, 1.0] and abs(float(dh[0, 3])) < 1e-14
     # d up at those points: dact * bf16(silu): silu(0) = 0, silu(40) = 40, silu(-40) = -0 (to bf16)
     assert [float(v) for v in dh[0, inter:inter + 3]] == [0.0, 0.0, 10.0] and abs(float(dh[0, inter + 3])) < 1e-14
+
+
+def test_grouped_layout_and_grouped_transposed_quantizer():
+    """The padded token axis of the grouped weight gradient: block tables worked out by hand (ragged counts, empty
+    experts, a malformed offset table read clamped), and every expert's piece of the grouped transposed quantizer
+    equal to the row-wise 1x128 quantizer applied to that expert's zero-padded rows, transposed."""
+    table, used = O.grouped_layout([130, 130, 430, 500], 512)
+    assert table == [(0, 130, 0, 2), (130, 0, 2, 1), (130, 300, 3, 3), (430, 70, 6, 1)] and used == 7
+    table, used = O.grouped_layout([128, 100, 9999], 300)                 # decreasing, then beyond the row count
+    assert table == [(0, 128, 0, 1), (128, 0, 1, 1), (128, 172, 2, 2)] and used == 4
+    assert O.grouped_layout([0, 0], 0) == ([(0, 0, 0, 1), (0, 0, 1, 1)], 2)
+    for offs, total in (([130, 130, 430, 500], 512), ([0, 7, 7, 263], 263)):
+        x = U.randn_bf16((total, 256), 77, 1.0, 0.002, 40.0)
+        xb = U.bits(x)
+        qt, st, sit = O.quantize_128x1_t_grouped(xb, offs)
+        e_cnt = len(offs)
+        assert qt.shape == (256, (total // 128 + e_cnt) * 128) and sit.shape == (256, total // 128 + e_cnt)
+        table, used = O.grouped_layout(offs, total)
+        assert used <= total // 128 + e_cnt
+        for start, rows, b0, nb in table:
+            padded = np.zeros((nb * 128, 256), np.uint16)
+            padded[:rows] = xb[start:start + rows]
+            c, s_, si = O.quantize_1x128(np.ascontiguousarray(padded.T))   # [K, nb * 128] with scales [K, nb]
+            assert np.array_equal(qt[:, b0 * 128:(b0 + nb) * 128], c)
+            assert np.array_equal(st[:, b0:b0 + nb].view(np.uint32), s_.view(np.uint32))
+            assert np.array_equal(sit[:, b0:b0 + nb].view(np.uint32), si.view(np.uint32))
+            assert not qt[:, b0 * 128 + rows:(b0 + nb) * 128].any()       # the fill is zero codes
+        assert not qt[:, used * 128:].any()
+
+
+def test_grouped_wgrad_against_float64_per_expert():
+    """`gemm_grouped_wgrad`: every expert's weight gradient equals the float64 product of that expert's dequantized
+    operands (so the zero fill adds nothing and no expert sees another's rows), an empty expert gets exact zeros,
+    and moving an expert's rows elsewhere in the batch does not change its result."""
+    offs, total, n, k = [130, 130, 430, 500], 512, 128, 256
+    go = U.randn_bf16((total, n), 81, 1e-2)
+    x = U.randn_bf16((total, k), 82, 1.0)
+    got, _, sgot = O.quantize_128x1_t_grouped(U.bits(go), offs)
+    xt, _, sxt = O.quantize_128x1_t_grouped(U.bits(x), offs)
+    dw, dw_bits = O.gemm_grouped_wgrad(got, sgot, xt, sxt, offs, total)
+    assert dw.shape == (4, n, k) and not dw[1].any()
+    table, _ = O.grouped_layout(offs, total)
+    for e, (start, rows, b0, nb) in enumerate(table):
+        cols = slice(b0 * 128, (b0 + nb) * 128)
+        ref = O.gemm_dequant_f64(got[:, cols], sgot[:, b0:b0 + nb], xt[:, cols], sxt[:, b0:b0 + nb])
+        assert np.linalg.norm(dw[e] - ref) <= 1e-6 * max(np.linalg.norm(ref), 1e-30)
+        if rows:
+            exact = go[start:start + rows].double().numpy().T @ x[start:start + rows].double().numpy()
+            assert np.linalg.norm(dw[e] - exact) / np.linalg.norm(exact) < 0.06
+    assert np.array_equal(dw_bits, O.f32_to_bf16_bits(dw))
+    # expert 2's 300 rows placed first in another batch: same gradient for it, bit for bit
+    perm = np.r_[130:430, 0:130, 430:512]
+    got2, _, sgot2 = O.quantize_128x1_t_grouped(U.bits(go)[perm], [300, 430, 430, 500])
+    xt2, _, sxt2 = O.quantize_128x1_t_grouped(U.bits(x)[perm], [300, 430, 430, 500])
+    dw2, _ = O.gemm_grouped_wgrad(got2, sgot2, xt2, sxt2, [300, 430, 430, 500], total)
+    assert np.array_equal(dw2[0].view(np.uint32), dw[2].view(np.uint32)) and np.array_equal(dw2[1].view(np.uint32), dw[0].view(np.uint32))
