@@ -11,7 +11,9 @@ on preallocated buffers.  One JSON line is printed:
     quantize   = the HBM-bound kernels alone, GB/s of algorithmic bytes, same timing method
     cpu_baseline = the CPU oracle's C restatement on a bounded sample of the same workload
 
-Usage: python bench.py [--gpus 1] [--steps 50] [--warmup 50] [--all] [--no-cpu-baseline]
+    other_configs = the kernels of configurations 1, 3, 4 and 5, each with its own roofline fraction
+
+Usage: python bench.py [--gpus 1] [--steps 50] [--warmup 50] [--all] [--headline-only] [--no-cpu-baseline]
 """
 import argparse
 import json
@@ -27,10 +29,40 @@ for p in (ROOT, os.path.join(ROOT, "hyper-parallel_amd")):
 M, N, K = 4096, 36864, 7168
 PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
-# Bytes per GEMM launch that crossed the L2 <-> memory-fabric boundary, from two rocprofv3 --pmc runs
-# (FETCH_SIZE x 1.9992 calibration + WRITE_SIZE, profiles/bench_cfg2_gemm_blockwise_and_quantizers.md):
-# 1,582,999 KiB fetched + 294,946 KiB written.  Algorithmic operand + output bytes are 582,591 KiB.
-GEMM_TRAFFIC_BYTES = (1582999 + 294946) * 1024   # FETCH_SIZE x 1.9992 + WRITE_SIZE of the GEMM, KiB per dispatch
+# Bytes per GEMM launch that crossed the L2 <-> memory-fabric boundary come from two rocprofv3 --pmc runs
+# (FETCH_SIZE, calibrated on a copy of known size, + WRITE_SIZE) whose summary is kept in PROFILE; the summary
+# names the tiling of the kernel it was measured on, and the figure is only reported while csrc/gemm.hip still has
+# that tiling (otherwise `traffic` is null until the counters are collected again).
+PROFILE = os.path.join(ROOT, "profiles", "bench_cfg2_gemm_blockwise_and_quantizers.md")
+GEMM_SOURCE = os.path.join(ROOT, "hyper-parallel_amd", "csrc", "gemm.hip")
+
+
+def gemm_tiling_signature(path=GEMM_SOURCE):
+    """The constants of csrc/gemm.hip that decide how often operand panels are fetched from beyond L2."""
+    import re
+    text = open(path).read()
+    sig = []
+    for name in ("BM", "BN", "BK", "kRectTiles", "kXcds"):
+        m = re.search(r"\b%s\s*=\s*(\d+)" % name, text)
+        sig.append(f"{name}={m.group(1) if m else '?'}")
+    m = re.search(r"b_stages\(int mode\)\s*\{[^}]*\?\s*(\d+)\s*:\s*(\d+)", text)
+    sig.append(f"b_stages={m.group(2) if m else '?'}")
+    return " ".join(sig)
+
+
+def gemm_traffic_bytes():
+    """(bytes per launch, or None when the profile is absent or was taken on another tiling; the reason)."""
+    import re
+    try:
+        text = open(PROFILE).read()
+    except OSError:
+        return None, "no profile summary"
+    m = re.search(r"traffic_bytes=(\d+)\s+gemm_tiling=\"([^\"]*)\"", text)
+    if not m:
+        return None, "profile summary has no traffic line"
+    if m.group(2) != gemm_tiling_signature():
+        return None, f"profile was taken on tiling [{m.group(2)}], the kernel now has [{gemm_tiling_signature()}]"
+    return int(m.group(1)), "profiles/" + os.path.basename(PROFILE)
 
 
 def make_inputs(dev):
@@ -115,28 +147,131 @@ def _time(fn, iters=30, warm=40):
     return s0.elapsed_time(s1) / iters
 
 
-def other_configs(dev):
-    """Kernel times of configurations 1, 3, 4 and 5 (HIP events, back-to-back launches)."""
+def _tf(flops, ms):
+    return {"ms": ms, "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_FP8_TFLOPS}
+
+
+def _gb(nbytes, ms):
+    return {"ms": ms, "GB/s": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+
+
+def zipf_counts(experts, total, seed=0):
+    """Rows per expert of configuration 4: multinomial over p_e ~ rank^-1.1 (seeded permutation of the experts), the
+    two least popular experts emptied into the most popular one."""
+    import torch
+    gc = torch.Generator(device="cpu").manual_seed(seed)
+    perm = torch.randperm(experts, generator=gc)
+    pz = (torch.arange(1, experts + 1, dtype=torch.float64) ** -1.1)[perm]
+    pz = pz / pz.sum()
+    counts = torch.multinomial(pz, total, replacement=True, generator=gc).bincount(minlength=experts)
+    order = torch.argsort(pz)
+    for z in order[:2]:
+        counts[order[-1]] += counts[z]
+        counts[z] = 0
+    return counts
+
+
+def other_configs_compact(dev):
+    """The other four benchmark configurations, each kernel with its own roofline fraction (HIP events around
+    back-to-back launches after a warm-up): cfg 1 per-tensor quantize + GEMM, cfg 3 backward GEMMs and transposed
+    requantizers, cfg 4 MoE grouped GEMMs and the whole grouped layer, cfg 5 bucket quantize / dequantize."""
     import torch
     import hpfp8
+    from hpfp8 import ops
     res = {}
     g = torch.Generator(device=dev).manual_seed(0)
-
-    def tf(flops, ms):
-        return {"ms": ms, "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_FP8_TFLOPS}
-
-    def gb(nbytes, ms):
-        return {"ms": ms, "GB/s": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
-
-    # cfg 1: per-tensor linear 2048x1024x1024
+    # cfg 1: per-tensor linear 2048 x 1024 x 1024 (launch-bound: times include the launches)
     x = torch.randn((2048, 1024), generator=g, device=dev).to(torch.bfloat16)
     w = (torch.randn((1024, 1024), generator=g, device=dev) * 0.02).to(torch.bfloat16)
     xq, _, sx = hpfp8.quantize_per_tensor(x)
     wq, _, sw = hpfp8.quantize_per_tensor(w)
-    res["cfg1_per_tensor"] = {
-        "quantize_x": gb(x.numel() * 5, _time(lambda: hpfp8.quantize_per_tensor(x))),
-        "gemm": tf(2.0 * 2048 * 1024 * 1024, _time(lambda: hpfp8.gemm_per_tensor(xq, sx, wq, sw))),
+    t_q = _time(lambda: hpfp8.quantize_per_tensor(x), iters=100)
+    t_g = _time(lambda: hpfp8.gemm_per_tensor(xq, sx, wq, sw), iters=100)
+    res["cfg1_per_tensor"] = {"quantize_x": _gb(x.numel() * 3, t_q), "gemm": _tf(2.0 * 2048 * 1024 * 1024, t_g),
+                              "quantize_x_plus_gemm_us": (t_q + t_g) * 1e3}
+    del x, w, xq, wq
+    # cfg 3: o_proj backward, M = 4096 tokens, W[7168, 16384]
+    m, n, k = 4096, 7168, 16384
+    x = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
+    u = torch.rand((m, n), generator=g, device=dev) - 0.5
+    go = (-(2 ** -0.5) * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999)) * 1e-3).to(torch.bfloat16)
+    w = (torch.randn((n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16)
+    wq, sw, wqt = hpfp8.quantize_128x128(w, with_transpose=True)
+    goq, sgo = hpfp8.quantize_1x128(go, kmajor=True)
+    got, sgot = hpfp8.quantize_128x1_t(go, kmajor=True)
+    xt, sxt = hpfp8.quantize_128x1_t(x, kmajor=True)
+    fl = 2.0 * m * n * k
+    res["cfg3_backward"] = {
+        "dgrad_gemm": _tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq, sgo, wqt, sw.t()))),
+        "wgrad_gemm": _tf(fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1))),
+        "requant_t_x": _gb(m * k * 3 + k * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(x, kmajor=True))),
+        "requant_t_grad_out": _gb(m * n * 3 + n * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(go, kmajor=True))),
+        "quantize_grad_out": _gb(m * n * 3 + m * (n // 128) * 4, _time(lambda: hpfp8.quantize_1x128(go, kmajor=True))),
+        "quantize_both_forms_x": _gb(m * k * 4 + 2 * m * (k // 128) * 4,
+                                     _time(lambda: hpfp8.quantize_1x128_and_128x1_t(x, kmajor=True))),
+        "quantize_both_forms_grad_out": _gb(m * n * 4 + 2 * m * (n // 128) * 4,
+                                            _time(lambda: hpfp8.quantize_1x128_and_128x1_t(go, kmajor=True))),
+        "quantize_w_with_transpose": _gb(n * k * 4 + (n // 128) * (k // 128) * 4,
+                                         _time(lambda: hpfp8.quantize_128x128(w, with_transpose=True))),
     }
+    del x, go, w, wq, wqt, goq, got, xt, u
+    torch.cuda.empty_cache()
+    # cfg 4: MoE grouped, 32 experts, 131072 routed rows, Zipf(1.1) counts, two empty experts
+    e, n, k, total = 32, 4096, 7168, 131072
+    counts = zipf_counts(e, total)
+    offs = counts.cumsum(0).to(torch.int32).to(dev)
+    xg4 = torch.randn((total, k), generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+    wg4 = (torch.randn((e, n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16).requires_grad_(True)
+    go4 = (torch.randn((total, n), generator=g, device=dev) * 1e-3).to(torch.bfloat16)
+    layout = ops.grouped_layout(offs, total)
+    xq, sx, xt, sxt = ops.quantize_128x1_t_grouped(xg4.detach(), layout, e, with_1x128=True)
+    goq, sgo, got, sgot = ops.quantize_128x1_t_grouped(go4, layout, e, with_1x128=True)
+    f8 = hpfp8.quantize_grouped_weight(wg4.detach())
+    fl = 2.0 * total * n * k
+    r4 = {"rows": total, "experts": e, "min_rows": int(counts.min()), "max_rows": int(counts.max())}
+    r4["forward_gemm"] = _tf(fl, _time(lambda: ops.gemm_grouped_blockwise(xq, sx, f8.codes, f8.scale_inv, offs), iters=5, warm=5))
+    r4["dgrad_gemm"] = _tf(fl, _time(lambda: ops.gemm_grouped_blockwise_t(goq, sgo, f8.codes_t, f8.scale_inv, offs), iters=5, warm=3))
+    r4["wgrad_gemm"] = _tf(fl, _time(lambda: ops.gemm_grouped_wgrad(got, sgot, xt, sxt, layout, e, total), iters=5, warm=3))
+    r4["quantize_both_forms_x_grouped"] = _gb(total * k * 4 + 2 * total * (k // 128) * 4, _time(
+        lambda: ops.quantize_128x1_t_grouped(xg4.detach(), layout, e, with_1x128=True), iters=5, warm=3))
+    del xq, xt, goq, got
+    torch.cuda.empty_cache()
+
+    def grouped_train(f8w):
+        hpfp8.fp8_grouped_linear(xg4, wg4, offs, weight_fp8=f8w).backward(go4)
+        xg4.grad = wg4.grad = None
+    r4["layer_forward_backward"] = dict(_tf(3 * fl, _time(lambda: grouped_train(f8), iters=3, warm=3)),
+                                        note="weights' FP8 form made once per optimizer step (weight_fp8); quantizers of x "
+                                             "and grad_out, grouped forward, dgrad and wgrad GEMMs; no host read of offs")
+    r4["layer_forward_backward_weights_quantized_inside"] = _tf(3 * fl, _time(lambda: grouped_train(None), iters=3, warm=2))
+    res["cfg4_moe_grouped"] = r4
+    del xg4, wg4, go4, f8
+    torch.cuda.empty_cache()
+    # cfg 5: gradient bucket, 2^29 elements
+    nel = 1 << 29
+    flat = torch.randn(nel, generator=g, device=dev) * 1e-4
+    idx = torch.randint(0, nel, (nel // 10000,), generator=g, device=dev)
+    flat[idx] *= 1e3
+    flat = flat.to(torch.bfloat16)
+    nbytes = nel * 3 + (nel // 128) * 4
+    codes, si = hpfp8.quantize_bucket(flat)
+    res["cfg5_bucket"] = {"quantize": _gb(nbytes, _time(lambda: hpfp8.quantize_bucket(flat))),
+                          "dequantize": _gb(nbytes, _time(lambda: hpfp8.dequantize_bucket(codes, si)))}
+    del flat, codes, si
+    torch.cuda.empty_cache()
+    return res
+
+
+def more_measurements(dev):
+    """--all: what the layers around the benchmarked kernels cost (the dense-MLP block with its fused SwiGLU, a
+    training step of cfg 2's layer), the optional power-of-two recipe, the vendor library's per-tensor GEMM for
+    orientation, and the fused bucket pack / unpack."""
+    import torch
+    import torch.nn.functional as F
+    import hpfp8
+    res = {}
+    g = torch.Generator(device=dev).manual_seed(0)
+    tf, gb = _tf, _gb
     # the step after cfg 2 in the MLP: SwiGLU of the gate/up output fused with the 1x128 quantization for the
     # down projection (read 2 x 2 bytes, write 1 byte + scales per activation)
     hgu = torch.randn((4096, 36864), generator=g, device=dev).to(torch.bfloat16)
@@ -147,7 +282,6 @@ def other_configs(dev):
     res["cfg2_swiglu_quantize_both_forms_fast"] = gb(4096 * 18432 * 6 + 2 * 4096 * (18432 // 128) * 4, _time(
         lambda: hpfp8.ops.swiglu_quantize_1x128_and_128x1_t(hgu, fast=True)))
     # the whole dense-MLP block forward: gate/up linear, SwiGLU, down linear [7168 <- 18432]
-    import torch.nn.functional as F
     wd_bf16 = (torch.randn((7168, 18432), device=dev) * 0.006).to(torch.bfloat16)
     wgu_bf16 = (torch.randn((36864, 7168), device=dev) * 0.006).to(torch.bfloat16)
     x_mlp = torch.randn((4096, 7168), device=dev).to(torch.bfloat16)
@@ -178,11 +312,9 @@ def other_configs(dev):
     res["cfg2_mlp_block_forward_backward"] = {"fp8_ms": t_fp8, "TFLOP/s": 3 * mlp_flop / t_fp8 / 1e9, "torch_bf16_ms": t_bf16}
     dact = torch.randn((4096, 18432), device=dev).to(torch.bfloat16)
     res["cfg2_swiglu_backward"] = gb(4096 * 18432 * 10, _time(lambda: hpfp8.ops.swiglu_backward(hgu, dact)))
-    del wd_bf16, wgu_bf16, x_mlp, gu_q, dn_q, xg_, wgu_p, wd_p, go_mlp, dact
-    del hgu
+    del wd_bf16, wgu_bf16, x_mlp, gu_q, dn_q, xg_, wgu_p, wd_p, go_mlp, dact, hgu
     # cfg 2 as a training step of the module: forward + backward through fp8_linear (the weight's FP8 form
     # made beforehand, as Fp8Linear's cache does), beside torch's bf16 F.linear on the same tensors
-    import torch.nn.functional as F
     xt_ = torch.randn((4096, 7168), generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
     wt_ = (torch.randn((36864, 7168), generator=g, device=dev) * 0.006).to(torch.bfloat16).requires_grad_(True)
     got_ = (torch.randn((4096, 36864), generator=g, device=dev) * 1e-3).to(torch.bfloat16)
@@ -219,104 +351,47 @@ def other_configs(dev):
     except Exception as err:          # (absent or differently named in another torch build)
         orient["vendor_scaled_mm"] = f"unavailable: {type(err).__name__}"
     res["cfg2_shape_per_tensor_for_orientation"] = orient
-    del wf2_, xq2_, sx2_
-    del xt_, wt_, got_, wf_
+    del wf2_, xq2_, sx2_, xt_, wt_, got_, wf_
     torch.cuda.empty_cache()
-    # cfg 3: o_proj backward
+    # cfg 3 under the optional recipe, and its weight gradient added onto an fp32 main gradient
     m, n, k = 4096, 7168, 16384
     x = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
-    u = torch.rand((m, n), generator=g, device=dev) - 0.5
-    go = (-(2 ** -0.5) * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999)) * 1e-3).to(torch.bfloat16)
+    go = (torch.randn((m, n), generator=g, device=dev) * 1e-3).to(torch.bfloat16)
     w = (torch.randn((n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16)
-    wq, sw, wqt = hpfp8.quantize_128x128(w, with_transpose=True)
-    goq, sgo = hpfp8.quantize_1x128(go, kmajor=True)
-    got, sgot = hpfp8.quantize_128x1_t(go, kmajor=True)
-    xt, sxt = hpfp8.quantize_128x1_t(x, kmajor=True)
     fl = 2.0 * m * n * k
-    res["cfg3_backward"] = {
-        "quantize_w_with_transpose": gb(n * k * 4 + (n // 128) * (k // 128) * 4,
-                                        _time(lambda: hpfp8.quantize_128x128(w, with_transpose=True))),
-        "requant_t_x": gb(m * k * 3 + k * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(x, kmajor=True))),
-        "requant_t_grad_out": gb(m * n * 3 + n * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(go, kmajor=True))),
-        "quantize_grad_out": gb(m * n * 3 + m * (n // 128) * 4, _time(lambda: hpfp8.quantize_1x128(go, kmajor=True))),
-        # both operand forms from one read (what fp8_linear uses in training): 2 + 1 + 1 bytes per element + scales
-        "quantize_both_forms_x": gb(m * k * 4 + 2 * m * (k // 128) * 4,
-                                    _time(lambda: hpfp8.quantize_1x128_and_128x1_t(x, kmajor=True))),
-        "quantize_both_forms_grad_out": gb(m * n * 4 + 2 * m * (n // 128) * 4,
-                                           _time(lambda: hpfp8.quantize_1x128_and_128x1_t(go, kmajor=True))),
-        "dgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq, sgo, wqt, sw.t()))),
-        "wgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1))),
-    }
     got2, sgot2 = hpfp8.quantize_128x1_t(go, kmajor=True, pow2=True)
     xt2, sxt2 = hpfp8.quantize_128x1_t(x, kmajor=True, pow2=True)
     goq2, sgo2 = hpfp8.quantize_1x128(go, kmajor=True, pow2=True)
     wq2, sw2, wqt2 = hpfp8.quantize_128x128(w, with_transpose=True, pow2=True)
-    res.setdefault("recipe_blockwise_pow2", {}).update({
+    res["recipe_blockwise_pow2"].update({
         "cfg3_dgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq2, sgo2, wqt2, sw2.t(), pow2_scales=True))),
         "cfg3_wgrad_gemm": tf(fl, _time(lambda: hpfp8.gemm_blockwise(got2, sgot2, xt2, sxt2, sb_gran=1, pow2_scales=True))),
     })
     del got2, xt2, goq2, wq2, wqt2
-    # the same weight gradient added onto an fp32 main gradient (apply_grad_on_fp32_main_grad)
+    got, sgot = hpfp8.quantize_128x1_t(go, kmajor=True)
+    xt, sxt = hpfp8.quantize_128x1_t(x, kmajor=True)
     main_grad = torch.zeros((n, k), dtype=torch.float32, device=dev)
-    res["cfg3_backward"]["wgrad_gemm_into_fp32_main_grad"] = tf(
+    res["cfg3_wgrad_gemm_into_fp32_main_grad"] = tf(
         fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=main_grad, accumulate=True)))
-    del main_grad
-    del x, go, w, wq, wqt, goq, got, xt
+    del main_grad, x, go, w, got, xt
     torch.cuda.empty_cache()
-    # cfg 4: MoE grouped, 32 experts, 131072 routed rows, Zipf(1.1) counts, two empty experts
+    # cfg 4's grouped GEMM under the optional recipe (timing only: the same codes under power-of-two scales)
     e, n, k, total = 32, 4096, 7168, 131072
-    gc = torch.Generator(device="cpu").manual_seed(0)
-    perm = torch.randperm(e, generator=gc)
-    pz = (torch.arange(1, e + 1, dtype=torch.float64) ** -1.1)[perm]
-    pz = pz / pz.sum()
-    counts = torch.multinomial(pz, total, replacement=True, generator=gc).bincount(minlength=e)
-    order = torch.argsort(pz)
-    for z in order[:2]:
-        counts[order[-1]] += counts[z]
-        counts[z] = 0
-    offs = counts.cumsum(0).to(torch.int32).to(dev)
-    x = torch.randn((total, k), generator=g, device=dev).to(torch.bfloat16)
-    w = (torch.randn((e * n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16)
-    xq, sx = hpfp8.quantize_1x128(x, kmajor=True)
-    wq, sw = hpfp8.quantize_128x128(w)
-    del x, w
-    ms = _time(lambda: hpfp8.gemm_grouped_blockwise(xq, sx, wq.view(e, n, k), sw.view(e, n // 128, k // 128), offs), iters=5)
-    res["cfg4_moe_grouped"] = dict(tf(2.0 * total * n * k, ms), rows=total, experts=e,
-                                   min_rows=int(counts.min()), max_rows=int(counts.max()))
-    sx2 = torch.exp2(torch.ceil(torch.log2(sx)))           # (timing only: the same codes under power-of-two scales)
+    offs = zipf_counts(e, total).cumsum(0).to(torch.int32).to(dev)
+    xq, sx = hpfp8.quantize_1x128(torch.randn((total, k), generator=g, device=dev).to(torch.bfloat16), kmajor=True)
+    wq, sw = hpfp8.quantize_128x128((torch.randn((e * n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16))
+    sx2 = torch.exp2(torch.ceil(torch.log2(sx)))
     sw2 = torch.exp2(torch.ceil(torch.log2(sw)))
     ms2 = _time(lambda: hpfp8.gemm_grouped_blockwise(xq, sx2, wq.view(e, n, k), sw2.view(e, n // 128, k // 128), offs,
                                                      pow2_scales=True), iters=5)
-    res.setdefault("recipe_blockwise_pow2", {})["cfg4_moe_grouped_gemm"] = tf(2.0 * total * n * k, ms2)
+    res["recipe_blockwise_pow2"]["cfg4_moe_grouped_gemm"] = tf(2.0 * total * n * k, ms2)
     del xq, sx, wq, sw, sx2, sw2
     torch.cuda.empty_cache()
-    # the same layer in training: forward + backward of the grouped linear (weights quantized inside the step)
-    xg4 = torch.randn((total, k), generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
-    wg4 = (torch.randn((e, n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16).requires_grad_(True)
-    go4 = (torch.randn((total, n), generator=g, device=dev) * 1e-3).to(torch.bfloat16)
-
-    def grouped_train():
-        hpfp8.fp8_grouped_linear(xg4, wg4, offs).backward(go4)
-        xg4.grad = wg4.grad = None
-    ms3 = _time(grouped_train, iters=3, warm=3)
-    res["cfg4_moe_grouped_forward_backward"] = dict(tf(3 * 2.0 * total * n * k, ms3),
-                                                    note="quantizers (weights included), grouped forward, dgrad and wgrad GEMMs: no host read of offs")
-    del xg4, wg4, go4
-    torch.cuda.empty_cache()
-    # cfg 5: gradient bucket, 2^29 elements
+    # cfg 5's 2^29 elements as 72 separate gradients (64 of 2048x4096 minus 8 of them split into bias-sized
+    # pieces): packing fused with the quantization, and the cast back fused with the unpacking
     nel = 1 << 29
-    flat = torch.randn(nel, generator=g, device=dev) * 1e-4
-    idx = torch.randint(0, nel, (nel // 10000,), generator=g, device=dev)
-    flat[idx] *= 1e3
-    flat = flat.to(torch.bfloat16)
+    flat = (torch.randn(nel, generator=g, device=dev) * 1e-4).to(torch.bfloat16)
     nbytes = nel * 3 + (nel // 128) * 4
-    codes, si = hpfp8.quantize_bucket(flat)
-    res["cfg5_bucket"] = {
-        "quantize": gb(nbytes, _time(lambda: hpfp8.quantize_bucket(flat))),
-        "dequantize": gb(nbytes, _time(lambda: hpfp8.dequantize_bucket(codes, si))),
-    }
-    # the same 2^29 elements as 72 separate gradients (64 of 2048x4096 minus 8 of them split into
-    # bias-sized pieces): packing fused with the quantization, and the cast back fused with the unpacking
     sizes = [2048 * 4096] * 56 + [7168] * 8 + [2048 * 4096 * 8 - 7168 * 8]
     views, pos = [], 0
     for n_ in sizes:
@@ -325,9 +400,8 @@ def other_configs(dev):
     bucket = hpfp8.Fp8GradBucket(sizes, shard_size=1, grad_scale=0.5)
     q2, si2 = bucket.pack(views)
     outs = [torch.empty(n_, dtype=torch.bfloat16, device=dev) for n_ in sizes]
-    res["cfg5_bucket"]["pack_and_quantize_72_grads"] = gb(nbytes, _time(lambda: bucket.pack(views)))
-    res["cfg5_bucket"]["dequantize_and_unpack_72_grads"] = gb(
-        nbytes, _time(lambda: bucket.unpack(q2[0], si2[0], outs)))
+    res["cfg5_bucket_fused"] = {"pack_and_quantize_72_grads": gb(nbytes, _time(lambda: bucket.pack(views))),
+                                "dequantize_and_unpack_72_grads": gb(nbytes, _time(lambda: bucket.unpack(q2[0], si2[0], outs)))}
     return res
 
 
@@ -338,7 +412,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)   # the clock needs ~25 ms of load to leave its idle state
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--all", action="store_true",
-                    help="also time the kernels of the other benchmark configurations (adds an 'other_configs' key)")
+                    help="also time the layers around the kernels, the optional recipe and the fused bucket forms "
+                         "(adds a 'more' key; the other four configurations are always under 'other_configs')")
+    ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU's share of the path; this build has no multi-GPU leg "
@@ -435,6 +511,7 @@ def main():
     err = float((y[:256, :256].double() - ref).norm() / ref.norm())
     assert err < 1e-2, f"GEMM output is wrong: rel Frobenius error {err}"
 
+    traffic, traffic_source = gemm_traffic_bytes()
     out = {
         "metric": "FP8 linear TFLOP/s & % FP8 MFMA peak; quantize GB/s & % HBM peak (1 GPU)",
         "value": flops / (ms_step * 1e-3) / 1e12,
@@ -462,7 +539,8 @@ def main():
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_tflops / PEAK_FP8_TFLOPS,
-            "traffic": GEMM_TRAFFIC_BYTES,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
             "ms": t_g,
         },
         "quantize": {
@@ -478,10 +556,12 @@ def main():
         import numpy as np
         host_copies = (x[:2048].cpu().view(torch.int16).numpy().view(np.uint16),
                        w.cpu().view(torch.int16).numpy().view(np.uint16))
+    del x, w, xq, wq, y
+    torch.cuda.empty_cache()
+    if not args.headline_only:
+        out["other_configs"] = other_configs_compact(dev)
     if args.all:
-        del x, w, xq, wq, y
-        torch.cuda.empty_cache()
-        out["other_configs"] = other_configs(dev)
+        out["more"] = more_measurements(dev)
     if host_copies is not None:
         out["cpu_baseline"] = cpu_baseline(*host_copies)
     print(json.dumps(out))

@@ -27,4 +27,18 @@ def test_cpu_baseline_fields_on_a_small_sample(monkeypatch):
     out = bench.cpu_baseline(x, w, target_seconds=0.5)
     assert out["kind"] == "port" and out["unit"] == "TFLOP/s" and out["cores"] >= 1 and out["value"] > 0
     assert isinstance(out["sample"], str) and out["aten_linear_bf16_on_cpu"]["value"] > 0
-    assert bench.GEMM_TRAFFIC_BYTES > 2 * (4096 * 7168 + 36864 * 7168)      # at least the operands once
+
+
+def test_reported_gemm_traffic_belongs_to_the_kernel_as_it_is_now():
+    """`roofline.traffic` comes from a rocprofv3 counter run kept under profiles/; the summary names the tiling it
+    was measured on, and bench.py reports the figure only while csrc/gemm.hip still has that tiling.  This test
+    fails when the tiling constants were changed without collecting the counters again (bench.py itself then
+    reports null rather than a stale number)."""
+    sys.path.insert(0, ROOT)
+    import bench
+    sig = bench.gemm_tiling_signature()
+    assert "?" not in sig, sig
+    traffic, source = bench.gemm_traffic_bytes()
+    assert traffic is not None, source
+    assert traffic > 2 * (4096 * 7168 + 36864 * 7168)      # at least the operands once
+    assert source.startswith("profiles/")
