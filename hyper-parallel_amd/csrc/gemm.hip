@@ -73,6 +73,12 @@ struct GemmParams {
   int M, N, K;            // M = total rows of a; grouped along the contraction: K = the padded token axis
   int tiles;              // dense: number of output tiles; grouped along the contraction: per expert
   int accumulate;
+  // SwiGLU epilogue: b = W_gate_up codes [2 * inter, K] (gate rows first), N = 2 * inter; c = codes of the
+  // activation [M, inter] (row stride ldc bytes), q_scale (may be null) / q_scale_inv its 1x128 scales, [inter / 128, M]
+  int inter;
+  int pow2_out;
+  float* q_scale;
+  float* q_scale_inv;
 };
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -167,8 +173,14 @@ __device__ __forceinline__ int expert_end(int off, int prev, int total_rows) {
 
 // SA4: the activation scales have unit stride over rows (the k-block-major layout), so a lane's four
 // of them are one 16-byte load.
-template <int MODE, int GROUPED, bool OUT_F32, bool ACC, bool SA4>
+// EPI: 0 = c is the GEMM's result; 1 / 2 = the gate/up projection of a SwiGLU MLP with the activation and its
+// 1x128 quantization as the epilogue (1: exactly specified silu, 2: hardware exponential and reciprocal).  A tile's
+// 256 columns are then the 128 gate columns and the 128 up columns of one scaling group of the activation: the b
+// tile's upper 128 rows come from `inter` rows further down, the two waves that share 64 rows hold gate and up.
+template <int MODE, int GROUPED, bool OUT_F32, bool ACC, bool SA4, int EPI = 0>
 __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) {
+  static_assert(EPI == 0 || ((MODE == kScaleBlock || MODE == kScalePow2) && GROUPED == kDense && !OUT_F32 && !ACC),
+                "SwiGLU epilogue: dense block-scaled forward");
   static_assert(!ACC || (OUT_F32 && MODE != kScaleTensor), "accumulating onto c: fp32 output, sums that start from c's values");
   static_assert(GROUPED != kGroupedK || (!ACC && (MODE == kScaleRow || MODE == kScalePow2Row)),
                 "grouped along the contraction: the wgrad form");
@@ -302,8 +314,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
                                              0x00020000);
   };
   auto rsrc_b_of = [&](const TileInfo& ti) {
-    const int rows = N - ti.n0 > 0 ? N - ti.n0 : 0;
-    const uint8_t* base = p.b + (GROUPED == kGroupedRows ? (int64_t)ti.expert * p.b_se : 0) + (int64_t)(rows ? ti.n0 : 0) * p.ldb;
+    // (SwiGLU epilogue: the tile's first b row is gate row n0 / 2; its up rows lie `inter` rows further down)
+    const int brow0 = EPI ? ti.n0 >> 1 : ti.n0;
+    const int rows = N - ti.n0 > 0 ? N - brow0 : 0;
+    const uint8_t* base = p.b + (GROUPED == kGroupedRows ? (int64_t)ti.expert * p.b_se : 0) + (int64_t)(rows ? brow0 : 0) * p.ldb;
     return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, span_bytes(rows, p.ldb), 0x00020000);
   };
   uint32_t a_off[4], b_off[4];
@@ -318,7 +332,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
     // rows of c.  (The b tile keeps its order.)
     const int ra = (r & ~63) + (r & 15) * 4 + ((r >> 4) & 3);
     a_off[i] = (uint32_t)ra * (uint32_t)p.lda + chunk * 16;
-    b_off[i] = (uint32_t)r * (uint32_t)p.ldb + chunk * 16;
+    b_off[i] = (uint32_t)(EPI && r >= 128 ? r - 128 + p.inter : r) * (uint32_t)p.ldb + chunk * 16;
   }
   // wgrad form: the 256 per-row scales of the b tile for one k-block are one more 1 KB transfer
   // (wave 0), possible because that scale array is k-block-major (unit stride over rows).
@@ -371,7 +385,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       // (SA4 does not clamp: words past the end of the array read as zero, and rows past M are never stored)
       sa_voff[j] = SA4 ? (uint32_t)r * 4u : (uint32_t)(r < p.M ? r : p.M - 1) * (uint32_t)((int)p.sa_sm * 4);
     }
-    int nblk_idx = (ti.n0 + wn * 128) >> 7;
+    int nblk_idx = EPI ? (ti.n0 >> 8) + wn * (p.inter >> 7) : (ti.n0 + wn * 128) >> 7;
     if (nblk_idx > (N >> 7) - 1) nblk_idx = (N >> 7) - 1;
     sb_soff = ((GROUPED == kGroupedRows ? ti.expert * (int)p.sb_se : 0) + nblk_idx * (int)p.sb_sn) * 4;
   };
@@ -767,7 +781,65 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
       }
     }
   };
-  if (cols_ok) {
+  if constexpr (EPI != 0) {
+    // SwiGLU epilogue.  Per pass j (16 of the wave's 64 rows) both waves of a pair write their bf16-rounded
+    // results -- gate from the wave with wn = 0, up from its neighbour -- into their staging slices as for a plain
+    // store; after a barrier each wave of the pair takes 8 of the 16 rows, reads gate and up of a row from the two
+    // slices (16 lanes x 8 columns: one scaling group of the activation), and computes, quantizes and stores
+    // the activation exactly as the stand-alone kernel does on a bf16 gate/up tensor.  A second barrier keeps the
+    // next pass's writes (and, after the last pass, the next tile's transfers) off slices still being read.
+    static_assert(kBStages == 3, "staging rows 0..15 of a wave are contiguous");
+    const uint8_t* gate_s = stg - wave * 4096 + (wave & ~1) * 4096;
+    const uint8_t* up_s = gate_s + 4096;
+    const uint32_t stg_we = (uint32_t)(uintptr_t)(lds_ptr_t)(stg + l16e * 256);   // this lane's staging row
+    const int gcol = n0 >> 1;                        // first activation column of the tile's scaling group
+    const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(reinterpret_cast<uint8_t*>(p.c) + (int64_t)row0 * p.ldc + gcol), 0,
+        rows_valid > 0 ? (int)(((int64_t)rows_valid - 1) * p.ldc + 128) : 0, 0x00020000);
+    const int64_t s_first = (int64_t)(n0 >> 8) * p.M + row0;
+    const __amdgpu_buffer_rsrc_t rsrc_si = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(p.q_scale_inv + s_first), 0, rows_valid > 0 ? rows_valid * 4 : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_sc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(p.q_scale ? p.q_scale + s_first : p.q_scale_inv), 0, p.q_scale && rows_valid > 0 ? rows_valid * 4 : 0,
+        0x00020000);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int ii = 0; ii < 8; ++ii) {
+        u32x2 o;
+        o[0] = pack_bf16x2(acc[ii][j][0], acc[ii][j][1]);
+        o[1] = pack_bf16x2(acc[ii][j][2], acc[ii][j][3]);
+        asm volatile("ds_write_b64 %0, %1" ::"v"(stg_we + (((ii * 2 + (ge >> 1)) ^ l16e) * 16) + (ge & 1) * 8), "v"(o)
+                     : "memory");
+        acc[ii][j] = zero;
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+      for (int it = 0; it < 2; ++it) {
+        const int srow = 8 * wn + 4 * it + ge;                   // staging row: tile row wm * 64 + 4 * srow + j
+        const int soff = srow * 256 + ((l16e ^ srow) * 16);
+        const v4i gv = *reinterpret_cast<const v4i*>(gate_s + soff);
+        const v4i uv = *reinterpret_cast<const v4i*>(up_s + soff);
+        uint4 a;
+        a.x = swiglu2<EPI == 2>((uint32_t)gv[0], (uint32_t)uv[0]);
+        a.y = swiglu2<EPI == 2>((uint32_t)gv[1], (uint32_t)uv[1]);
+        a.z = swiglu2<EPI == 2>((uint32_t)gv[2], (uint32_t)uv[2]);
+        a.w = swiglu2<EPI == 2>((uint32_t)gv[3], (uint32_t)uv[3]);
+        const uint32_t m = row16_max_u32(mag8(a));
+        float sc, sci;
+        scales_from_amax(__uint_as_float(m << 16), sc, sci, p.pow2_out);
+        const uint2 codes = cvt8<false>(a, sc);
+        const int trow = wm * 64 + 4 * srow + j;
+        u32x2 cw = {codes.x, codes.y};
+        __builtin_amdgcn_raw_buffer_store_b64(cw, rsrc_q, (uint32_t)trow * (uint32_t)p.ldc + l16e * 8, 0, 2);
+        if (l16e == 0) {
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sci), rsrc_si, trow * 4, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sc), rsrc_sc, trow * 4, 0, 0);
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+  } else if (cols_ok) {
     if (!p.bias) store_tile(std::false_type{});
     else store_tile(std::true_type{});
   } else {
@@ -921,6 +993,54 @@ int hpfp8_gemm_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64
                               int out_type, int accumulate, hpfp8_stream_t stream) {
   return gemm_blockwise_impl(a, lda, sa, sa_stride_m, sa_stride_k, b, ldb, sb, sb_stride_n, sb_stride_k, sb_gran, M, N, K,
                              bias, c, ldc, out_type, accumulate, true, stream);
+}
+
+int hpfp8_gemm_blockwise_swiglu_quantize(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m,
+                                         int64_t sa_stride_k, const void* b, int64_t ldb, const float* sb,
+                                         int64_t sb_stride_n, int64_t sb_stride_k, int64_t M, int64_t inter, int64_t K,
+                                         int fast, int pow2, int pow2_out, void* q, int64_t ldq, float* scale,
+                                         float* scale_inv, hpfp8_stream_t stream) {
+  const char* what = "gemm_blockwise_swiglu_quantize";
+  HPFP8_REQUIRE((fast == 0 || fast == 1) && (pow2 == 0 || pow2 == 1) && (pow2_out == 0 || pow2_out == 1), HPFP8_ERR_ARG,
+                "%s: fast, pow2 and pow2_out must be 0 or 1", what);
+  HPFP8_REQUIRE(inter >= 0 && inter % kBlock == 0 && inter < (1 << 29), HPFP8_ERR_SHAPE,
+                "%s: the activation's width %lld must be a multiple of 128", what, (long long)inter);
+  HPFP8_REQUIRE(ldq >= inter && ldq % 16 == 0, HPFP8_ERR_SHAPE, "%s: ldq=%lld must be a multiple of 16 and at least the width",
+                what, (long long)ldq);
+  // (the common checks see the gate/up matrix this call does not write, [M, 2 * inter]; the code matrix it does
+  // write is checked here: a tile's 256 rows are addressed with 32-bit byte offsets)
+  HPFP8_REQUIRE(BM * ldq < (int64_t)0x7FFFF000, HPFP8_ERR_SHAPE, "%s: the row stride of q must stay below 8 MiB", what);
+  int rc = check_common(what, a, lda, b, ldb, sa, sb, M, 2 * inter, K, nullptr, q, 2 * inter, HPFP8_OUT_F32, 0);
+  if (rc <= 0) return rc;
+  HPFP8_REQUIRE(scale_inv != nullptr, HPFP8_ERR_ARG, "%s: null scale_inv", what);
+  // the up rows of a b tile are addressed `inter` rows past its gate rows, inside one buffer resource
+  HPFP8_REQUIRE(2 * inter * ldb < (int64_t)0x7FFFF000, HPFP8_ERR_SHAPE, "%s: the weight's codes must span less than 2 GiB", what);
+  GemmParams p{};
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.sa = sa; p.sb = sb; p.lda = lda; p.ldb = ldb;
+  p.sa_sm = sa_stride_m; p.sa_sk = sa_stride_k; p.sb_sn = sb_stride_n; p.sb_sk = sb_stride_k;
+  rc = check_scale_span(what, M, K / BK, sa_stride_m, sa_stride_k, "sa");
+  if (rc <= 0) return rc;
+  rc = check_scale_span(what, 2 * inter / kBlock, K / BK, sb_stride_n, sb_stride_k, "sb");
+  if (rc <= 0) return rc;
+  p.sb_bytes = (int)(((2 * inter / kBlock - 1) * sb_stride_n + (K / BK - 1) * sb_stride_k + 1) * 4);
+  p.c = q; p.ldc = ldq;
+  p.M = (int)M; p.N = (int)(2 * inter); p.K = (int)K;
+  p.inter = (int)inter; p.pow2_out = pow2_out; p.q_scale = scale; p.q_scale_inv = scale_inv;
+  const int64_t tiles = ((M + BM - 1) / BM) * (inter / kBlock);
+  p.tiles = (int)tiles;
+  dim3 grid((unsigned)persistent_grid(tiles)), block(kGemmThreads);
+  hipStream_t st = (hipStream_t)stream;
+  const bool sa4 = sa_stride_m == 1;
+#define HPFP8_LAUNCH_EPI(MODE, SA4, EPI) gemm_kernel<MODE, kDense, false, false, SA4, EPI><<<grid, block, 0, st>>>(p)
+  if (pow2) {
+    if (sa4) { if (fast) HPFP8_LAUNCH_EPI(kScalePow2, true, 2); else HPFP8_LAUNCH_EPI(kScalePow2, true, 1); }
+    else { if (fast) HPFP8_LAUNCH_EPI(kScalePow2, false, 2); else HPFP8_LAUNCH_EPI(kScalePow2, false, 1); }
+  } else {
+    if (sa4) { if (fast) HPFP8_LAUNCH_EPI(kScaleBlock, true, 2); else HPFP8_LAUNCH_EPI(kScaleBlock, true, 1); }
+    else { if (fast) HPFP8_LAUNCH_EPI(kScaleBlock, false, 2); else HPFP8_LAUNCH_EPI(kScaleBlock, false, 1); }
+  }
+#undef HPFP8_LAUNCH_EPI
+  return check_launch(what);
 }
 
 int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,

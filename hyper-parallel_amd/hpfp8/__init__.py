@@ -8,7 +8,7 @@ _lib.load()
 
 from .ops import (amax, quantize_per_tensor, quantize_1x128, quantize_128x128, quantize_128x1_t,  # noqa: E402
                   quantize_1x128_and_128x1_t, transpose_codes, swiglu_quantize_1x128,
-                  dequantize_1x128, dequantize_1x128_accumulate, dequantize_128x128, dequantize_per_tensor, gemm_blockwise, gemm_per_tensor,
+                  dequantize_1x128, dequantize_1x128_accumulate, dequantize_128x128, dequantize_per_tensor, gemm_blockwise, gemm_blockwise_swiglu_quantize, gemm_per_tensor,
                   gemm_grouped_blockwise)
 from .linear import (fp8_linear, Fp8Linear, fp8_grouped_linear, fp8_swiglu_mlp, Fp8SwiGLUMLP, Fp8Weight,  # noqa: E402
                      quantize_weight, quantize_grouped_weight, invalidate_fp8_caches, attach_optimizer)
@@ -21,7 +21,7 @@ __all__ = [
     "amax", "quantize_per_tensor", "quantize_1x128", "quantize_128x128", "quantize_128x1_t",
     "quantize_1x128_and_128x1_t", "transpose_codes", "swiglu_quantize_1x128", "Fp8Weight", "quantize_weight", "fsdp", "checkpoint",
     "invalidate_fp8_caches", "attach_optimizer", "quantize_grouped_weight",
-    "dequantize_1x128", "dequantize_1x128_accumulate", "dequantize_128x128", "dequantize_per_tensor", "gemm_blockwise", "gemm_per_tensor",
+    "dequantize_1x128", "dequantize_1x128_accumulate", "dequantize_128x128", "dequantize_per_tensor", "gemm_blockwise", "gemm_blockwise_swiglu_quantize", "gemm_per_tensor",
     "gemm_grouped_blockwise", "fp8_linear", "Fp8Linear", "fp8_grouped_linear", "fp8_swiglu_mlp", "Fp8SwiGLUMLP",
     "quantize_bucket", "dequantize_bucket", "Fp8GradBucket",
 ]

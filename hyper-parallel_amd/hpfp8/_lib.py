@@ -50,6 +50,8 @@ SIGNATURES = {
                              _vp, _i64, _int, _int, _vp],
     "hpfp8_gemm_blockwise_pow2": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _int, _i64, _i64, _i64, _vp,
                                   _vp, _i64, _int, _int, _vp],
+    "hpfp8_gemm_blockwise_swiglu_quantize": [_vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _i64,
+                                             _int, _int, _int, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_gemm_per_tensor": [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _int, _vp],
     "hpfp8_gemm_grouped_blockwise": [_vp, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _i64,
                                      _int, _vp],

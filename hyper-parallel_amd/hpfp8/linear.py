@@ -572,8 +572,10 @@ def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True,
     with torch.no_grad():
         x2 = _flatten(input)
         xq, sx = ops.quantize_1x128(x2, kmajor=True, pow2=gu.pow2)
-        h = ops.gemm_blockwise(xq, sx, gu.codes, gu.scale_inv, pow2_scales=gu.pow2)
-        aq, sa = ops.swiglu_quantize_1x128(h, kmajor=True, pow2=dn.pow2, fast=fast)
+        # SwiGLU and the quantization of the down projection's input are the gate/up GEMM's epilogue: the gate/up
+        # output never exists in bf16
+        aq, sa = ops.gemm_blockwise_swiglu_quantize(xq, sx, gu.codes, gu.scale_inv, fast=fast, pow2_scales=gu.pow2,
+                                                    pow2_out=dn.pow2)
         y = ops.gemm_blockwise(aq, sa, dn.codes, dn.scale_inv, pow2_scales=dn.pow2)
     return y.reshape(input.shape[:-1] + (dn.codes.shape[0],))
 

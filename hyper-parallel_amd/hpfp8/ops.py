@@ -459,6 +459,36 @@ def gemm_blockwise(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch
     return out
 
 
+def gemm_blockwise_swiglu_quantize(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor, *,
+                                   fast: bool = False, pow2_scales: bool = False, pow2_out: bool = False,
+                                   want_scale: bool = False):
+    """The gate/up projection with SwiGLU and the 1x128 quantization of its result as the GEMM's epilogue.
+
+    a[M, K] codes with scales sa[M, K/128]; b = codes of W_gate_up [2I, K] (gate rows first) with 128x128 scales
+    sb[2I/128, K/128].  Returns (codes[M, I], scale_inv[M, I/128]) of act = silu(gate) * up -- bit for bit what
+    `gemm_blockwise` followed by `swiglu_quantize_1x128(kmajor=True)` returns -- without the bf16 gate/up tensor."""
+    a = _check_codes_2d(a, "a")
+    b = _check_codes_2d(b, "b")
+    sa = _check_f32(sa, "sa")
+    sb = _check_f32(sb, "sb")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"a {tuple(a.shape)} and b {tuple(b.shape)} must be 2-D with equal last dim")
+    m, k = a.shape
+    n = b.shape[0]
+    if k % BLOCK or n % (2 * BLOCK) or k == 0:
+        raise ValueError(f"K={k} must be a positive multiple of 128 and the weight's rows {n} a multiple of 256")
+    kb, inter = k // BLOCK, n // 2
+    if tuple(sa.shape) != (m, kb) or tuple(sb.shape) != (n // BLOCK, kb):
+        raise ValueError(f"sa must be [{m}, {kb}] and sb [{n // BLOCK}, {kb}]")
+    q = torch.empty((m, inter), dtype=FP8, device=a.device)
+    s_inv = torch.empty((inter // BLOCK, m), dtype=torch.float32, device=a.device)
+    s = torch.empty_like(s_inv) if want_scale else None
+    _lib.call("hpfp8_gemm_blockwise_swiglu_quantize", _ptr(a), _ld(a), _ptr(sa), sa.stride(0), sa.stride(1), _ptr(b),
+              _ld(b), _ptr(sb), sb.stride(0), sb.stride(1), m, inter, k, int(fast), int(pow2_scales), int(pow2_out),
+              _ptr(q), inter, _ptr(s), _ptr(s_inv), _stream())
+    return (q, s_inv.t(), s.t()) if want_scale else (q, s_inv.t())
+
+
 def gemm_per_tensor(a: torch.Tensor, sa_inv: torch.Tensor, b: torch.Tensor, sb_inv: torch.Tensor,
                     bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """c = (a . b^T) * (sa_inv * sb_inv) (+ bias); sa_inv / sb_inv are 0-dim (or 1-element) fp32."""

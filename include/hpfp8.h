@@ -280,6 +280,24 @@ int hpfp8_gemm_blockwise_pow2(const void* a, int64_t lda, const float* sa, int64
                               int sb_gran, int64_t M, int64_t N, int64_t K, const void* bias, void* c, int64_t ldc,
                               int out_type, int accumulate, hpfp8_stream_t stream);
 
+/* The gate/up projection of a SwiGLU MLP with the activation and the 1x128 quantization of the down projection's
+ * input as the GEMM's epilogue: no bf16 gate/up tensor is written or read (the eager graph this replaces is two
+ * aten::linear calls dispatched at hyper_parallel/core/shard/_op_dispatch.py:277-283 with F.silu(gate) * up
+ * between them).  a[M, K], sa as in hpfp8_gemm_blockwise; b = codes of W_gate_up [2 * inter, K] (gate rows
+ * [0, inter), up rows [inter, 2 * inter); must span less than 2 GiB) with 128x128 scales
+ * sb(n / 128, kb) = sb[(n / 128) * sb_stride_n + kb * sb_stride_k]; inter and K multiples of 128.
+ *   h = bf16(gate | up) as hpfp8_gemm_blockwise[_pow2] (pow2 = 0 / 1: which of the two, by the operands' scales)
+ *       would write it; act = bf16(bf16(silu(gate)) * up) as hpfp8_swiglu_quantize_1x128_bf16 (fast = 0) or
+ *       hpfp8_swiglu_quantize_1x128_fast_bf16 (fast = 1) defines it;
+ *   q[M, inter] (row stride ldq bytes, a multiple of 16), scale (may be NULL) and scale_inv [inter / 128, M]
+ *       (k-block-major): bit for bit what those two calls in a row give, with power-of-two scales when
+ *       pow2_out = 1. */
+int hpfp8_gemm_blockwise_swiglu_quantize(const void* a, int64_t lda, const float* sa, int64_t sa_stride_m,
+                                         int64_t sa_stride_k, const void* b, int64_t ldb, const float* sb,
+                                         int64_t sb_stride_n, int64_t sb_stride_k, int64_t M, int64_t inter, int64_t K,
+                                         int fast, int pow2, int pow2_out, void* q, int64_t ldq, float* scale,
+                                         float* scale_inv, hpfp8_stream_t stream);
+
 /* Per-tensor scales: c = (a . b^T) * (sa_inv[0] * sb_inv[0]) (+ bias), accumulation over the whole
  * K inside the matrix cores.  K a multiple of 128, N a multiple of 128. */
 int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,
