@@ -858,6 +858,198 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
 }
 
+// ---------------------------------------------------------------------------------------------
+// small problems: fewer 256 x 256 tiles than compute units
+// ---------------------------------------------------------------------------------------------
+// One 128 x 128 output tile per workgroup of 4 waves (2 x 2, wave tile 64 x 64), no persistence: four times as
+// many workgroups as the kernel above has tiles, each with a quarter of the matrix work per k-block.  Same
+// operand layout in LDS (global -> LDS transfers, swizzle, fragment reads), five stages of one a tile and one b
+// tile (16 KB each), transfers four k-blocks ahead, one barrier per k-block.  Same arithmetic in the same order as
+// the kernel above (one matrix instruction per 16 x 16 subtile and k-block; block form: acc += partial * (sa * sb)),
+// so the two give identical results.  Per-tensor and 128x128-block scale forms, dense, bf16 or fp32 output, bias.
+constexpr int kSmallThreads = 256;
+constexpr int kSmallTile = 128;
+constexpr int kSmallStageBytes = 2 * kSmallTile * BK;   // a tile + b tile
+constexpr int kSmallStages = 5;
+
+template <int MODE, bool OUT_F32>
+__global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmParams p) {
+  static_assert(MODE == kScaleTensor || MODE == kScaleBlock, "per-tensor or block scales");
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kSmallStages * kSmallStageBytes];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 1, wm = wave >> 1;
+  const int l16 = lane & 15, g = lane >> 4;
+  const int kblocks = p.K / BK;
+  const int tiles_n = p.N / kSmallTile;
+  const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+  const int row0 = tm * kSmallTile, n0 = tn * kSmallTile;
+  const int rows_valid = p.M - row0 < kSmallTile ? p.M - row0 : kSmallTile;
+
+  // transfers: as in gemm_kernel, a wave moves 8 rows x 128 B per instruction, four per operand tile and k-block;
+  // the resources start at the tile's first row and end with the tensor (rows past it read as zero); k-blocks
+  // past the end go through an empty resource and fetch nothing
+  auto span = [&](int64_t rows, int64_t ld) {
+    const int64_t bytes = rows > 0 ? (rows - 1) * ld + p.K : 0;
+    return (int)(bytes < (int64_t)0x7FFFF000 ? bytes : (int64_t)0x7FFFF000);
+  };
+  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc((void*)(p.a + (int64_t)row0 * p.lda), 0,
+                                                                      span(p.M - row0, p.lda), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc((void*)(p.b + (int64_t)n0 * p.ldb), 0,
+                                                                      span(p.N - n0, p.ldb), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_none = __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, 0, 0x00020000);
+  uint32_t a_off[4], b_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (wave * 4 + i) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ row_swizzle(r);
+    a_off[i] = (uint32_t)r * (uint32_t)p.lda + chunk * 16 - i * 1024;
+    b_off[i] = (uint32_t)r * (uint32_t)p.ldb + chunk * 16 - i * 1024;
+  }
+  auto issue_stage = [&](int kb, int stage) {
+    const bool ok = kb < kblocks;
+    const __amdgpu_buffer_rsrc_t ra = ok ? rs_a : rs_none, rb = ok ? rs_b : rs_none;
+    uint8_t* sa_base = lds + stage * kSmallStageBytes + wave * 4096;
+    uint8_t* sb_base = sa_base + kSmallTile * BK;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[0], kb * BK, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[1], kb * BK, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[2], kb * BK, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[3], kb * BK, 3072, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[0], kb * BK, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[1], kb * BK, 1024, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[2], kb * BK, 2048, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[3], kb * BK, 3072, 0);
+  };
+  const int pc0 = (2 * g) ^ row_swizzle(l16);
+  const int a_frag = (wm * 64 + l16) * BK, b_frag = kSmallTile * BK + (wn * 64 + l16) * BK;
+
+  // scales of the block form: this lane's four rows of a (clamped: rows past M are never stored), the tile's
+  // one 128-row block of b
+  const float* sa_row[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = row0 + wm * 64 + j * 16 + l16;
+    sa_row[j] = p.sa + (int64_t)(r < p.M ? r : p.M - 1) * p.sa_sm;
+  }
+  const float* sb_blk = p.sb + (int64_t)(n0 >> 7) * p.sb_sn;
+
+  const v4f zero = {0.f, 0.f, 0.f, 0.f};
+  v4f acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = zero;
+
+  // Transfers run four k-blocks ahead (five stages); the block form's scales are fetched three k-blocks ahead
+  // into a ring of registers, so that waiting for them never waits for a transfer that is not needed yet
+  // (vector-memory operations complete in order).  Issue order per iteration i: wait + barrier, scale loads of
+  // k-block i + 3, transfers of k-block i + 4.
+  float s_ring[4][5];
+  auto load_scales = [&](int kb, float raw[5]) {
+    if (MODE == kScaleBlock) {
+      const int kk = kb < kblocks ? kb : kblocks - 1;
+      raw[4] = sb_blk[(int64_t)kk * p.sb_sk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) raw[j] = sa_row[j][(int64_t)kk * p.sa_sk];
+    }
+  };
+  issue_stage(0, 0);
+  load_scales(0, s_ring[0]);
+  issue_stage(1, 1);
+  load_scales(1, s_ring[1]);
+  issue_stage(2, 2);
+  load_scales(2, s_ring[2]);
+  issue_stage(3, 3);
+  int st = 0, st_issue = 4;
+  // one k-block; Q = kb % 4 is the ring slot that holds its scales (static, so the ring needs no register moves:
+  // a move would have to wait for the load it moves)
+  auto k_block = [&](int kb, auto q_tag) {
+    constexpr int Q = decltype(q_tag)::value;
+    // all but the youngest transfers of three k-blocks (and, block form, the scale loads issued between them)
+    // have landed: this k-block's tiles of this wave; after the barrier everyone's, and everyone has left the
+    // stage that is refilled next
+    if (MODE == kScaleBlock) asm volatile("s_waitcnt vmcnt(34)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
+    load_scales(kb + 3, s_ring[(Q + 3) & 3]);
+    asm volatile("" ::: "memory");       // (keeps the scale loads ahead of the transfers, as the wait above counts them)
+    issue_stage(kb + 4, st_issue);
+    const uint8_t* base = lds + st * kSmallStageBytes;
+    st = st == kSmallStages - 1 ? 0 : st + 1;
+    st_issue = st_issue == kSmallStages - 1 ? 0 : st_issue + 1;
+    v8i xf[4], wf[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xf[j] = frag_read(base + a_frag + j * 16 * BK, pc0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wf[i] = frag_read(base + b_frag + i * 16 * BK, pc0);
+    if (MODE == kScaleTensor) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+    } else {
+      v4f part[4][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          part[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf[j], zero, 0, 0, 0, 0, 0, 0);
+      float s[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[j] = s_ring[Q][j] * s_ring[Q][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(part[i][j][r], s[j], acc[i][j][r]);
+    }
+  };
+  for (int kb = 0; kb < kblocks; kb += 4) {
+    k_block(kb, std::integral_constant<int, 0>{});
+    if (kb + 1 < kblocks) k_block(kb + 1, std::integral_constant<int, 1>{});
+    if (kb + 2 < kblocks) k_block(kb + 2, std::integral_constant<int, 2>{});
+    if (kb + 3 < kblocks) k_block(kb + 3, std::integral_constant<int, 3>{});
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // the transfers past the last k-block (they fetch nothing) still target this LDS
+
+  // store: a lane holds, per subtile, four consecutive columns of one row
+  float tensor_scale = 1.f;
+  if (MODE == kScaleTensor) tensor_scale = p.sa[0] * p.sb[0];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = wm * 64 + j * 16 + l16;
+    if (r >= rows_valid) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = n0 + wn * 64 + i * 16 + g * 4;
+      float v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v[q] = acc[i][j][q];
+        if (MODE == kScaleTensor) v[q] *= tensor_scale;
+      }
+      if (p.bias) {
+        const uint2 braw = *reinterpret_cast<const uint2*>(p.bias + col);
+        v[0] += bf16lo(braw.x); v[1] += bf16hi(braw.x); v[2] += bf16lo(braw.y); v[3] += bf16hi(braw.y);
+      }
+      const int64_t o = (int64_t)(row0 + r) * p.ldc + col;
+      if (OUT_F32) {
+        *reinterpret_cast<v4f*>(reinterpret_cast<float*>(p.c) + o) = v4f{v[0], v[1], v[2], v[3]};
+      } else {
+        u32x2 w2;
+        w2[0] = pack_bf16x2(v[0], v[1]);
+        w2[1] = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(p.c) + o) = w2;
+      }
+    }
+  }
+}
+
+// 0: the small-tile kernel serves problems with fewer 256 x 256 tiles than half the compute units (and more
+// 128 x 128 tiles than that); 1: never; 2: whenever its forms allow (test hook)
+static int g_small_gemm_mode = 0;
+
 // Workgroups to launch for `tiles` tiles: one per CU, a multiple of 8 (one share per XCD) unless
 // there are fewer than 8 tiles.
 static int persistent_grid(int64_t tiles) {
@@ -871,6 +1063,24 @@ static int persistent_grid(int64_t tiles) {
   int64_t g = tiles < cus ? tiles : cus;
   if (g >= kXcds) g -= g % kXcds;
   return (int)g;
+}
+
+static bool use_small_kernel(int64_t M, int64_t N) {
+  if (g_small_gemm_mode == 1) return false;
+  if (g_small_gemm_mode == 2) return true;
+  const int64_t big = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const int64_t small = ((M + kSmallTile - 1) / kSmallTile) * (N / kSmallTile);
+  const int cus = persistent_grid((int64_t)1 << 40);
+  return 2 * big < cus && small > big && small < (int64_t)0x7FFFFFFF;
+}
+
+template <int MODE>
+static int launch_small(const GemmParams& p, int out_type, hipStream_t stream) {
+  const int64_t tiles = (((int64_t)p.M + kSmallTile - 1) / kSmallTile) * (p.N / kSmallTile);
+  dim3 grid((unsigned)tiles), block(kSmallThreads);
+  if (out_type == HPFP8_OUT_F32) gemm_small_kernel<MODE, true><<<grid, block, 0, stream>>>(p);
+  else gemm_small_kernel<MODE, false><<<grid, block, 0, stream>>>(p);
+  return check_launch("gemm (small tiles)");
 }
 
 template <int MODE, int GROUPED, bool SA4>
@@ -965,6 +1175,7 @@ static int gemm_blockwise_impl(const void* a, int64_t lda, const float* sa, int6
   p.tiles = (int)tiles;
   if (sb_gran == 128) {
     if (pow2) return launch<kScalePow2, kDense>(p, out_type, tiles, (hipStream_t)stream);
+    if (!accumulate && use_small_kernel(M, N)) return launch_small<kScaleBlock>(p, out_type, (hipStream_t)stream);
     return launch<kScaleBlock, kDense>(p, out_type, tiles, (hipStream_t)stream);
   }
   // per-row b scales travel to LDS as one contiguous 1 KB piece per k-block
@@ -1043,6 +1254,8 @@ int hpfp8_gemm_blockwise_swiglu_quantize(const void* a, int64_t lda, const float
   return check_launch(what);
 }
 
+void hpfp8_debug_set_small_gemm(int mode) { g_small_gemm_mode = mode == 1 || mode == 2 ? mode : 0; }
+
 int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,
                           const float* sb_inv, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
                           int64_t ldc, int out_type, hpfp8_stream_t stream) {
@@ -1054,6 +1267,7 @@ int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const
   p.M = (int)M; p.N = (int)N; p.K = (int)K;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   p.tiles = (int)tiles;
+  if (use_small_kernel(M, N)) return launch_small<kScaleTensor>(p, out_type, (hipStream_t)stream);
   return launch<kScaleTensor, kDense>(p, out_type, tiles, (hipStream_t)stream);
 }
 

@@ -100,6 +100,8 @@ def load():
         fn.restype = _i64
     lib.hpfp8_debug_set_spin_limit.argtypes = [ctypes.c_uint32]
     lib.hpfp8_debug_set_spin_limit.restype = None
+    lib.hpfp8_debug_set_small_gemm.argtypes = [_int]
+    lib.hpfp8_debug_set_small_gemm.restype = None
     lib.hpfp8_last_error.argtypes = []
     lib.hpfp8_last_error.restype = ctypes.c_char_p
     _lib = lib

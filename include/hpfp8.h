@@ -304,6 +304,12 @@ int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const
                           const float* sb_inv, int64_t M, int64_t N, int64_t K, const void* bias, void* c,
                           int64_t ldc, int out_type, hpfp8_stream_t stream);
 
+/* Small problems.  When a problem has fewer 256 x 256 output tiles than half the GPU's compute units (cfg-1-sized
+ * layers, decode-sized M), hpfp8_gemm_per_tensor and hpfp8_gemm_blockwise (sb_gran = 128, no accumulate) run a
+ * kernel with 128 x 128 tiles instead, four times as many workgroups; same arithmetic in the same order, identical
+ * results.  Test hook, not part of the path: mode 0 = that rule (default), 1 = never, 2 = whenever the form allows. */
+void hpfp8_debug_set_small_gemm(int mode);
+
 /* MoE grouped form (one rank's local experts; no counterpart in the reference, whose expert
  * parallelism is unimplemented): rows of a[total_m, K] (row stride lda) are sorted by expert; offs[e] (int32,
  * device) is the inclusive prefix sum of per-expert row counts, a count may be 0, rows past

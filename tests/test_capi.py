@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} is declared in include/hpfp8.h but not exported"
-    bound = set(_lib.SIGNATURES) | set(_lib.SIZE_FUNCTIONS) | {"hpfp8_last_error", "hpfp8_debug_set_spin_limit"}
+    bound = set(_lib.SIGNATURES) | set(_lib.SIZE_FUNCTIONS) | {"hpfp8_last_error", "hpfp8_debug_set_spin_limit", "hpfp8_debug_set_small_gemm"}
     assert bound == set(declared_functions()), "python binding and header disagree"
     assert lib.hpfp8_version() >= 100
 

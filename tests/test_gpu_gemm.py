@@ -20,6 +20,18 @@ TOL_F32 = 1e-4           # fp32 output vs float64 reference
 TOL_BF16 = 3e-3          # bf16 output: one rounding (2^-9 relative per element)
 
 
+@pytest.fixture(autouse=True, params=["large tiles only", "default rule"])
+def gemm_kernel_choice(request):
+    """Most shapes here have few tiles, which the library would hand to its small-tile kernel: every test of this
+    module runs once with that kernel switched off (so the 256 x 256-tile kernel sees the small, ragged and edge
+    cases too) and once under the default rule."""
+    from hpfp8 import _lib
+    lib = _lib.load()
+    lib.hpfp8_debug_set_small_gemm(1 if request.param == "large tiles only" else 0)
+    yield
+    lib.hpfp8_debug_set_small_gemm(0)
+
+
 def rel(a, b):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
@@ -694,3 +706,65 @@ def test_weight_matrix_larger_than_2_gib(gpu):
     yg = hpfp8.gemm_grouped_blockwise(xq, sx, b.view(E, Ne, K), sb.view(E, Ne // 128, K // 128), offs)
     assert torch.equal(yg[:100], hpfp8.gemm_blockwise(xq[:100], sx[:100], b[78 * Ne:79 * Ne], sb[78 * 32:79 * 32]))
     assert torch.equal(yg[100:], hpfp8.gemm_blockwise(xq[100:], sx[100:], b[79 * Ne:], sb[79 * 32:]))
+
+
+@pytest.fixture
+def small_gemm_mode():
+    """Sets the kernel-selection hook for one test and restores the default rule afterwards."""
+    from hpfp8 import _lib
+    lib = _lib.load()
+    yield lib.hpfp8_debug_set_small_gemm
+    lib.hpfp8_debug_set_small_gemm(0)
+
+
+@pytest.mark.parametrize("shape", [(2048, 1024, 1024), (1, 128, 128), (130, 384, 256), (64, 2304, 512), (257, 128, 1152),
+                                   (1000, 640, 384)])
+def test_small_tile_kernel_equals_the_large_tile_kernel_and_the_oracle(gpu, shape, small_gemm_mode):
+    """The 128 x 128-tile kernel (problems with few tiles: BASELINE configuration 1, decode-sized M) does the same
+    arithmetic in the same order as the 256 x 256-tile kernel: identical bits for the block and the per-tensor
+    form, fp32 and bf16 output, with and without bias, ragged M; and the fp32 output agrees with the oracle as the
+    large kernel's does."""
+    import hpfp8
+    m, n, k = shape
+    x = U.randn_bf16((m, k), 40 + m, 1.0, 0.001, 30.0).to(gpu)
+    w = U.randn_bf16((n, k), 41 + n, 0.05).to(gpu)
+    bias = U.randn_bf16((n,), 42, 0.5).to(gpu)
+    xq, sx = hpfp8.quantize_1x128(x)
+    wq, sw = hpfp8.quantize_128x128(w)
+    xt, _, sxt = hpfp8.quantize_per_tensor(x)
+    wt, _, swt = hpfp8.quantize_per_tensor(w)
+    out = {}
+    for mode in (1, 2):
+        small_gemm_mode(mode)
+        out[mode] = [hpfp8.gemm_blockwise(xq, sx, wq, sw, out_dtype=torch.float32),
+                     hpfp8.gemm_blockwise(xq, sx, wq, sw, bias=bias),
+                     hpfp8.gemm_per_tensor(xt, sxt, wt, swt, out_dtype=torch.float32),
+                     hpfp8.gemm_per_tensor(xt, sxt, wt, swt, bias=bias)]
+    for big, small in zip(out[1], out[2]):
+        assert torch.equal(big.view(torch.int32) if big.dtype == torch.float32 else big.view(torch.int16),
+                           small.view(torch.int32) if small.dtype == torch.float32 else small.view(torch.int16))
+    if m * n * k <= 2048 * 1024 * 1024:
+        want, _ = O.gemm_blockwise(U.codes(xq), U.f32(sx), U.codes(wq), U.f32(sw))
+        assert rel(U.f32(out[2][0]), want) < TOL_F32
+    # a strided a operand and k-block-major scales take the same path
+    small_gemm_mode(2)
+    xq2, sx2 = hpfp8.quantize_1x128(x, kmajor=True)
+    c2 = hpfp8.gemm_blockwise(xq2, sx2, wq, sw, out_dtype=torch.float32)
+    assert torch.equal(c2, out[2][0])
+
+
+def test_small_problems_select_the_small_tile_kernel(gpu, small_gemm_mode):
+    """Under the default rule configuration 1 (32 large tiles) runs the small-tile kernel and configuration 2 does
+    not; observable through the hook: forcing either kernel gives the same bits, so only timing can tell -- here
+    the rule itself is checked through identical results in all three modes on a small and a larger problem."""
+    import hpfp8
+    for m, n, k in ((2048, 1024, 1024), (1024, 8192, 256)):
+        x = U.randn_bf16((m, k), 50, 1.0).to(gpu)
+        w = U.randn_bf16((n, k), 51, 0.05).to(gpu)
+        xq, sx = hpfp8.quantize_1x128(x, kmajor=True)
+        wq, sw = hpfp8.quantize_128x128(w)
+        res = []
+        for mode in (0, 1, 2):
+            small_gemm_mode(mode)
+            res.append(hpfp8.gemm_blockwise(xq, sx, wq, sw))
+        assert torch.equal(res[0], res[1]) and torch.equal(res[0], res[2])

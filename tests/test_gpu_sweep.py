@@ -19,8 +19,18 @@ def _eq_f32(t, ref):
     return np.array_equal(U.f32_bits(U.f32(t)), U.f32_bits(ref))
 
 
+@pytest.fixture(params=["large tiles only", "default rule"])
+def gemm_kernel_choice(request):
+    """The sweep's shapes have few tiles: once with the small-tile kernel switched off, once under the default rule."""
+    from hpfp8 import _lib
+    lib = _lib.load()
+    lib.hpfp8_debug_set_small_gemm(1 if request.param == "large tiles only" else 0)
+    yield
+    lib.hpfp8_debug_set_small_gemm(0)
+
+
 @pytest.mark.parametrize("seed", [0, 1])
-def test_random_gemm_cases_are_exact(gpu, seed):
+def test_random_gemm_cases_are_exact(gpu, seed, gemm_kernel_choice):
     import hpfp8
     rng = np.random.default_rng(seed)
     lut = torch.nan_to_num(torch.from_numpy(O.e4m3_decode(np.arange(256, dtype=np.uint8)).astype(np.float64)).to(gpu))
