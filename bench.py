@@ -204,6 +204,21 @@ def other_configs_compact(dev):
                               "note": "launch-bound: three launches (clear two words, one-pass amax + cast, 128 x 128-tile GEMM), "
                                       "times include the launches"}
     del x, w, xq, wq, q1, c1
+    # cfg 2's layer as an inference MLP block: the gate/up GEMM with SwiGLU + the 1x128 quantizer as its epilogue
+    # (no bf16 gate/up tensor), then the down projection
+    x = torch.randn((4096, 7168), generator=g, device=dev).to(torch.bfloat16)
+    gu = hpfp8.quantize_weight((torch.randn((36864, 7168), generator=g, device=dev) * 0.006).to(torch.bfloat16), with_transpose=False)
+    dn = hpfp8.quantize_weight((torch.randn((7168, 18432), generator=g, device=dev) * 0.006).to(torch.bfloat16), with_transpose=False)
+    xq, sx = hpfp8.quantize_1x128(x, kmajor=True)
+    fl_gu, fl_mlp = 2.0 * 4096 * 36864 * 7168, 2.0 * 4096 * 7168 * (36864 + 18432)
+    with torch.no_grad():
+        res["cfg2_mlp_inference"] = {
+            "gate_up_gemm_with_swiglu_quantize_epilogue": _tf(fl_gu, _time(
+                lambda: ops.gemm_blockwise_swiglu_quantize(xq, sx, gu.codes, gu.scale_inv, fast=True), iters=20)),
+            "block_forward": _tf(fl_mlp, _time(lambda: hpfp8.fp8_swiglu_mlp(x, gu, dn, fast=True), iters=20)),
+        }
+    del x, gu, dn, xq, sx
+    torch.cuda.empty_cache()
     # cfg 3: o_proj backward, M = 4096 tokens, W[7168, 16384]
     m, n, k = 4096, 7168, 16384
     x = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
