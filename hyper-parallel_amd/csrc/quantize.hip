@@ -588,7 +588,11 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // With SW (1: exactly specified silu, 2: hardware exponential and reciprocal) the source is h[M, 2K] = gate | up
 // and what is quantized is act = silu(gate) * up, computed as the tile is loaded: both operand forms of the
 // down projection's input from one read of the gate/up output, the bf16 activation never written.
-// ld_src: row stride of the source in elements (K, or at least 2K with SW).
+// With SW = 3 the source is again h[M, K] = gate | up (K = 2 * inter) together with dact[M, K / 2], and what is
+// quantized is the gradient of SwiGLU, d gate | d up [M, K], computed as the tile is loaded exactly as
+// swiglu_backward_kernel computes it: both operand forms of the gate/up projection's output gradient (dgrad and
+// wgrad) without the bf16 gradient ever being written.
+// ld_src: row stride of the source in elements (K, or at least 2K with SW = 1, 2).
 // With GROUPED (MoE: rows of x sorted by expert) the 128-row groups restart at every expert's first row and the
 // transposed output lives on the padded token axis of `layout` (grouped.hip): output block tr belongs to expert
 // layout[5E + 1 + tr], holds that expert's rows [128 j, 128 j + 128) (j = tr - the expert's first block) and is
@@ -603,7 +607,7 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
                                                             uint8_t* __restrict__ q, float* __restrict__ scale_r,
                                                             float* __restrict__ scale_inv_r, int pow2,
                                                             const int32_t* __restrict__ layout = nullptr, int experts = 0,
-                                                            int padded_blocks = 0) {
+                                                            int padded_blocks = 0, const uint16_t* __restrict__ dact = nullptr) {
   static_assert(!GROUPED || (SW == 0 && kTilesPerBlock == 1), "grouped form: plain source, one tile per workgroup");
   const int kb = k >> 7, mb = GROUPED ? padded_blocks : m >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
@@ -630,6 +634,32 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
   }
   auto load_tile = [&](int t, uint4 v[8]) {
     const int tc = t / mb, tr = t % mb;
+    if (SW == 3) {
+      // tile columns [0, inter) are d gate (from gate, up and d act), [inter, 2 inter) are d up (from gate and d act)
+      const int inter = k >> 1;
+      const bool is_gate = tc * 128 < inter;
+      const int c0 = tc * 128 - (is_gate ? 0 : inter) + cg * 8;     // column inside the gate / up half and inside d act
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const int64_t row = (int64_t)tr * 128 + tile_row(rq, p);
+        const uint4 gv = nt_load16(x + row * ld_src + c0);
+        const uint4 dv = nt_load16(dact + row * inter + c0);
+        uint32_t unused;
+        if (is_gate) {
+          const uint4 uv = nt_load16(x + row * ld_src + inter + c0);
+          swiglu_bwd2(gv.x, uv.x, dv.x, v[p].x, unused);
+          swiglu_bwd2(gv.y, uv.y, dv.y, v[p].y, unused);
+          swiglu_bwd2(gv.z, uv.z, dv.z, v[p].z, unused);
+          swiglu_bwd2(gv.w, uv.w, dv.w, v[p].w, unused);
+        } else {
+          swiglu_bwd2(gv.x, 0u, dv.x, unused, v[p].x);
+          swiglu_bwd2(gv.y, 0u, dv.y, unused, v[p].y);
+          swiglu_bwd2(gv.z, 0u, dv.z, unused, v[p].z);
+          swiglu_bwd2(gv.w, 0u, dv.w, unused, v[p].w);
+        }
+      }
+      return;
+    }
     const int64_t off = (int64_t)(GROUPED ? g_row0 : tr * 128) * ld_src + tc * 128 + cg * 8;
 #pragma unroll
     for (int p = 0; p < 8; ++p)
@@ -1112,6 +1142,31 @@ int hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, in
   else
     quant_128x1_t_kernel<true, true, 1><<<grid, 256, 0, s>>>((const uint16_t*)h, ld_h, (int)rows, (int)inter, (uint8_t*)q_t, ld_t,
                                                             scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0);
+  return check_launch(what);
+}
+
+int hpfp8_swiglu_backward_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h,
+                                                          const void* dact, void* q, float* scale, float* scale_inv,
+                                                          void* q_t, int64_t ld_t, float* scale_t, float* scale_inv_t,
+                                                          hpfp8_stream_t stream) {
+  const char* what = "swiglu_backward_quantize_1x128_and_128x1_t";
+  HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
+  HPFP8_REQUIRE(rows % kBlock == 0 && inter % kBlock == 0, HPFP8_ERR_SHAPE,
+                "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)rows, (long long)inter);
+  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 29), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
+  const int64_t blocks = (rows / kBlock) * (2 * inter / kBlock);
+  if (blocks == 0) return HPFP8_OK;
+  HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
+  HPFP8_REQUIRE(h && dact && q && scale_inv && q_t && scale_inv_t, HPFP8_ERR_ARG, "%s: null buffer", what);
+  HPFP8_REQUIRE(aligned16(h) && aligned16(dact) && aligned16(q) && aligned16(q_t), HPFP8_ERR_ALIGN,
+                "%s: buffers must be 16-byte aligned", what);
+  HPFP8_REQUIRE(ld_h >= 2 * inter && ld_h % 8 == 0, HPFP8_ERR_SHAPE,
+                "%s: ld_h=%lld must be a multiple of 8 and at least twice the width", what, (long long)ld_h);
+  HPFP8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, HPFP8_ERR_SHAPE, "%s: ld_t=%lld must be a multiple of 16 and at least rows",
+                what, (long long)ld_t);
+  quant_128x1_t_kernel<true, true, 3><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)h, ld_h, (int)rows, (int)(2 * inter), (uint8_t*)q_t, ld_t, scale_t, scale_inv_t, (uint8_t*)q, scale,
+      scale_inv, 0, nullptr, 0, 0, (const uint16_t*)dact);
   return check_launch(what);
 }
 

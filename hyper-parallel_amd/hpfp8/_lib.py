@@ -30,6 +30,7 @@ SIGNATURES = {
     "hpfp8_swiglu_quantize_1x128_bf16": [_vp, _i64, _i64, _i64, ctypes.c_int, _vp, _vp, _vp, _vp, _vp],
     "hpfp8_swiglu_quantize_1x128_pow2_bf16": [_vp, _i64, _i64, _i64, ctypes.c_int, _vp, _vp, _vp, _vp, _vp],
     "hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16": [_vp, _i64, _i64, _i64, ctypes.c_int, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp],
+    "hpfp8_swiglu_backward_quantize_1x128_and_128x1_t_bf16": [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_swiglu_backward_bf16": [_vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp],
     "hpfp8_swiglu_quantize_1x128_fast_bf16": [_vp, _i64, _i64, _i64, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp],
     "hpfp8_dequantize_1x128_accumulate_f32": [_vp, _vp, _i64, _i64, _vp, ctypes.c_float, _vp],

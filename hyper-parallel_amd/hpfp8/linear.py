@@ -538,6 +538,47 @@ class _Fp8SwiGLUDown(torch.autograd.Function):
         return dh, dw, None, None, None, None
 
 
+class _Fp8SwiGLUMLPBlock(torch.autograd.Function):
+    """The whole block y = F.linear(silu(gate) * up, w_down), gate | up = F.linear(x, w_gate_up), as one autograd node
+    (blockwise recipe, both weights trained, token count a multiple of 128).  Every bf16 tensor between the GEMMs is
+    read once: x, the gate/up output and grad_out each give both of their operand forms in one pass, and in backward
+    the gradient of SwiGLU is quantized for the gate/up projection's two GEMMs as it is computed, so d gate | d up is
+    never written in bf16."""
+
+    @staticmethod
+    def forward(ctx, x, w_gate_up, w_down, fast, gu8, dn8):
+        x2 = _flatten(x).contiguous()
+        need_dx = x.requires_grad
+        xq, sx, xt, sxt = ops.quantize_1x128_and_128x1_t(x2, kmajor=True)
+
+        def forms(w, f8):
+            if f8 is None:
+                return ops.quantize_128x128(w, with_transpose=True)
+            return f8.codes, f8.scale_inv, f8.codes_t if f8.codes_t is not None else ops.transpose_codes(f8.codes)
+        gq, gs, gqt = forms(w_gate_up, gu8)
+        dq, ds, dqt = forms(w_down, dn8)
+        h = ops.gemm_blockwise(xq, sx, gq, gs)
+        aq, sa, at, sat = ops.swiglu_quantize_1x128_and_128x1_t(h, fast=fast)
+        y = ops.gemm_blockwise(aq, sa, dq, ds)
+        ctx.save_for_backward(h, xt, sxt, gqt if need_dx else None, gs, dqt, ds, at, sat)
+        ctx.x_shape, ctx.need_dx = x.shape, need_dx
+        return y.reshape(x.shape[:-1] + (w_down.shape[0],))
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        h, xt, sxt, gqt, gs, dqt, ds, at, sat = ctx.saved_tensors
+        go = _flatten(grad_out)
+        if go.dtype != torch.bfloat16:
+            go = go.to(torch.bfloat16)
+        goq, sgo, got, sgot = ops.quantize_1x128_and_128x1_t(go.contiguous(), kmajor=True)
+        dw_down = ops.gemm_blockwise(got, sgot, at, sat, sb_gran=1)
+        dact = ops.gemm_blockwise(goq, sgo, dqt, ds.t())
+        dhq, sdh, dht, sdht = ops.swiglu_backward_quantize_1x128_and_128x1_t(h, dact)
+        dx = ops.gemm_blockwise(dhq, sdh, gqt, gs.t()).reshape(ctx.x_shape) if ctx.need_dx else None
+        dw_gate_up = ops.gemm_blockwise(dht, sdht, xt, sxt, sb_gran=1)
+        return dx, dw_gate_up, dw_down, None, None, None
+
+
 def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True,
                    gate_up_fp8: Optional[Fp8Weight] = None, down_fp8: Optional[Fp8Weight] = None) -> torch.Tensor:
     """A SwiGLU MLP block (DeepSeekV3 dense MLP): ``F.linear(F.silu(gate) * up, w_down)`` with
@@ -559,10 +600,18 @@ def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True,
         for f8 in (gate_up_fp8, down_fp8):
             if f8 is not None and f8.pow2:
                 raise ValueError("the training path of fp8_swiglu_mlp uses the blockwise recipe with plain fp32 scales")
-        h = fp8_linear(input, w_gate_up, weight_fp8=gate_up_fp8)
         d8 = down_fp8
         if d8 is not None and d8.codes.shape != w_down.shape:
             raise ValueError("down_fp8 does not belong to w_down")
+        if gate_up_fp8 is not None and gate_up_fp8.codes.shape != w_gate_up.shape:
+            raise ValueError("gate_up_fp8 does not belong to w_gate_up")
+        if input.shape[-1] != w_gate_up.shape[1]:
+            raise ValueError(f"input last dim {input.shape[-1]} != w_gate_up in_features {w_gate_up.shape[1]}")
+        rows = input.numel() // max(input.shape[-1], 1)
+        if (w_gate_up.requires_grad and w_down.requires_grad and rows > 0 and rows % ops.BLOCK == 0
+                and input.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and w_down.dtype == torch.bfloat16):
+            return _Fp8SwiGLUMLPBlock.apply(input, w_gate_up, w_down, fast, gate_up_fp8, d8)
+        h = fp8_linear(input, w_gate_up, weight_fp8=gate_up_fp8)
         return _Fp8SwiGLUDown.apply(h, w_down, fast, *((d8.codes, d8.scale_inv, d8.codes_t) if d8 is not None else ()))
     gu = w_gate_up if isinstance(w_gate_up, Fp8Weight) else (gate_up_fp8 or quantize_weight(w_gate_up.detach(), with_transpose=False))
     dn = w_down if isinstance(w_down, Fp8Weight) else (down_fp8 or quantize_weight(w_down.detach(), with_transpose=False))

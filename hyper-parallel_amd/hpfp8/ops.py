@@ -254,6 +254,26 @@ def swiglu_backward(h: torch.Tensor, dact: torch.Tensor) -> torch.Tensor:
     return dh
 
 
+def swiglu_backward_quantize_1x128_and_128x1_t(h: torch.Tensor, dact: torch.Tensor):
+    """`swiglu_backward` fused with both quantized forms of its result dh = [d gate | d up] ([M, 2I]; never written in
+    bf16): (codes[M, 2I], scale_inv[M, 2I/128], codes_t[2I, M], scale_inv_t[2I, M/128]), k-block-major scales,
+    bit-identical to ``quantize_1x128_and_128x1_t(swiglu_backward(h, dact))``.  M and I multiples of 128."""
+    h = _check_bf16(h, "h", contiguous=False)
+    dact = _check_bf16(dact, "dact")
+    if h.dim() != 2 or h.shape[1] % (2 * BLOCK) or h.shape[0] % BLOCK or dact.shape != (h.shape[0], h.shape[1] // 2):
+        raise ValueError("h must be [M, 2I] with M and I multiples of 128 and dact [M, I]")
+    if h.stride(1) != 1 or h.stride(0) % 8 or h.data_ptr() % 16:
+        h = h.contiguous()
+    m, inter = dact.shape
+    q = torch.empty((m, 2 * inter), dtype=FP8, device=h.device)
+    qt = _empty_codes_t(2 * inter, m, h.device)
+    s_inv = torch.empty((2 * inter // BLOCK, m), dtype=torch.float32, device=h.device)
+    st_inv = torch.empty((m // BLOCK, 2 * inter), dtype=torch.float32, device=h.device)
+    _lib.call("hpfp8_swiglu_backward_quantize_1x128_and_128x1_t_bf16", _ptr(h), m, inter, h.stride(0) if m > 1 else 2 * inter,
+              _ptr(dact), _ptr(q), None, _ptr(s_inv), _ptr(qt), _ld(qt), None, _ptr(st_inv), _stream())
+    return q, s_inv.t(), qt, st_inv.t()
+
+
 def transpose_codes(q: torch.Tensor) -> torch.Tensor:
     """codes[R, C] -> codes_t[C, R] (byte transpose; R, C multiples of 128).  With 128x128 scaling blocks
     the transposed codes of a weight are its dgrad operand, scales reused with swapped strides."""

@@ -190,6 +190,17 @@ int hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, in
 int hpfp8_swiglu_backward_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h, const void* dact, void* dh,
                                int64_t ld_dh, hpfp8_stream_t stream);
 
+/* hpfp8_swiglu_backward_bf16 fused with both quantized forms of its result (training: the output gradient of the
+ * gate/up projection as its dgrad operand and its wgrad operand, from one read of h and dact; the bf16 gradient
+ * d gate | d up is never written): with dh the [rows, 2 * inter] tensor hpfp8_swiglu_backward_bf16 would write,
+ * q[rows, 2 * inter], scale / scale_inv [2 * inter / 128, rows] are hpfp8_quantize_1x128_kmajor_bf16(dh) and
+ * q_t[2 * inter, rows] (row stride ld_t), scale_t / scale_inv_t [rows / 128, 2 * inter] are
+ * hpfp8_quantize_128x1_t_kmajor_bf16(dh), bit for bit.  rows and inter multiples of 128; dact contiguous. */
+int hpfp8_swiglu_backward_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, int64_t inter, int64_t ld_h,
+                                                          const void* dact, void* q, float* scale, float* scale_inv,
+                                                          void* q_t, int64_t ld_t, float* scale_t, float* scale_inv_t,
+                                                          hpfp8_stream_t stream);
+
 /* Byte transpose of a code matrix: q[rows, cols] (row stride ld) -> q_t[cols, rows] (row stride ld_t);
  * rows, cols multiples of 128.  128x128 scaling blocks are symmetric, so this turns the codes of a
  * weight into its dgrad operand without requantizing, e.g. after FP8 shards were all-gathered: the

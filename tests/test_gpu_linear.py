@@ -493,6 +493,55 @@ def test_swiglu_mlp_training_step_vs_torch(gpu):
     assert torch.equal(y2, y) and rel(x2.grad, gx) < 1e-6
 
 
+def test_swiglu_backward_fused_with_both_quantized_forms(gpu):
+    """The gradient of SwiGLU quantized for the gate/up projection's dgrad and wgrad as it is computed: codes and
+    scales of both forms equal, bit for bit, the two quantizers applied to the bf16 gradient that the stand-alone
+    backward kernel writes (rows of a wider buffer as h give the same); and the MLP block as one autograd node
+    (which uses it) returns the same output and the same three gradients, bit for bit, as the chain of
+    fp8_linear and the SwiGLU + down-projection node that it replaces."""
+    import hpfp8
+    from hpfp8 import ops
+    from hpfp8.linear import _Fp8SwiGLUDown
+    m, inter = 384, 640
+    h = U.randn_bf16((m, 2 * inter), 31, 2.0, 0.001, 20.0).to(gpu)
+    h[0, :6] = torch.tensor([0.0, -0.0, 88.5, -88.5, -200.0, 200.0], dtype=torch.bfloat16)
+    dact = U.randn_bf16((m, inter), 32, 1e-2, 0.001, 50.0).to(gpu)
+    dh = ops.swiglu_backward(h, dact)
+    q1, s1, qt1, st1 = hpfp8.quantize_1x128_and_128x1_t(dh, kmajor=True)
+    q, s, qt, st = ops.swiglu_backward_quantize_1x128_and_128x1_t(h, dact)
+    assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(s, s1)
+    assert torch.equal(qt.view(torch.uint8), qt1.view(torch.uint8)) and torch.equal(st, st1)
+    assert s.stride(0) == 1 and st.stride(0) == 1
+    wide = torch.zeros((m, 2 * inter + 64), dtype=torch.bfloat16, device=gpu)
+    wide[:, :2 * inter] = h
+    q2, s2, qt2, st2 = ops.swiglu_backward_quantize_1x128_and_128x1_t(wide[:, :2 * inter], dact)
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(qt2.view(torch.uint8), qt.view(torch.uint8))
+    assert torch.equal(s2, s) and torch.equal(st2, st)
+    with pytest.raises(ValueError):
+        ops.swiglu_backward_quantize_1x128_and_128x1_t(h[:100], dact[:100])
+    # the block as one node against the two nodes it replaces
+    g = torch.Generator(device="cpu").manual_seed(9)
+    k, n = 512, 384
+    x = torch.randn((m, k), generator=g).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    wgu = (torch.randn((2 * inter, k), generator=g) * 0.05).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    wd = (torch.randn((n, inter), generator=g) * 0.05).to(torch.bfloat16).to(gpu).requires_grad_(True)
+    go = (torch.randn((m, n), generator=g) * 1e-2).to(torch.bfloat16).to(gpu)
+    for fast in (True, False):
+        y = hpfp8.fp8_swiglu_mlp(x, wgu, wd, fast=fast)
+        assert type(y.grad_fn).__name__.startswith("_Fp8SwiGLUMLPBlock")
+        got = torch.autograd.grad(y, (x, wgu, wd), go)
+        y0 = _Fp8SwiGLUDown.apply(hpfp8.fp8_linear(x, wgu), wd, fast)
+        want = torch.autograd.grad(y0, (x, wgu, wd), go)
+        assert torch.equal(y, y0)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+    # an input that needs no gradient: the same weight gradients
+    y = hpfp8.fp8_swiglu_mlp(x.detach(), wgu, wd)
+    got2 = torch.autograd.grad(y, (wgu, wd), go)
+    ref2 = torch.autograd.grad(hpfp8.fp8_swiglu_mlp(x, wgu, wd), (wgu, wd), go)
+    assert torch.equal(got2[0], ref2[0]) and torch.equal(got2[1], ref2[1])
+
+
 def test_mlp_training_step_replays_from_a_captured_graph(gpu):
     """Forward and backward of the MLP block captured into one graph (weights prequantized outside it): every
     replay, with eager work and synchronisations in between, gives the eager step's output and gradients for
