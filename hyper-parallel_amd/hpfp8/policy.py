@@ -76,3 +76,19 @@ def cast_fp_tensor(dtype: torch.dtype, x):
         q, _, scale_inv = ops.quantize_per_tensor(src.contiguous())
         return Fp8Tensor(q, scale_inv)
     return x.to(dtype)
+
+
+# `TorchPlatform.tensor_type_cast`'s name -> dtype table (hyper_parallel/platform/torch/platform.py:195-206) with the
+# two names this path adds
+_TYPE_NAMES = {"float32": torch.float32, "float16": torch.float16, "int64": torch.int64, "int32": torch.int32,
+               "bfloat16": torch.bfloat16, "float8_e4m3fn": ops.FP8}
+
+
+def tensor_type_cast(input_data: torch.Tensor, cast_type: str):
+    """`TorchPlatform.tensor_type_cast` (hyper_parallel/platform/torch/platform.py:195-206) with "float8_e4m3fn"
+    among its names: that name gives an `Fp8Tensor` through `cast_fp_tensor`, the others are `.to(dtype)`; an
+    unknown name raises the reference's ValueError."""
+    if cast_type not in _TYPE_NAMES:
+        raise ValueError(f"Unknown cast type: {cast_type}. Supported types: {list(_TYPE_NAMES.keys())}")
+    dtype = _TYPE_NAMES[cast_type]
+    return cast_fp_tensor(dtype, input_data) if dtype == ops.FP8 else input_data.to(dtype)

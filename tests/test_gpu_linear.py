@@ -375,6 +375,12 @@ def test_policy_record_and_fp8_cast_hook(gpu):
     oq, _, osi = O.quantize_per_tensor(U.bits(x.reshape(-1)[:3007]))
     assert np.array_equal(U.bits(odd.dequantize()), O.dequantize_per_tensor(oq, osi))
     assert np.array_equal(U.f32_bits(U.f32(odd.dequantize(torch.float32))), U.f32_bits(O.dequantize_per_tensor_f32(oq, osi)))
+    # the name-keyed cast of the reference's platform, with the FP8 name added
+    t2 = hpfp8.tensor_type_cast(x, "float8_e4m3fn")
+    assert torch.equal(t2.codes.view(torch.uint8), t.codes.view(torch.uint8)) and torch.equal(t2.scale_inv, t.scale_inv)
+    assert hpfp8.tensor_type_cast(x, "float32").dtype == torch.float32 and hpfp8.tensor_type_cast(ints, "int32").dtype == torch.int32
+    with pytest.raises(ValueError, match="Unknown cast type"):
+        hpfp8.tensor_type_cast(x, "float8")
     pol = hpfp8.Fp8MixedPrecisionPolicy(apply_grad_on_fp32_main_grad=True, fp8_recipe="blockwise_pow2")
     w = U.randn_bf16((256, 384), 92, 0.02).to(gpu).requires_grad_(True)
     hpfp8.fp8_linear(x, w, **pol.linear_kwargs()).backward(U.randn_bf16((256, 256), 93, 1e-3).to(gpu))
