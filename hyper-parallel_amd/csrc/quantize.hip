@@ -163,13 +163,21 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* part) {
   return m;                       // the same in every thread
 }
 
-template <int VEC>
+// SYNC3: the grid agrees through three words of the caller's that are zero at launch and zero again when the
+// kernel ends -- amax_word (maximum), count_word (arrivals) and a third word counting departures: a workgroup adds
+// to it after its last touch of the other two, and the last one to leave clears all three.  No word needs
+// clearing before the launch then, and the results go to their own outputs (amax_out, scale_out, scale_inv_out).
+// (A workgroup whose wait ran out computes the maximum alone and publishes nothing: the words could already be
+// cleared.)
+template <int VEC, bool SYNC3 = false>
 __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(const uint16_t* __restrict__ x, int64_t n,
                                                                      uint32_t* __restrict__ amax_word,
                                                                      uint32_t* __restrict__ count_word,
                                                                      uint8_t* __restrict__ q,
                                                                      float* __restrict__ scale_out,
-                                                                     uint32_t spin_limit) {
+                                                                     uint32_t spin_limit,
+                                                                     float* __restrict__ amax_out = nullptr,
+                                                                     float* __restrict__ scale_inv_out = nullptr) {
   __shared__ uint32_t part[16];
   __shared__ uint32_t s_amax, s_alone, s_repair;
   const uint4* xv = reinterpret_cast<const uint4*>(x);
@@ -205,6 +213,15 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
     __atomic_thread_fence(__ATOMIC_ACQUIRE);          // (agent scope and wider)
     s_amax = __hip_atomic_load(amax_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 16;
     s_alone = seen < grid ? 1u : 0u;
+    if (SYNC3) {
+      // this workgroup is done with the words; the last one to say so clears them for the next launch
+      uint32_t* depart = count_word + 1;
+      if (__hip_atomic_fetch_add(depart, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) + 1u == grid) {
+        __hip_atomic_store(amax_word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(count_word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(depart, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
   }
   __syncthreads();
   uint32_t amax16 = s_amax;
@@ -213,7 +230,7 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
     for (int64_t i = threadIdx.x; i < nvec; i += kFusedThreads) mm = umax(mm, mag8(xv[i]));
     if (threadIdx.x < (n & 7)) mm = umax(mm, x[(nvec << 3) + threadIdx.x] & 0x7FFFu);
     amax16 = block_max_u32(mm, part);
-    if (threadIdx.x == 0) __hip_atomic_fetch_max(amax_word, amax16 << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!SYNC3 && threadIdx.x == 0) __hip_atomic_fetch_max(amax_word, amax16 << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   float scale, scale_inv;
   scales_from_amax(__uint_as_float(amax16 << 16), scale, scale_inv);
@@ -224,6 +241,14 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
     if (i < nvec) nt_store8(&qv[i], cvt8<true>(v[u], scale));
   }
   if (has_tail) q[(nvec << 3) + threadIdx.x] = (uint8_t)(cvt2<false, true>(0u, tail, scale) & 0xFFu);
+  if (SYNC3) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+      if (amax_out) *amax_out = __uint_as_float(amax16 << 16);
+      if (scale_out) *scale_out = scale;
+      if (scale_inv_out) *scale_inv_out = scale_inv;
+    }
+    return;
+  }
   if (threadIdx.x == 0 && (blockIdx.x == 0 || s_repair)) {
     if (scale_out) *scale_out = scale;
     // scale_inv takes the place of the count (ordered after the maximum this workgroup may have published)
@@ -231,6 +256,8 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
   }
 }
 
+// (SYNC3: the `seen > grid` repair of the two-word form cannot occur -- every workgroup arrives exactly once
+// between two clearings.)
 // Polls a waiting workgroup makes before it stops relying on the others (about a microsecond each).
 static uint32_t g_spin_limit = 1u << 22;
 
@@ -984,6 +1011,31 @@ int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* ama
 }
 
 void hpfp8_debug_set_spin_limit(uint32_t polls) { g_spin_limit = polls; }
+
+int hpfp8_quantize_per_tensor_sync_bf16(const void* x, int64_t n, void* q, float* amax, float* scale, float* scale_inv,
+                                        uint32_t* sync, hpfp8_stream_t stream) {
+  const char* what = "quantize_per_tensor_sync";
+  HPFP8_REQUIRE(n >= 0, HPFP8_ERR_SHAPE, "%s: negative size", what);
+  HPFP8_REQUIRE(n <= kFusedMaxElems, HPFP8_ERR_SHAPE, "%s: at most %lld elements (the one-pass form); larger tensors take "
+                "hpfp8_quantize_per_tensor_bf16", what, (long long)kFusedMaxElems);
+  if (n == 0) return hpfp8_quantize_per_tensor_bf16(x, n, q, amax, scale, scale_inv, stream);
+  HPFP8_REQUIRE(x && q && sync, HPFP8_ERR_ARG, "%s: null buffer", what);
+  HPFP8_REQUIRE(aligned16(x) && aligned16(q) && aligned16(sync), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
+  const int64_t nvec = (n >> 3) > 0 ? (n >> 3) : 1;
+  const int64_t per_thread = (nvec + (int64_t)kFusedMaxBlocks * kFusedThreads - 1) / ((int64_t)kFusedMaxBlocks * kFusedThreads);
+  const int vec = per_thread <= 1 ? 1 : (per_thread <= 2 ? 2 : (per_thread <= 4 ? 4 : 8));
+  const unsigned grid = (unsigned)((nvec + kFusedThreads * vec - 1) / (kFusedThreads * vec));
+  const uint16_t* xs = (const uint16_t*)x;
+  uint8_t* q8 = (uint8_t*)q;
+  hipStream_t s = (hipStream_t)stream;
+  switch (vec) {
+    case 1: quant_per_tensor_fused_kernel<1, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
+    case 2: quant_per_tensor_fused_kernel<2, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
+    case 4: quant_per_tensor_fused_kernel<4, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
+    default: quant_per_tensor_fused_kernel<8, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
+  }
+  return check_launch(what);
+}
 
 int hpfp8_quantize_per_tensor_noalloc_bf16(const void* x, int64_t n, void* q, float* scale, float* scale_inv,
                                            hpfp8_stream_t stream) {

@@ -23,6 +23,7 @@ SIGNATURES = {
     "hpfp8_amax_bf16": [_vp, _i64, _vp, _vp],
     "hpfp8_cast_per_tensor_bf16": [_vp, _i64, _vp, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_per_tensor_bf16": [_vp, _i64, _vp, _vp, _vp, _vp, _vp],
+    "hpfp8_quantize_per_tensor_sync_bf16": [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_per_tensor_noalloc_bf16": [_vp, _i64, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_1x128_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_1x128_kmajor_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],

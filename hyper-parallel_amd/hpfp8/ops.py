@@ -108,6 +108,22 @@ def amax(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+# 16 bytes per (device, stream) that hpfp8_quantize_per_tensor_sync_bf16's grid synchronises through: zero when
+# created, and left zero by every call, so calls on one stream can share them
+_SYNC_WORDS = {}
+_ONE_PASS_MAX = 1 << 22
+
+
+def _sync_words(device: torch.device) -> Optional[torch.Tensor]:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream())
+    t = _SYNC_WORDS.get(key)
+    if t is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None          # (creating them would record a fill into the graph; the two-launch form needs none)
+        t = _SYNC_WORDS[key] = torch.zeros(4, dtype=torch.int32, device=device)
+    return t
+
+
 def quantize_per_tensor(x: torch.Tensor, amax_in: Optional[torch.Tensor] = None
                         ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """One scale for the whole tensor: returns (codes like x, scale, scale_inv).
@@ -120,6 +136,11 @@ def quantize_per_tensor(x: torch.Tensor, amax_in: Optional[torch.Tensor] = None
     scale = torch.empty((), dtype=torch.float32, device=x.device)
     scale_inv = torch.empty((), dtype=torch.float32, device=x.device)
     if amax_in is None:
+        sync = _sync_words(x.device) if 0 < x.numel() <= _ONE_PASS_MAX else None
+        if sync is not None:      # one launch: amax and cast in one pass over x
+            _lib.call("hpfp8_quantize_per_tensor_sync_bf16", _ptr(x), x.numel(), _ptr(q), None, _ptr(scale), _ptr(scale_inv),
+                      _ptr(sync), _stream())
+            return q, scale, scale_inv
         am = torch.empty((), dtype=torch.float32, device=x.device)
         _lib.call("hpfp8_quantize_per_tensor_bf16", _ptr(x), x.numel(), _ptr(q), _ptr(am), _ptr(scale),
                   _ptr(scale_inv), _stream())

@@ -536,6 +536,71 @@ def test_per_tensor_one_pass_form_and_its_bounded_wait(gpu, n):
     assert np.array_equal(U.codes(q2), rq) and U.f32_bits(U.f32(si2)) == U.f32_bits(rsi)
 
 
+def test_per_tensor_single_launch_form_with_self_clearing_sync_words(gpu):
+    """hpfp8_quantize_per_tensor_sync_bf16: one launch, the grid synchronising through 16 bytes of the caller's that
+    are zero before the first call.  Calls of different sizes in a row on the same words give the oracle's codes,
+    scales and amax each time and leave the words zero -- also with every workgroup's wait cut to nothing (each then
+    computes the maximum alone and the words are still cleared); the call replays from a captured graph on changing
+    data; sizes beyond the one-pass limit and a misaligned pointer are refused."""
+    import hpfp8
+    from hpfp8 import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    sync = torch.zeros(4, dtype=torch.int32, device=gpu)
+    try:
+        for limit in (1 << 22, 0):
+            lib.hpfp8_debug_set_spin_limit(limit)
+            for n in (2048 * 1024, 5, 3007, 4 * 1024 * 1024, 8, 300000):
+                x = U.randn_bf16((n,), 200 + n % 11, 1.0 + n % 3, 0.0005, 30.0).to(gpu)
+                rq, rs, rsi = O.quantize_per_tensor(U.bits(x))
+                q = torch.empty((n,), dtype=torch.float8_e4m3fn, device=gpu)
+                out = torch.full((3,), float("nan"), dtype=torch.float32, device=gpu)
+                _lib.call("hpfp8_quantize_per_tensor_sync_bf16", x.data_ptr(), n, q.data_ptr(), out.data_ptr(), out.data_ptr() + 4,
+                          out.data_ptr() + 8, sync.data_ptr(), st)
+                torch.cuda.synchronize()
+                assert np.array_equal(U.codes(q), rq), (limit, n)
+                o = U.f32_bits(U.f32(out))
+                assert o[0] == U.f32_bits(np.float32(np.abs(x.float().cpu().numpy()).max()))
+                assert o[1] == U.f32_bits(rs) and o[2] == U.f32_bits(rsi)
+                assert int(sync.abs().sum()) == 0, "the sync words were not left zero"
+    finally:
+        lib.hpfp8_debug_set_spin_limit(1 << 22)
+    # the Python wrapper takes this form for small tensors (same bits as the two-launch form)
+    x = U.randn_bf16((2048, 1024), 7, 1.0, 0.001, 20.0).to(gpu)
+    q1, s1, si1 = hpfp8.quantize_per_tensor(x)
+    rq, rs, rsi = O.quantize_per_tensor(U.bits(x))
+    assert np.array_equal(U.codes(q1), rq) and U.f32_bits(U.f32(si1)) == U.f32_bits(rsi) and U.f32_bits(U.f32(s1)) == U.f32_bits(rs)
+    # graph replay on changing data (no clearing between replays)
+    xs = [U.randn_bf16((1024, 512), 300 + i, 1.0 + i).to(gpu) for i in range(4)]
+    x_static = xs[0].clone()
+    qg = torch.empty((1024, 512), dtype=torch.float8_e4m3fn, device=gpu)
+    og = torch.zeros(3, dtype=torch.float32, device=gpu)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _lib.call("hpfp8_quantize_per_tensor_sync_bf16", x_static.data_ptr(), x_static.numel(), qg.data_ptr(), og.data_ptr(),
+                  og.data_ptr() + 4, og.data_ptr() + 8, sync.data_ptr(), side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.call("hpfp8_quantize_per_tensor_sync_bf16", x_static.data_ptr(), x_static.numel(), qg.data_ptr(), og.data_ptr(),
+                  og.data_ptr() + 4, og.data_ptr() + 8, sync.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    for x in xs[1:] + xs[:2]:
+        x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        rq, rs, rsi = O.quantize_per_tensor(U.bits(x))
+        assert np.array_equal(U.codes(qg), rq) and U.f32_bits(U.f32(og))[2] == U.f32_bits(rsi)
+        assert int(sync.abs().sum()) == 0
+    # limits
+    big = torch.zeros(4 * 1024 * 1024 + 8, dtype=torch.bfloat16, device=gpu)
+    qb = torch.empty(big.shape, dtype=torch.float8_e4m3fn, device=gpu)
+    assert lib.hpfp8_quantize_per_tensor_sync_bf16(big.data_ptr(), big.numel(), qb.data_ptr(), None, None, og.data_ptr(), sync.data_ptr(), st) == -2
+    assert lib.hpfp8_quantize_per_tensor_sync_bf16(big.data_ptr(), 1024, qb.data_ptr(), None, None, og.data_ptr(), sync.data_ptr() + 4, st) == -3
+    assert lib.hpfp8_quantize_per_tensor_sync_bf16(big.data_ptr(), 1024, qb.data_ptr(), None, None, og.data_ptr(), None, st) == -1
+
+
 def test_tensors_beyond_2_31_elements(gpu):
     """4.3 GB of bf16 (2.15e9 elements): element offsets no longer fit 32 bits.  Every quantizer gives, on
     row blocks at the start, across the 2^31-element mark and at the end, the bits it gives for those rows
