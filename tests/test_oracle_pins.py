@@ -622,3 +622,39 @@ def test_grouped_wgrad_against_float64_per_expert():
     xt2, _, sxt2 = O.quantize_128x1_t_grouped(U.bits(x)[perm], [300, 430, 430, 500])
     dw2, _ = O.gemm_grouped_wgrad(got2, sgot2, xt2, sxt2, [300, 430, 430, 500], total)
     assert np.array_equal(dw2[0].view(np.uint32), dw[2].view(np.uint32)) and np.array_equal(dw2[1].view(np.uint32), dw[0].view(np.uint32))
+
+
+def test_block_quantizer_against_an_independent_implementation_of_the_same_convention():
+    """A third implementation that none of this build's authors wrote: the 128x128 block quantizer that the
+    `transformers` package ships for DeepSeek-V3-style FP8 checkpoints (transformers/integrations/finegrained_fp8.py,
+    `Fp8Quantize._quantize_one`: scale = 448 / max|block|, clamp, cast, store 1 / scale as weight_scale_inv).  On
+    blocks that are not all zero it must produce the oracle's codes bit for bit (same multiplier, same rounding); its
+    stored inverse is 1 / (448 / amax) where the oracle divides amax / 448, so the two inverses agree to one unit in
+    the last place and are equal in most blocks; and its power-of-two format ("ue8m0": the inverse rounded up to a
+    power of two, the multiplier its reciprocal) gives the codes and scales of the oracle's pow2 recipe."""
+    fg = pytest.importorskip("transformers.integrations.finegrained_fp8")
+    if not hasattr(fg, "Fp8Quantize") or not hasattr(fg.Fp8Quantize, "_quantize_one"):
+        pytest.skip("this transformers version has no Fp8Quantize._quantize_one")
+    import types
+    w = U.randn_bf16((384, 512), 77, 0.02, 0.002, 25.0)
+    w[128:256, 0:128] *= 1e-3                                    # a block of small values
+    w[0, 0] = 0.75                                               # a block whose maximum is a power of two times 1.5
+
+    def theirs(fmt):
+        cfg = types.SimpleNamespace(weight_block_size=(128, 128), scale_fmt=fmt)
+        stub = types.SimpleNamespace(hf_quantizer=types.SimpleNamespace(quantization_config=cfg))
+        stub._resolve_block_size = lambda value: (128, 128)
+        out = fg.Fp8Quantize._quantize_one(stub, "layer.weight", w)
+        return out["layer.weight"].view(torch.uint8).numpy(), out["layer.weight_scale_inv"].to(torch.float32).numpy()
+
+    q, _, si = O.quantize_128x128(U.bits(w))
+    tq, tsi = theirs("float")
+    assert np.array_equal(tq, q), f"{int((tq != q).sum())} codes differ"
+    ulps = np.abs(tsi.view(np.int32).astype(np.int64) - si.view(np.int32).astype(np.int64))
+    assert ulps.max() <= 1 and (ulps == 0).mean() >= 0.5
+    try:
+        tq2, tsi2 = theirs("ue8m0")
+    except Exception as e:                                       # (a torch build without the E8M0 dtype)
+        pytest.skip(f"power-of-two format not available: {e}")
+    q2, _, si2 = O.quantize_128x128(U.bits(w), pow2=True)
+    assert np.array_equal(tsi2, si2) and np.array_equal(tq2, q2)
