@@ -193,7 +193,7 @@ def other_configs_compact(dev):
     w3 = torch.zeros(3, dtype=torch.float32, device=dev)
     c1 = torch.empty((2048, 1024), dtype=torch.bfloat16, device=dev)
     pw = w3.data_ptr()
-    sync = torch.zeros(4, dtype=torch.int32, device=dev)
+    sync = torch.zeros(128, dtype=torch.int32, device=dev)
     quant = lambda: _lib.call("hpfp8_quantize_per_tensor_sync_bf16", x.data_ptr(), x.numel(), q1.data_ptr(), pw, pw + 4, pw + 8,
                               sync.data_ptr(), st)
     gemm = lambda: _lib.call("hpfp8_gemm_per_tensor", xq.data_ptr(), 1024, sx.data_ptr(), wq.data_ptr(), 1024, sw.data_ptr(),

@@ -163,12 +163,15 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t m, uint32_t* part) {
   return m;                       // the same in every thread
 }
 
-// SYNC3: the grid agrees through three words of the caller's that are zero at launch and zero again when the
-// kernel ends -- amax_word (maximum), count_word (arrivals) and a third word counting departures: a workgroup adds
-// to it after its last touch of the other two, and the last one to leave clears all three.  No word needs
-// clearing before the launch then, and the results go to their own outputs (amax_out, scale_out, scale_inv_out).
-// (A workgroup whose wait ran out computes the maximum alone and publishes nothing: the words could already be
-// cleared.)
+// SYNC3: the grid agrees through a block of the caller's that is zero at launch and zero again when the kernel ends:
+// 64 slots, one per workgroup (amax_word points at them), and a departure count (count_word).  A workgroup STORES
+// its own maximum, tagged valid, into its slot -- no read-modify-write on a shared word, whose 64 arrivals would
+// queue up behind each other across the chip -- and its first wave then polls all slots with one 256-byte load per
+// poll until every slot of the grid is valid; the maximum over the slots is the tensor's.  After its last read of
+// the slots a workgroup adds to the departure count (behind the cast's stores, off the critical path), and the last
+// one to leave clears slots and count.  No word needs clearing before the launch, and the results go to their own
+// outputs (amax_out, scale_out, scale_inv_out).  (A workgroup whose wait ran out computes the maximum alone.)
+constexpr uint32_t kSlotValid = 0x80000000u;
 template <int VEC, bool SYNC3 = false>
 __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(const uint16_t* __restrict__ x, int64_t n,
                                                                      uint32_t* __restrict__ amax_word,
@@ -200,7 +203,30 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
   }
   m = block_max_u32(m, part);
   const uint32_t grid = gridDim.x;
-  if (threadIdx.x == 0) {
+  if (SYNC3) {
+    if (threadIdx.x < 64) {              // the first wave: lane l watches slot l
+      const uint32_t lane = threadIdx.x;
+      if (lane == 0) __hip_atomic_store(amax_word + blockIdx.x, kSlotValid | m, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      uint32_t spins = 0, slot = 0;
+      bool all = false;
+      while (true) {
+        slot = lane < grid ? __hip_atomic_load(amax_word + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : kSlotValid;
+        all = __ballot((slot & kSlotValid) != 0) == ~0ull;
+        if (all || spins++ >= spin_limit) break;
+        __builtin_amdgcn_s_sleep(1);
+      }
+      __atomic_thread_fence(__ATOMIC_ACQUIRE);
+      uint32_t mx = (slot & kSlotValid) ? (slot & 0xFFFFu) : 0u;
+      mx = row16_max_u32(mx);
+      mx = umax(mx, (uint32_t)__shfl_xor((int)mx, 16));
+      mx = umax(mx, (uint32_t)__shfl_xor((int)mx, 32));
+      if (lane == 0) {
+        s_amax = mx;
+        s_alone = all ? 0u : 1u;
+        s_repair = 0u;
+      }
+    }
+  } else if (threadIdx.x == 0) {
     if ((m << 16) > __hip_atomic_load(amax_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
       __hip_atomic_fetch_max(amax_word, m << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     uint32_t seen = __hip_atomic_fetch_add(count_word, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT) + 1u;
@@ -213,15 +239,6 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
     __atomic_thread_fence(__ATOMIC_ACQUIRE);          // (agent scope and wider)
     s_amax = __hip_atomic_load(amax_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 16;
     s_alone = seen < grid ? 1u : 0u;
-    if (SYNC3) {
-      // this workgroup is done with the words; the last one to say so clears them for the next launch
-      uint32_t* depart = count_word + 1;
-      if (__hip_atomic_fetch_add(depart, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) + 1u == grid) {
-        __hip_atomic_store(amax_word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(count_word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(depart, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
   }
   __syncthreads();
   uint32_t amax16 = s_amax;
@@ -246,6 +263,18 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
       if (amax_out) *amax_out = __uint_as_float(amax16 << 16);
       if (scale_out) *scale_out = scale;
       if (scale_inv_out) *scale_inv_out = scale_inv;
+    }
+    // this workgroup has read the slots for the last time (before the barrier above); the last one to say so clears
+    // them for the next launch
+    if (threadIdx.x < 64) {
+      uint32_t last = 0;
+      if (threadIdx.x == 0)
+        last = __hip_atomic_fetch_add(count_word, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) + 1u == grid ? 1u : 0u;
+      last = (uint32_t)__shfl((int)last, 0);
+      if (last) {
+        __hip_atomic_store(amax_word + threadIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) __hip_atomic_store(count_word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
     return;
   }
@@ -1020,7 +1049,8 @@ int hpfp8_quantize_per_tensor_sync_bf16(const void* x, int64_t n, void* q, float
                 "hpfp8_quantize_per_tensor_bf16", what, (long long)kFusedMaxElems);
   if (n == 0) return hpfp8_quantize_per_tensor_bf16(x, n, q, amax, scale, scale_inv, stream);
   HPFP8_REQUIRE(x && q && sync, HPFP8_ERR_ARG, "%s: null buffer", what);
-  HPFP8_REQUIRE(aligned16(x) && aligned16(q) && aligned16(sync), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
+  HPFP8_REQUIRE(aligned16(x) && aligned16(q), HPFP8_ERR_ALIGN, "%s: buffers must be 16-byte aligned", what);
+  HPFP8_REQUIRE((reinterpret_cast<uintptr_t>(sync) & 255u) == 0, HPFP8_ERR_ALIGN, "%s: sync must be 256-byte aligned", what);
   const int64_t nvec = (n >> 3) > 0 ? (n >> 3) : 1;
   const int64_t per_thread = (nvec + (int64_t)kFusedMaxBlocks * kFusedThreads - 1) / ((int64_t)kFusedMaxBlocks * kFusedThreads);
   const int vec = per_thread <= 1 ? 1 : (per_thread <= 2 ? 2 : (per_thread <= 4 ? 4 : 8));
@@ -1029,10 +1059,10 @@ int hpfp8_quantize_per_tensor_sync_bf16(const void* x, int64_t n, void* q, float
   uint8_t* q8 = (uint8_t*)q;
   hipStream_t s = (hipStream_t)stream;
   switch (vec) {
-    case 1: quant_per_tensor_fused_kernel<1, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
-    case 2: quant_per_tensor_fused_kernel<2, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
-    case 4: quant_per_tensor_fused_kernel<4, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
-    default: quant_per_tensor_fused_kernel<8, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 1, q8, scale, g_spin_limit, amax, scale_inv); break;
+    case 1: quant_per_tensor_fused_kernel<1, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
+    case 2: quant_per_tensor_fused_kernel<2, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
+    case 4: quant_per_tensor_fused_kernel<4, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
+    default: quant_per_tensor_fused_kernel<8, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
   }
   return check_launch(what);
 }

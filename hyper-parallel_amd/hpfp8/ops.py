@@ -108,7 +108,7 @@ def amax(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
-# 16 bytes per (device, stream) that hpfp8_quantize_per_tensor_sync_bf16's grid synchronises through: zero when
+# 512 bytes per (device, stream) that hpfp8_quantize_per_tensor_sync_bf16's grid synchronises through: zero when
 # created, and left zero by every call, so calls on one stream can share them
 _SYNC_WORDS = {}
 _ONE_PASS_MAX = 1 << 22
@@ -120,7 +120,7 @@ def _sync_words(device: torch.device) -> Optional[torch.Tensor]:
     if t is None:
         if torch.cuda.is_current_stream_capturing():
             return None          # (creating them would record a fill into the graph; the two-launch form needs none)
-        t = _SYNC_WORDS[key] = torch.zeros(4, dtype=torch.int32, device=device)
+        t = _SYNC_WORDS[key] = torch.zeros(128, dtype=torch.int32, device=device)
     return t
 
 

@@ -75,8 +75,8 @@ int hpfp8_cast_per_tensor_bf16(const void* x, int64_t n, const float* amax, void
 int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* amax, float* scale,
                                    float* scale_inv, hpfp8_stream_t stream);
 
-/* The same in ONE launch, for tensors of up to 4 Mi elements (more is HPFP8_ERR_SHAPE): `sync` points at 16 bytes of
- * device memory (16-byte aligned) that the caller keeps for this purpose, zero before the first call; every call
+/* The same in ONE launch, for tensors of up to 4 Mi elements (more is HPFP8_ERR_SHAPE): `sync` points at 512 bytes of
+ * device memory (256-byte aligned) that the caller keeps for this purpose, zero before the first call; every call
  * finds it zero and leaves it zero (the last workgroup to finish with it clears it), so calls that follow each other
  * on a stream -- or replays of a captured graph -- need nothing cleared in between.  Calls that may overlap on the
  * GPU need a `sync` of their own each.  amax, scale and scale_inv (each may be NULL) receive max |x| and the two

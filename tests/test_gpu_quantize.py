@@ -546,7 +546,7 @@ def test_per_tensor_single_launch_form_with_self_clearing_sync_words(gpu):
     from hpfp8 import _lib
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
-    sync = torch.zeros(4, dtype=torch.int32, device=gpu)
+    sync = torch.zeros(128, dtype=torch.int32, device=gpu)
     try:
         for limit in (1 << 22, 0):
             lib.hpfp8_debug_set_spin_limit(limit)
@@ -597,7 +597,7 @@ def test_per_tensor_single_launch_form_with_self_clearing_sync_words(gpu):
     big = torch.zeros(4 * 1024 * 1024 + 8, dtype=torch.bfloat16, device=gpu)
     qb = torch.empty(big.shape, dtype=torch.float8_e4m3fn, device=gpu)
     assert lib.hpfp8_quantize_per_tensor_sync_bf16(big.data_ptr(), big.numel(), qb.data_ptr(), None, None, og.data_ptr(), sync.data_ptr(), st) == -2
-    assert lib.hpfp8_quantize_per_tensor_sync_bf16(big.data_ptr(), 1024, qb.data_ptr(), None, None, og.data_ptr(), sync.data_ptr() + 4, st) == -3
+    assert lib.hpfp8_quantize_per_tensor_sync_bf16(big.data_ptr(), 1024, qb.data_ptr(), None, None, og.data_ptr(), sync.data_ptr() + 16, st) == -3
     assert lib.hpfp8_quantize_per_tensor_sync_bf16(big.data_ptr(), 1024, qb.data_ptr(), None, None, og.data_ptr(), None, st) == -1
 
 
