@@ -293,6 +293,53 @@ def other_configs_compact(dev):
     return res
 
 
+def board_power(fns, launches=1200):
+    """Mean board power (W), its cap (W) and the mean shader clock (MHz) while each callable runs `launches` times back
+    to back, read from the amdgpu driver's hwmon files of the card; {} when the files are not there."""
+    import glob
+    import threading
+    import torch
+    base = "/sys/class/drm/card*/device/hwmon/hwmon*/"
+    pw = sorted(glob.glob(base + "power1_input") or glob.glob(base + "power1_average"))[:1]
+    fq = sorted(glob.glob(base + "freq1_input"))[:1]
+    cap = sorted(glob.glob(base + "power1_cap"))[:1]
+    if not pw:
+        return {}
+
+    def read(path):
+        try:
+            return int(open(path).read().strip())
+        except (OSError, ValueError):
+            return None
+    out = {"cap_W": (read(cap[0]) or 0) / 1e6 if cap else None}
+    for name, fn in fns.items():
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                samples.append((read(pw[0]), read(fq[0]) if fq else None))
+                time.sleep(0.02)
+        th = threading.Thread(target=sampler)
+        th.start()
+        s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s0.record()
+        for _ in range(launches):
+            fn()
+        s1.record()
+        torch.cuda.synchronize()
+        stop.set()
+        th.join()
+        tail = samples[len(samples) // 4:]                      # (the first quarter: clocks and the sensor's average settling)
+        p_ = [a for a, _ in tail if a]
+        f_ = [b for _, b in tail if b]
+        out[name] = {"ms": s0.elapsed_time(s1) / launches, "board_W": sum(p_) / len(p_) / 1e6 if p_ else None,
+                     "sclk_MHz": sum(f_) / len(f_) / 1e6 if f_ else None, "samples": len(tail)}
+    return out
+
+
 def more_measurements(dev):
     """--all: what the layers around the benchmarked kernels cost (the dense-MLP block with its fused SwiGLU, a
     training step of cfg 2's layer), the optional power-of-two recipe, the vendor library's per-tensor GEMM for
@@ -382,6 +429,14 @@ def more_measurements(dev):
     except Exception as err:          # (absent or differently named in another torch build)
         orient["vendor_scaled_mm"] = f"unavailable: {type(err).__name__}"
     res["cfg2_shape_per_tensor_for_orientation"] = orient
+    # what the board draws and clocks at while these GEMMs run back to back (the driver's hwmon files, sampled from a
+    # host thread every 20 ms during about a second of launches each; absent files leave the entry empty)
+    power_fns = {"blockwise_gemm": lambda: hpfp8.gemm_blockwise(xq2_, sx2_, wf2_.codes, wf2_.scale_inv),
+                 "per_tensor_gemm": lambda: hpfp8.gemm_per_tensor(xq2_, one_, wf2_.codes, one_)}
+    if "vendor_scaled_mm" in orient:
+        power_fns["vendor_scaled_mm"] = lambda: torch._scaled_mm(xq2_, wf2_.codes.t(), scale_a=one_, scale_b=one_,
+                                                                 out_dtype=torch.bfloat16)
+    res["board_power_during_gemms"] = board_power(power_fns)
     del wf2_, xq2_, sx2_, xt_, wt_, got_, wf_
     torch.cuda.empty_cache()
     # cfg 3 under the optional recipe, and its weight gradient added onto an fp32 main gradient
