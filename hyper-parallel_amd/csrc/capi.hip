@@ -12,7 +12,7 @@ char* error_buffer() {
 
 extern "C" {
 
-int hpfp8_version(void) { return 400; }  // 0.4.0
+int hpfp8_version(void) { return 500; }  // 0.5.0
 
 const char* hpfp8_last_error(void) { return hpfp8::error_buffer(); }
 
