@@ -428,6 +428,14 @@ def more_measurements(dev):
                                                                             out_dtype=torch.bfloat16)))
     except Exception as err:          # (absent or differently named in another torch build)
         orient["vendor_scaled_mm"] = f"unavailable: {type(err).__name__}"
+    try:   # the vendor library's finest scaling on this stack: one scale per row of a and per row of b, applied at the end
+        ra_, rb_ = torch.ones((4096, 1), device=dev), torch.ones((1, 36864), device=dev)
+        orient["vendor_scaled_mm_rowwise"] = tf(fl2, _time(lambda: torch._scaled_mm(xq2_, wf2_.codes.t(), scale_a=ra_, scale_b=rb_,
+                                                                                    out_dtype=torch.bfloat16)))
+        torch._scaled_mm(xq2_, wf2_.codes.t(), scale_a=sx2_.contiguous(), scale_b=wf2_.scale_inv, out_dtype=torch.bfloat16)
+        orient["vendor_blockwise_1x128_128x128"] = "available"
+    except Exception as err:
+        orient["vendor_blockwise_1x128_128x128"] = f"unavailable: {str(err).splitlines()[0][:80]}"
     res["cfg2_shape_per_tensor_for_orientation"] = orient
     # what the board draws and clocks at while these GEMMs run back to back (the driver's hwmon files, sampled from a
     # host thread every 20 ms during about a second of launches each; absent files leave the entry empty)
