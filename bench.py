@@ -219,6 +219,19 @@ def other_configs_compact(dev):
                 lambda: ops.gemm_blockwise_swiglu_quantize(xq, sx, gu.codes, gu.scale_inv, fast=True), iters=20)),
             "block_forward": _tf(fl_mlp, _time(lambda: hpfp8.fp8_swiglu_mlp(x, gu, dn, fast=True), iters=20)),
         }
+    # for orientation, on the same codes: this library's block-scaled kernel beside the vendor library's FP8 GEMMs
+    # (one scale per tensor; one scale per row of each operand, its finest scaling here)
+    one = torch.ones((), dtype=torch.float32, device=dev)
+    orient = {"this_library_blockwise": _tf(fl_gu, _time(lambda: ops.gemm_blockwise(xq, sx, gu.codes, gu.scale_inv), iters=20))}
+    try:
+        orient["vendor_per_tensor"] = _tf(fl_gu, _time(lambda: torch._scaled_mm(
+            xq, gu.codes.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), iters=20))
+        ra, rb = torch.ones((4096, 1), device=dev), torch.ones((1, 36864), device=dev)
+        orient["vendor_rowwise"] = _tf(fl_gu, _time(lambda: torch._scaled_mm(
+            xq, gu.codes.t(), scale_a=ra, scale_b=rb, out_dtype=torch.bfloat16), iters=20))
+    except Exception as err:          # (absent or differently named in another torch build)
+        orient["vendor"] = f"unavailable: {type(err).__name__}"
+    res["cfg2_gemm_beside_vendor_library"] = orient
     del x, gu, dn, xq, sx
     torch.cuda.empty_cache()
     # cfg 3: o_proj backward, M = 4096 tokens, W[7168, 16384]
