@@ -71,6 +71,37 @@ def test_argument_errors_are_reported_without_launching():
     assert lib.hpfp8_gemm_per_tensor(None, 128, None, None, 128, None, 0, 128, 128, None, None, 128, 0, None) == 0
 
 
+def test_argument_errors_of_the_fused_and_one_launch_entry_points():
+    """The gate/up GEMM with the SwiGLU + quantizer epilogue, the fused SwiGLU-backward quantizer and the one-launch
+    per-tensor quantizer check their arguments before anything is launched."""
+    from hpfp8 import _lib
+    lib = _lib.load()
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.cast(buf, ctypes.c_void_p).value + 255) & ~255
+    ep = lib.hpfp8_gemm_blockwise_swiglu_quantize
+    # flags other than 0 / 1; a width that is not a multiple of 128; ldq below the width; null scale_inv
+    assert ep(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 128, 128, 2, 0, 0, p, 128, None, p, None) == -1
+    assert ep(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 100, 128, 0, 0, 0, p, 128, None, p, None) == -2
+    assert b"multiple of 128" in lib.hpfp8_last_error()
+    assert ep(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 256, 128, 0, 0, 0, p, 128, None, p, None) == -2
+    assert ep(p, 128, p, 1, 1, p, 128, p, 1, 1, 128, 128, 128, 0, 0, 0, p, 128, None, None, None) == -1
+    # a weight whose codes span 2 GiB or more cannot be addressed from one tile's buffer resource
+    assert ep(p, 1 << 14, p, 1, 1, p, 1 << 14, p, 1, 1, 128, 1 << 16, 1 << 14, 0, 0, 0, p, 1 << 16, None, p, None) == -2
+    assert b"2 GiB" in lib.hpfp8_last_error()
+    # empty problems succeed
+    assert ep(None, 128, None, 1, 1, None, 128, None, 1, 1, 0, 128, 128, 0, 0, 0, None, 128, None, None, None) == 0
+    bw = lib.hpfp8_swiglu_backward_quantize_1x128_and_128x1_t_bf16
+    assert bw(p, 100, 128, 256, p, p, None, p, p, 128, None, p, None) == -2          # rows not a multiple of 128
+    assert bw(p, 128, 128, 200, p, p, None, p, p, 128, None, p, None) == -2          # ld_h below twice the width
+    assert bw(p, 128, 128, 256, None, p, None, p, p, 128, None, p, None) == -1       # no dact
+    assert bw(p, 128, 128, 256, p, p, None, p, p, 64, None, p, None) == -2           # ld_t below the row count
+    sy = lib.hpfp8_quantize_per_tensor_sync_bf16
+    assert sy(p, (1 << 22) + 8, p, None, None, p, p, None) == -2 and b"one-pass" in lib.hpfp8_last_error()
+    assert sy(p, 1024, p, None, None, p, None, None) == -1
+    assert sy(p, 1024, p, None, None, p, p + 16, None) == -3
+    assert sy(p + 2, 1024, p, None, None, p, p, None) == -3
+
+
 def test_python_wrappers_reject_cpu_tensors_and_bad_shapes():
     import torch
     import hpfp8
