@@ -38,6 +38,14 @@ class Fp8Weight(NamedTuple):
     codes_t: Optional[torch.Tensor]     # e4m3 [K, N] (dgrad operand) or None
     pow2: bool = False                  # scales are powers of two ("blockwise_pow2")
 
+    def __repr__(self) -> str:
+        # Shapes and addresses, never element values: the reference's dispatcher makes its layout-cache key from
+        # str() of every non-tensor argument (hyper_parallel/core/shard/_op_dispatch.py:205-210, :226-231), and a
+        # tuple's default repr would print (and copy to the host) whole device tensors on every call.
+        def one(t):
+            return "None" if t is None else f"{tuple(t.shape)}@{t.data_ptr():#x}"
+        return f"Fp8Weight(codes={one(self.codes)}, scale_inv={one(self.scale_inv)}, codes_t={one(self.codes_t)}, pow2={self.pow2})"
+
 
 def quantize_weight(weight: torch.Tensor, with_transpose: bool = True, pow2: bool = False,
                     per_tensor: bool = False) -> Fp8Weight:
@@ -51,6 +59,21 @@ def quantize_weight(weight: torch.Tensor, with_transpose: bool = True, pow2: boo
         return Fp8Weight(wq, sw, wqt, pow2)
     wq, sw = ops.quantize_128x128(weight, pow2=pow2)
     return Fp8Weight(wq, sw, None, pow2)
+
+
+def _hand_off(func, tensors, args, kwargs, defaults):
+    """The `__torch_function__` protocol for a Python-level operator: when any tensor argument is of a subclass that
+    overrides `__torch_function__` (the reference's DTensor, hyper_parallel/platform/torch/dtensor.py:50-62), the
+    call is given to that hook with THIS function object as `func` -- the reference derives its registry key from
+    `func.__name__` (hyper_parallel/platform/torch/platform.py:159-174) and, after layout inference, calls the
+    function again on the local tensors (hyper_parallel/core/shard/_op_dispatch.py:277-283), where this returns
+    NotImplemented and the kernels run.  Keyword arguments still at their defaults are left out, so that a plain
+    call reaches the hook as (input, weight, bias) exactly like `torch.nn.functional.linear` does."""
+    if not torch.overrides.has_torch_function(tensors):
+        return NotImplemented
+    kw = {k: v for k, v in kwargs.items()
+          if not (v is defaults[k] or (isinstance(v, (str, bool)) and v == defaults[k]))}
+    return torch.overrides.handle_torch_function(func, tensors, *args, **kw)
 
 
 def _flatten(x: torch.Tensor):
@@ -236,6 +259,11 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     `weight.main_grad` instead of `weight.grad`: a float32 [out_features, in_features] tensor that the
     first backward creates and every later one adds onto, inside the wgrad GEMM.
     """
+    out = _hand_off(fp8_linear, tuple(t for t in (input, weight, bias) if t is not None), (input, weight, bias),
+                    dict(recipe=recipe, weight_fp8=weight_fp8, apply_grad_on_fp32_main_grad=apply_grad_on_fp32_main_grad),
+                    _FP8_LINEAR_DEFAULTS)
+    if out is not NotImplemented:
+        return out
     if recipe not in RECIPES:
         raise ValueError(f"recipe must be one of {RECIPES}, got {recipe!r}")
     if weight.dim() != 2:
@@ -270,6 +298,9 @@ def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
         return _Fp8LinearBlockwise.apply(input, weight, bias, None, None, None, apply_grad_on_fp32_main_grad, pow2,
                                          torch.is_grad_enabled())
     return _Fp8LinearPerTensor.apply(input, weight, bias)
+
+
+_FP8_LINEAR_DEFAULTS = dict(recipe="blockwise", weight_fp8=None, apply_grad_on_fp32_main_grad=False)
 
 
 def _init_like_nn_linear(weight: torch.Tensor, bias: Optional[torch.Tensor]) -> None:
@@ -458,6 +489,10 @@ def fp8_grouped_linear(input: torch.Tensor, weight: torch.Tensor, offs: torch.Te
     are left uninitialised, as torch's grouped matmul leaves them (their input gradient is zero).  Differentiable in
     input and weight (blockwise recipe); neither forward nor backward reads offs on the host.  ``weight_fp8`` is the
     weight's FP8 form made earlier by `quantize_grouped_weight` (e.g. once per optimizer step)."""
+    out = _hand_off(fp8_grouped_linear, (input, weight, offs), (input, weight, offs), dict(weight_fp8=weight_fp8),
+                    dict(weight_fp8=None))
+    if out is not NotImplemented:
+        return out
     if input.dim() != 2 or weight.dim() != 3 or input.shape[1] != weight.shape[2]:
         raise ValueError("input must be [total_m, K] and weight [E, N, K]")
     if input.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
@@ -593,6 +628,11 @@ def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True,
     weights' FP8 forms made earlier by `quantize_weight` (e.g. once per optimizer step for all its micro-batches),
     as `fp8_linear`'s ``weight_fp8``.  ``fast`` selects the SwiGLU kernel that uses the hardware exponential and
     reciprocal."""
+    out = _hand_off(fp8_swiglu_mlp, tuple(t for t in (input, w_gate_up, w_down) if isinstance(t, torch.Tensor)),
+                    (input, w_gate_up, w_down), dict(fast=fast, gate_up_fp8=gate_up_fp8, down_fp8=down_fp8),
+                    _FP8_MLP_DEFAULTS)
+    if out is not NotImplemented:
+        return out
     fp8_weights = isinstance(w_gate_up, Fp8Weight) or isinstance(w_down, Fp8Weight)
     if not fp8_weights and torch.is_grad_enabled() and (input.requires_grad or w_gate_up.requires_grad or w_down.requires_grad):
         if w_gate_up.shape[0] % (2 * ops.BLOCK) or w_down.shape[1] != w_gate_up.shape[0] // 2:
@@ -627,6 +667,9 @@ def fp8_swiglu_mlp(input: torch.Tensor, w_gate_up, w_down, *, fast: bool = True,
                                                     pow2_out=dn.pow2)
         y = ops.gemm_blockwise(aq, sa, dn.codes, dn.scale_inv, pow2_scales=dn.pow2)
     return y.reshape(input.shape[:-1] + (dn.codes.shape[0],))
+
+
+_FP8_MLP_DEFAULTS = dict(fast=True, gate_up_fp8=None, down_fp8=None)
 
 
 class Fp8SwiGLUMLP(nn.Module):

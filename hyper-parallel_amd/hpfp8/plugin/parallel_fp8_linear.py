@@ -37,9 +37,15 @@ class Fp8LinearDistributedOp(DistributedOp):
     """Distributed implementation for fp8_linear(input, weight, bias)."""
 
     def infer_layout(self, layouts, extra_args):
-        if len(layouts) != 3:
+        # (input, weight, bias) always arrive positionally; the dispatcher appends one entry per keyword argument
+        # (hyper_parallel/core/shard/_op_dispatch.py:224-241), and fp8_linear's keywords (recipe, weight_fp8,
+        # apply_grad_on_fp32_main_grad) are not tensors, so their entries carry no layout.
+        if len(layouts) < 3:
             raise ValueError(f"fp8_linear layout length is not 3, but {len(layouts)}")
-        x_layout, w_layout, bias_layout = layouts
+        if any(extra is not None for extra in layouts[3:]):
+            raise ValueError("fp8_linear takes three tensors (input, weight, bias); its keyword arguments are not "
+                             "distributed tensors")
+        x_layout, w_layout, bias_layout = layouts[:3]
         if not x_layout or not w_layout:
             raise ValueError(f"x_layout : {x_layout}, w_layout : {w_layout}")
         if x_layout.mesh_shape != w_layout.mesh_shape:
@@ -63,8 +69,8 @@ class Fp8LinearDistributedOp(DistributedOp):
         factor = bias_divisor(x_layout.alias_tensor_map, x_layout.mesh_shape, x_layout.alias_name)
         rescale = factor != 1 and bool(layouts[2])
 
-        def expand_impl(x, w, bias=None):
+        def expand_impl(x, w, bias=None, **kwargs):
             check_local_shapes(x, w)
-            return func(x, w, bias / factor if rescale and bias is not None else bias)
+            return func(x, w, bias / factor if rescale and bias is not None else bias, **kwargs)
 
         return expand_impl

@@ -9,10 +9,23 @@ They restate the interface the plugin touches, nothing more:
     `partial`.
   * `DistributedOp` -- hyper_parallel/core/shard/ops/parallel_ops.py:23-84: constructed with the operator name,
     which registers the instance; `infer_layout` / `get_expand_impl` are what subclasses override.
+  * `DTensor` and `Dispatcher` -- the route of one operator call: `DTensorBase.__torch_function__`
+    (hyper_parallel/platform/torch/dtensor.py:50-62) hands (func, args, kwargs) to `OpDispatcher.dispatch`
+    (hyper_parallel/core/shard/_op_dispatch.py:634-673): name = `func.__name__`
+    (hyper_parallel/platform/torch/platform.py:159-174); whitelisted names run on the unwrapped tensors; a name without
+    a registered rule raises RuntimeError; otherwise `_with_layout_infer` (:245-298, argument handling :190-243):
+    positional tensors with a layout are replaced by their local tensors, everything else goes to `extra_args`, every
+    keyword adds one (layout or None) entry, `infer_layout(layouts, extra_args)` gives the output layout,
+    `get_expand_impl(func, output_layout, layouts, extra_args)` an optional wrapper, the (wrapper or) function runs on
+    the local tensors and the result is wrapped with the output layout.  `layout_infer_ops` /
+    `_register_single_distributed_op` (:148-186) are the two members a late registration uses.
 """
 import copy
+import importlib
 import sys
 import types
+
+import torch
 
 REGISTRY = {}
 
@@ -73,6 +86,74 @@ class DistributedOp:
 
     def get_expand_impl(self, func, output_layout, layouts, extra_args):
         return None
+
+
+class DTensor(torch.Tensor):
+    """A local tensor plus a layout, whose operator calls all go to DISPATCHER (set by the test)."""
+    DISPATCHER = None
+
+    @staticmethod
+    def __new__(cls, local, layout):
+        t = torch.Tensor._make_subclass(cls, local, local.requires_grad)
+        t._local_tensor, t._layout = local, layout
+        return t
+
+    @property
+    def layout(self):
+        return self._layout
+
+    def to_local(self):
+        return self._local_tensor
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        return cls.DISPATCHER.dispatch(func, args, kwargs or {})
+
+
+class Dispatcher:
+    WHITELIST = ("__get__", "__set__", "dim", "__len__", "__bool__", "__format__", "item", "requires_grad_")
+
+    def __init__(self):
+        self.layout_infer_ops = {}
+        self.seen = []                                  # operator names in the order they arrived
+
+    def _register_single_distributed_op(self, op_name, config):
+        mod = importlib.import_module(config["distributed_op_module"] if "distributed_op_module" in config
+                                      else config["distributed_op_file"])
+        getattr(mod, config["distributed_op_class"])(op_name)
+
+    def dispatch(self, func, args, kwargs):
+        name = func.__name__ if hasattr(func, "__name__") else str(func)
+        self.seen.append(name)
+        if name in self.WHITELIST:
+            with torch._C.DisableTorchFunctionSubclass():
+                return func(*[a.to_local() if isinstance(a, DTensor) else a for a in args], **kwargs)
+        if name not in self.layout_infer_ops:
+            raise RuntimeError(f"Operator {name} dose not contain parallel layout infer func.")
+        layouts, extra, local_args, local_kwargs = [], [], [], dict(kwargs)
+        for a in args:
+            if a is None or not hasattr(a, "_layout"):
+                layouts.append(None)
+                local_args.append(a)
+                if a is not None:
+                    extra.append(a)
+                    str(a)                              # the reference's cache key prints every such argument
+            else:
+                layouts.append(a.layout)
+                local_args.append(a.to_local())
+        for k, v in kwargs.items():
+            if v is None or not hasattr(v, "_layout"):
+                layouts.append(None)
+                if v is not None:
+                    extra.append(v)
+                    str(v)
+            else:
+                layouts.append(v.layout)
+                local_kwargs[k] = v.to_local()
+        op = REGISTRY[name]
+        out_layout = op.infer_layout(layouts, extra)
+        impl = op.get_expand_impl(func, out_layout, layouts, extra) or func
+        return DTensor(impl(*local_args, **local_kwargs), out_layout)
 
 
 def install():
