@@ -555,84 +555,61 @@ __device__ __forceinline__ void store_tile_transposed(uint8_t* tile, const uint2
     const int pc = threadIdx.x & 7;
     const int chunk = pc ^ ((col >> 3) & 7);
     uint4 o = *reinterpret_cast<const uint4*>(&tile[col * 128 + pc * 16]);
-    *reinterpret_cast<uint4*>(dst + (int64_t)col * ld + chunk * 16) = o;
+    nt_store16(reinterpret_cast<char*>(dst) + ((uint32_t)col * (uint32_t)ld + (uint32_t)chunk * 16u), o);
   }
 }
 
 // ---------------------------------------------------------------------------------------------
 // 128x128 blocks (weights), optional transposed copy of the codes for dgrad
 // ---------------------------------------------------------------------------------------------
-// Tiles a workgroup of the transposing kernels walks through (down a tile column, prefetching the
-// next tile's loads).  Measured on MI355X: 1 is fastest (42 us vs 44.5 us at 4 for x[4096,16384]); more
-// resident workgroups hide latency better than the in-workgroup prefetch does.
-constexpr int kTilesPerBlock = 1;
-
+// One 128x128 tile per workgroup (several tiles per workgroup with the next tile's loads issued ahead were measured
+// and were slower: more resident workgroups hide latency better).  The grid is two-dimensional with x the fast index:
+// along_k = 1 walks along a tile row of the source, 0 down a tile column (see transpose_grid).
 template <bool WITH_T>
 __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __restrict__ w, int rows,
                                                             int cols, uint8_t* __restrict__ q,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale,
-                                                            float* __restrict__ scale_inv, int pow2) {
-  const int cb = cols >> 7, rb = rows >> 7;
+                                                            float* __restrict__ scale_inv, int pow2, int along_k) {
+  const int cb = cols >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   __shared__ uint32_t part[16];
   __shared__ float s_scale;
   __shared__ __attribute__((aligned(16))) uint8_t tile[WITH_T ? 128 * 128 : 16];
-  // Without a transposed copy: one tile per workgroup, row-major tile order.  With it: a workgroup
-  // walks kTilesPerBlock tiles down a block column, loading tile t+1 before the LDS phases of tile
-  // t, and its consecutive 128-byte pieces of each transposed row are neighbours in memory.
-  const int total = rb * cb;
-  const int t0 = WITH_T ? blockIdx.x * kTilesPerBlock : blockIdx.x;
-  const int t1 = WITH_T ? (t0 + kTilesPerBlock < total ? t0 + kTilesPerBlock : total) : t0 + 1;
-  auto tile_pos = [&](int t, int& br, int& bc) {
-    if (WITH_T) { bc = t / rb; br = t % rb; } else { bc = t % cb; br = t / cb; }
-  };
-  auto load_tile = [&](int t, uint4 v[8]) {
-    int br, bc;
-    tile_pos(t, br, bc);
-    const int64_t off = (int64_t)br * 128 * cols + bc * 128 + cg * 8;
+  const int br = along_k ? blockIdx.y : blockIdx.x, bc = along_k ? blockIdx.x : blockIdx.y;
+  // a tile's first element is a uniform 64-bit address, positions inside the tile are 32-bit byte offsets
+  const char* wbase = reinterpret_cast<const char*>(w + (int64_t)br * 128 * cols + bc * 128);
+  char* qbase = reinterpret_cast<char*>(q + (int64_t)br * 128 * cols + bc * 128);
+  const uint32_t ucols = (uint32_t)cols;
+  uint4 v[8];
 #pragma unroll
-    for (int p = 0; p < 8; ++p) v[p] = nt_load16(w + off + (int64_t)tile_row(rq, p) * cols);
-  };
-  uint4 v[8], vn[8];
-  load_tile(t0, v);
-  for (int t = t0; t < t1; ++t) {
-    if (WITH_T && t + 1 < t1) load_tile(t + 1, vn);
-    int br, bc;
-    tile_pos(t, br, bc);
-    const int sidx = br * cb + bc;
-    const int64_t tile_off = (int64_t)br * 128 * cols + bc * 128 + cg * 8;
-    uint32_t m = 0;
+  for (int p = 0; p < 8; ++p) v[p] = nt_load16(wbase + ((uint32_t)tile_row(rq, p) * ucols + (uint32_t)cg * 8u) * 2u);
+  const int sidx = br * cb + bc;
+  uint32_t m = 0;
 #pragma unroll
-    for (int p = 0; p < 8; ++p) m = umax(m, mag8(v[p]));
-    m = row16_max_u32(m);
-    if (cg == 0) part[rq] = m;
-    __syncthreads();
-    if (threadIdx.x < 16) {
-      m = row16_max_u32(part[threadIdx.x]);
-      if (threadIdx.x == 0) {
-        float s, si;
-        scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
-        s_scale = s;
-        if (scale) scale[sidx] = s;
-        scale_inv[sidx] = si;
-      }
-    }
-    __syncthreads();
-    const float s = s_scale;
-    uint2 c[8];
-#pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      c[p] = cvt8<false>(v[p], s);
-      *reinterpret_cast<uint2*>(q + tile_off + (int64_t)tile_row(rq, p) * cols) = c[p];
-    }
-    if (WITH_T) {
-      store_tile_transposed(tile, c, cg, rq, qt + (int64_t)bc * 128 * ld_t + br * 128, ld_t);
-      __syncthreads();   // the LDS tile, part[] and s_scale are reused by the next tile
-#pragma unroll
-      for (int p = 0; p < 8; ++p) v[p] = vn[p];
+  for (int p = 0; p < 8; ++p) m = umax(m, mag8(v[p]));
+  m = row16_max_u32(m);
+  if (cg == 0) part[rq] = m;
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    m = row16_max_u32(part[threadIdx.x]);
+    if (threadIdx.x == 0) {
+      float s, si;
+      scales_from_amax(__uint_as_float(m << 16), s, si, pow2);
+      s_scale = s;
+      if (scale) scale[sidx] = s;
+      scale_inv[sidx] = si;
     }
   }
+  __syncthreads();
+  const float s = s_scale;
+  uint2 c[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    c[p] = cvt8<false>(v[p], s);
+    nt_store8(qbase + ((uint32_t)tile_row(rq, p) * ucols + (uint32_t)cg * 8u), c[p]);
+  }
+  if (WITH_T) store_tile_transposed(tile, c, cg, rq, qt + (int64_t)bc * 128 * ld_t + br * 128, ld_t);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -655,16 +632,22 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // filled up with zero codes past the expert's last row; m is then the number of source rows (any count), mb the
 // number of padded blocks the grid covers, and blocks beyond those in use are left untouched.  The 1x128 form
 // (DUAL) is written for the rows that exist, at their own positions.
+// Tile order.  The grid is two-dimensional, x the fast index: with `along_k` = 0 consecutive workgroups walk down a
+// tile column of the source (tile row fastest: neighbours in x write neighbouring 128-byte pieces of the same
+// transposed rows), with 1 along a tile row (tile column fastest: neighbours read neighbouring 256-byte pieces of the
+// same source rows).  Which of the two is faster depends on the source's row stride: with a stride that is a multiple
+// of 16 KB the 128 rows of a tile column fall on few memory channels, and only the second order keeps all of them busy.
+// All address arithmetic per thread is 32-bit: a tile's first element is a uniform 64-bit pointer, a thread's position
+// inside the tile an unsigned byte offset (a tile spans less than 4 GB: row strides below 2^24 elements).
 template <bool KMAJOR, bool DUAL, int SW = 0, bool GROUPED = false>
 __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int m, int k,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale_t,
                                                             float* __restrict__ scale_inv_t,
                                                             uint8_t* __restrict__ q, float* __restrict__ scale_r,
-                                                            float* __restrict__ scale_inv_r, int pow2,
+                                                            float* __restrict__ scale_inv_r, int pow2, int along_k = 0,
                                                             const int32_t* __restrict__ layout = nullptr, int experts = 0,
                                                             int padded_blocks = 0, const uint16_t* __restrict__ dact = nullptr) {
-  static_assert(!GROUPED || (SW == 0 && kTilesPerBlock == 1), "grouped form: plain source, one tile per workgroup");
   const int kb = k >> 7, mb = GROUPED ? padded_blocks : m >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   const int wave = threadIdx.x >> 6;
@@ -672,15 +655,10 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
   __shared__ float s_scale[128];
   __shared__ float s_row[DUAL ? 256 : 2];   // scale, scale_inv of the tile's 128 rows
   __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
-  // A workgroup walks kTilesPerBlock tiles down a tile column (tr fastest), loading tile t+1 before
-  // the LDS phases of tile t.
-  const int total = kb * mb;
-  const int t0 = blockIdx.x * kTilesPerBlock;
-  const int t1 = t0 + kTilesPerBlock < total ? t0 + kTilesPerBlock : total;
+  const int tr = along_k ? blockIdx.y : blockIdx.x, tc = along_k ? blockIdx.x : blockIdx.y;
   // first source row of the tile and how many of its 128 rows exist (dense: tr * 128 and all of them)
-  int g_row0 = 0, g_valid = 128;
+  int g_row0 = tr * 128, g_valid = 128;
   if (GROUPED) {
-    const int tr = t0 % mb;
     const int e = layout[5 * experts + 1 + tr];
     if (e < 0) return;                                   // (uniform over the workgroup) a block no expert owns
     const int j = tr - layout[4 * e + 2];
@@ -688,143 +666,133 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
     g_valid = layout[4 * e + 1] - j * 128;
     g_valid = g_valid < 0 ? 0 : (g_valid > 128 ? 128 : g_valid);
   }
-  auto load_tile = [&](int t, uint4 v[8]) {
-    const int tc = t / mb, tr = t % mb;
-    if (SW == 3) {
-      // tile columns [0, inter) are d gate (from gate, up and d act), [inter, 2 inter) are d up (from gate and d act)
-      const int inter = k >> 1;
-      const bool is_gate = tc * 128 < inter;
-      const int c0 = tc * 128 - (is_gate ? 0 : inter) + cg * 8;     // column inside the gate / up half and inside d act
+  // byte offset of this thread's first element inside the source tile, and the row stride in bytes
+  const uint32_t ld_b = (uint32_t)ld_src * 2u;
+  const uint32_t t_off = (uint32_t)(4 * rq) * ld_b + (uint32_t)cg * 16u;
+  auto row_off = [&](int p) -> uint32_t { return t_off + (uint32_t)((p >> 2) * 64 + (p & 3)) * ld_b; };
+  uint4 v[8];
+  if (SW == 3) {
+    // tile columns [0, inter) are d gate (from gate, up and d act), [inter, 2 inter) are d up (from gate and d act)
+    const int inter = k >> 1;
+    const bool is_gate = tc * 128 < inter;
+    const int c0 = tc * 128 - (is_gate ? 0 : inter);                    // first column inside the gate / up half and inside d act
+    const char* gbase = reinterpret_cast<const char*>(x + (int64_t)g_row0 * ld_src + c0);
+    const char* dbase = reinterpret_cast<const char*>(dact + (int64_t)g_row0 * inter + c0);
+    const uint32_t ldd_b = (uint32_t)inter * 2u;
+    const uint32_t d_off = (uint32_t)(4 * rq) * ldd_b + (uint32_t)cg * 16u;
 #pragma unroll
-      for (int p = 0; p < 8; ++p) {
-        const int64_t row = (int64_t)tr * 128 + tile_row(rq, p);
-        const uint4 gv = nt_load16(x + row * ld_src + c0);
-        const uint4 dv = nt_load16(dact + row * inter + c0);
-        uint32_t unused;
-        if (is_gate) {
-          const uint4 uv = nt_load16(x + row * ld_src + inter + c0);
-          swiglu_bwd2(gv.x, uv.x, dv.x, v[p].x, unused);
-          swiglu_bwd2(gv.y, uv.y, dv.y, v[p].y, unused);
-          swiglu_bwd2(gv.z, uv.z, dv.z, v[p].z, unused);
-          swiglu_bwd2(gv.w, uv.w, dv.w, v[p].w, unused);
-        } else {
-          swiglu_bwd2(gv.x, 0u, dv.x, unused, v[p].x);
-          swiglu_bwd2(gv.y, 0u, dv.y, unused, v[p].y);
-          swiglu_bwd2(gv.z, 0u, dv.z, unused, v[p].z);
-          swiglu_bwd2(gv.w, 0u, dv.w, unused, v[p].w);
-        }
+    for (int p = 0; p < 8; ++p) {
+      const uint4 gv = nt_load16(gbase + row_off(p));
+      const uint4 dv = nt_load16(dbase + d_off + (uint32_t)((p >> 2) * 64 + (p & 3)) * ldd_b);
+      uint32_t unused;
+      if (is_gate) {
+        const uint4 uv = nt_load16(gbase + (uint32_t)inter * 2u + row_off(p));
+        swiglu_bwd2(gv.x, uv.x, dv.x, v[p].x, unused);
+        swiglu_bwd2(gv.y, uv.y, dv.y, v[p].y, unused);
+        swiglu_bwd2(gv.z, uv.z, dv.z, v[p].z, unused);
+        swiglu_bwd2(gv.w, uv.w, dv.w, v[p].w, unused);
+      } else {
+        swiglu_bwd2(gv.x, 0u, dv.x, unused, v[p].x);
+        swiglu_bwd2(gv.y, 0u, dv.y, unused, v[p].y);
+        swiglu_bwd2(gv.z, 0u, dv.z, unused, v[p].z);
+        swiglu_bwd2(gv.w, 0u, dv.w, unused, v[p].w);
       }
-      return;
     }
-    const int64_t off = (int64_t)(GROUPED ? g_row0 : tr * 128) * ld_src + tc * 128 + cg * 8;
+  } else {
+    const char* sbase = reinterpret_cast<const char*>(x + (int64_t)g_row0 * ld_src + tc * 128);
 #pragma unroll
     for (int p = 0; p < 8; ++p)
-      v[p] = (!GROUPED || tile_row(rq, p) < g_valid) ? nt_load16(x + off + (int64_t)tile_row(rq, p) * ld_src)
-                                                     : make_uint4(0, 0, 0, 0);
+      v[p] = (!GROUPED || tile_row(rq, p) < g_valid) ? nt_load16(sbase + row_off(p)) : make_uint4(0, 0, 0, 0);
     if (SW) {
 #pragma unroll
       for (int p = 0; p < 8; ++p) {
-        const uint4 u = nt_load16(x + off + (int64_t)tile_row(rq, p) * ld_src + k);
+        const uint4 u = nt_load16(sbase + (uint32_t)k * 2u + row_off(p));
         v[p].x = swiglu2<SW == 2>(v[p].x, u.x);
         v[p].y = swiglu2<SW == 2>(v[p].y, u.y);
         v[p].z = swiglu2<SW == 2>(v[p].z, u.z);
         v[p].w = swiglu2<SW == 2>(v[p].w, u.w);
       }
     }
-  };
-  uint4 v[8], vn[8];
-  load_tile(t0, v);
-  for (int t = t0; t < t1; ++t) {
-    if (t + 1 < t1) load_tile(t + 1, vn);
-    const int tc = t / mb, tr = t % mb;
-    // per-column magnitudes over this thread's 8 rows, two columns per word
-    uint32_t cm[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      cm[0] = pk_max_u16(cm[0], v[p].x & 0x7FFF7FFFu);
-      cm[1] = pk_max_u16(cm[1], v[p].y & 0x7FFF7FFFu);
-      cm[2] = pk_max_u16(cm[2], v[p].z & 0x7FFF7FFFu);
-      cm[3] = pk_max_u16(cm[3], v[p].w & 0x7FFF7FFFu);
-    }
-    // across the 4 row quads inside the wave (lanes differing in bits 4 and 5)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 16));
-      cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 32));
-    }
-    if ((threadIdx.x & 63) < 16) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) part[wave][cg * 4 + i] = cm[i];
-    }
-    if (DUAL) {
-      // the 16 threads of a row quad hold a whole 128-column group of each of their 8 rows
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        uint32_t mr[4];
-#pragma unroll
-        for (int p = 0; p < 4; ++p) mr[p] = row16_max_u32(mag8(v[4 * half + p]));
-        float s[4], mine, mine_inv;
-        scales4_from_amax(mr, cg, pow2, s, mine, mine_inv);
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          const int row = tile_row(rq, 4 * half + p);
-          if (!GROUPED || row < g_valid)
-            *reinterpret_cast<uint2*>(q + ((int64_t)(GROUPED ? g_row0 : tr * 128) + row) * k + tc * 128 + cg * 8) =
-                cvt8<false>(v[4 * half + p], s[p]);
-        }
-        if (cg < 4) {
-          const int row = tile_row(rq, 4 * half + cg);
-          s_row[row] = mine;
-          s_row[128 + row] = mine_inv;
-        }
-      }
-    }
-    __syncthreads();
-    if (DUAL && threadIdx.x >= 128) {
-      const int row = threadIdx.x - 128;
-      const int64_t r_abs = (int64_t)(GROUPED ? g_row0 : tr * 128) + row;
-      const int64_t o = KMAJOR ? (int64_t)tc * m + r_abs : r_abs * kb + tc;
-      if (!GROUPED || row < g_valid) {
-        if (scale_r) scale_r[o] = s_row[row];
-        scale_inv_r[o] = s_row[128 + row];
-      }
-    }
-    if (threadIdx.x < 128) {
-      const int col = threadIdx.x, word = col >> 1;
-      uint32_t mw = pk_max_u16(pk_max_u16(part[0][word], part[1][word]), pk_max_u16(part[2][word], part[3][word]));
-      uint32_t mag = (col & 1) ? (mw >> 16) : (mw & 0xFFFFu);
-      float s, si;
-      scales_from_amax(__uint_as_float(mag << 16), s, si, pow2);
-      s_scale[col] = s;
-      // row-major [k, m/128], or block-major [m/128, k] (unit stride over the output rows)
-      int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
-      if (scale_t) scale_t[o] = s;
-      scale_inv_t[o] = si;
-    }
-    __syncthreads();
-    float sc[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) sc[j] = s_scale[cg * 8 + j];
-    uint2 c[8];
-#pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const uint32_t ws[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
-      uint32_t pk[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        // scale from this very column's amax: the clamp to +-448 would be a no-op (see cvt2)
-        float a = bf16lo(ws[i]) * sc[2 * i];
-        float b = bf16hi(ws[i]) * sc[2 * i + 1];
-        pk[i] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
-      }
-      c[p].x = pk[0] | (pk[1] << 16);
-      c[p].y = pk[2] | (pk[3] << 16);
-    }
-    store_tile_transposed(tile, c, cg, rq, qt + (int64_t)tc * 128 * ld_t + tr * 128, ld_t);
-    __syncthreads();   // the LDS tile, part[] and s_scale are reused by the next tile
-#pragma unroll
-    for (int p = 0; p < 8; ++p) v[p] = vn[p];
   }
+  // per-column magnitudes over this thread's 8 rows, two columns per word
+  uint32_t cm[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    cm[0] = pk_max_u16(cm[0], v[p].x & 0x7FFF7FFFu);
+    cm[1] = pk_max_u16(cm[1], v[p].y & 0x7FFF7FFFu);
+    cm[2] = pk_max_u16(cm[2], v[p].z & 0x7FFF7FFFu);
+    cm[3] = pk_max_u16(cm[3], v[p].w & 0x7FFF7FFFu);
+  }
+  // across the 4 row quads inside the wave (lanes differing in bits 4 and 5)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 16));
+    cm[i] = pk_max_u16(cm[i], (uint32_t)__shfl_xor((int)cm[i], 32));
+  }
+  if ((threadIdx.x & 63) < 16)
+    *reinterpret_cast<uint4*>(&part[wave][cg * 4]) = make_uint4(cm[0], cm[1], cm[2], cm[3]);
+  if (DUAL) {
+    // the 16 threads of a row quad hold a whole 128-column group of each of their 8 rows
+    char* qbase = reinterpret_cast<char*>(q + (int64_t)g_row0 * k + tc * 128);
+    const uint32_t q_off = (uint32_t)(4 * rq) * (uint32_t)k + (uint32_t)cg * 8u;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint32_t mr[4];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) mr[p] = row16_max_u32(mag8(v[4 * half + p]));
+      float s[4], mine, mine_inv;
+      scales4_from_amax(mr, cg, pow2, s, mine, mine_inv);
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int row = tile_row(rq, 4 * half + p);
+        if (!GROUPED || row < g_valid)
+          nt_store8(qbase + q_off + (uint32_t)(half * 64 + p) * (uint32_t)k, cvt8<false>(v[4 * half + p], s[p]));
+      }
+      if (cg < 4) {
+        const int row = tile_row(rq, 4 * half + cg);
+        s_row[row] = mine;
+        s_row[128 + row] = mine_inv;
+      }
+    }
+  }
+  __syncthreads();
+  if (DUAL && threadIdx.x >= 128) {
+    const int row = threadIdx.x - 128;
+    const int64_t r_abs = (int64_t)g_row0 + row;
+    const int64_t o = KMAJOR ? (int64_t)tc * m + r_abs : r_abs * kb + tc;
+    if (!GROUPED || row < g_valid) {
+      if (scale_r) scale_r[o] = s_row[row];
+      scale_inv_r[o] = s_row[128 + row];
+    }
+  }
+  if (threadIdx.x < 128) {
+    const int col = threadIdx.x, word = col >> 1;
+    uint32_t mw = pk_max_u16(pk_max_u16(part[0][word], part[1][word]), pk_max_u16(part[2][word], part[3][word]));
+    uint32_t mag = (col & 1) ? (mw >> 16) : (mw & 0xFFFFu);
+    float s, si;
+    scales_from_amax(__uint_as_float(mag << 16), s, si, pow2);
+    s_scale[col] = s;
+    // row-major [k, m/128], or block-major [m/128, k] (unit stride over the output rows)
+    int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
+    if (scale_t) scale_t[o] = s;
+    scale_inv_t[o] = si;
+  }
+  __syncthreads();
+  const float4 sa = *reinterpret_cast<const float4*>(&s_scale[cg * 8]), sb = *reinterpret_cast<const float4*>(&s_scale[cg * 8 + 4]);
+  const float sc[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w};
+  uint2 c[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    // scale from this very column's amax: the clamp to +-448 would be a no-op (see cvt2)
+    const uint32_t ws[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
+    uint32_t lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[0]) * sc[0], bf16hi(ws[0]) * sc[1], 0, false);
+    lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[1]) * sc[2], bf16hi(ws[1]) * sc[3], (int)lo, true);
+    uint32_t hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[2]) * sc[4], bf16hi(ws[2]) * sc[5], 0, false);
+    hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[3]) * sc[6], bf16hi(ws[3]) * sc[7], (int)hi, true);
+    c[p].x = lo;
+    c[p].y = hi;
+  }
+  store_tile_transposed(tile, c, cg, rq, qt + (int64_t)tc * 128 * ld_t + tr * 128, ld_t);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -833,16 +801,16 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
 // 128x128 blocks are symmetric, so the transposed codes of a weight (dgrad operand) can be made
 // from its codes alone, e.g. after the codes of all shards were gathered; no requantization.
 __global__ __launch_bounds__(256) void transpose_codes_kernel(const uint8_t* __restrict__ q, int rows, int cols,
-                                                              int64_t ld, uint8_t* __restrict__ qt, int64_t ld_t) {
-  const int rb = rows >> 7;
+                                                              int64_t ld, uint8_t* __restrict__ qt, int64_t ld_t, int along_k) {
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
-  const int bc = blockIdx.x / rb, br = blockIdx.x % rb;
-  const uint8_t* src = q + (int64_t)br * 128 * ld + bc * 128 + cg * 8;
+  const int br = along_k ? blockIdx.y : blockIdx.x, bc = along_k ? blockIdx.x : blockIdx.y;
+  const char* src = reinterpret_cast<const char*>(q + (int64_t)br * 128 * ld + bc * 128);
   uint2 c[8];
 #pragma unroll
   for (int p = 0; p < 8; ++p) {
-    const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src + (int64_t)tile_row(rq, p) * ld));
+    const u32x2 t = __builtin_nontemporal_load(
+        reinterpret_cast<const u32x2*>(src + ((uint32_t)tile_row(rq, p) * (uint32_t)ld + (uint32_t)cg * 8u)));
     c[p] = make_uint2(t.x, t.y);
   }
   store_tile_transposed(tile, c, cg, rq, qt + (int64_t)bc * 128 * ld_t + br * 128, ld_t);
@@ -1130,6 +1098,22 @@ int hpfp8_quantize_1x128_kmajor_pow2_bf16(const void* x, int64_t rows, int64_t c
   return quantize_1x128_kmajor_impl(x, rows, cols, q, scale, scale_inv, 1, stream);
 }
 
+// Grid of the transposing tile kernels: x is the fast index.  along_k = 1 makes consecutive workgroups walk along a
+// tile row of the source, 0 down a tile column (which keeps the 128-byte pieces of one transposed row together).
+// Measured on MI355X with buffers rotating beyond the Infinity Cache: down a tile column is the faster order unless
+// the source's row stride puts a tile column's 128 rows on few memory channels -- a stride that is a multiple of
+// 16 KB for a kernel with one output stream, of 4 KB for one that also writes the row-major codes (`streams` = 2:
+// x[4096, 16384] both forms 56.6 -> 62.1 % of 8 TB/s, x[4096, 8192] transposed form 53.3 -> 60.3 %, while
+// x[16384, 7168], stride 14 KB, loses 7 points the other way round).  streams = 0 never walks along k (the byte
+// transpose, measured faster down the column at every stride).  A grid's y extent is limited to 65535, so a matrix
+// with more tiles than that in one direction keeps that direction in x.
+static dim3 transpose_grid(int64_t mb, int64_t kb, int64_t ld_src_bytes, int streams, int& along_k) {
+  along_k = streams == 0 ? 0 : (ld_src_bytes % (streams >= 2 ? 4096 : 16384) == 0 ? 1 : 0);
+  if (along_k && mb > 65535) along_k = 0;
+  if (!along_k && kb > 65535) along_k = 1;
+  return along_k ? dim3((unsigned)kb, (unsigned)mb) : dim3((unsigned)mb, (unsigned)kb);
+}
+
 static int quantize_128x128_impl(const void* w, int64_t rows, int64_t cols, void* q, void* q_t, int64_t ld_t,
                                  float* scale, float* scale_inv, int pow2, hpfp8_stream_t stream) {
   HPFP8_REQUIRE(rows >= 0 && cols >= 0, HPFP8_ERR_SHAPE, "quantize_128x128: negative shape");
@@ -1142,15 +1126,24 @@ static int quantize_128x128_impl(const void* w, int64_t rows, int64_t cols, void
   HPFP8_REQUIRE(w && q && scale_inv, HPFP8_ERR_ARG, "quantize_128x128: null buffer");
   HPFP8_REQUIRE(aligned16(w) && aligned16(q) && (!q_t || aligned16(q_t)), HPFP8_ERR_ALIGN,
                 "quantize_128x128: buffers must be 16-byte aligned");
+  HPFP8_REQUIRE(cols < (1 << 24) && (!q_t || ld_t < (1 << 24)), HPFP8_ERR_SHAPE,
+                "quantize_128x128: cols and ld_t must be below 2^24");
   HPFP8_REQUIRE(!q_t || (ld_t >= rows && ld_t % 16 == 0), HPFP8_ERR_SHAPE,
                 "quantize_128x128: ld_t=%lld must be a multiple of 16 and at least rows", (long long)ld_t);
   hipStream_t s = (hipStream_t)stream;
-  if (q_t)
-    quant_128x128_kernel<true><<<(unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock), 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
-                                                                (uint8_t*)q, (uint8_t*)q_t, ld_t, scale, scale_inv, pow2);
-  else
-    quant_128x128_kernel<false><<<(unsigned)blocks, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols,
-                                                                 (uint8_t*)q, nullptr, 0, scale, scale_inv, pow2);
+  int ak = 1;
+  if (q_t) {
+    const dim3 grid = transpose_grid(rows / kBlock, cols / kBlock, cols * 2, 2, ak);
+    quant_128x128_kernel<true><<<grid, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols, (uint8_t*)q, (uint8_t*)q_t, ld_t,
+                                                    scale, scale_inv, pow2, ak);
+  } else {
+    // no transposed copy: always along the source rows (a plain streaming order)
+    const bool x_is_cols = cols / kBlock <= 65535 || rows / kBlock > 65535;
+    ak = x_is_cols ? 1 : 0;
+    const dim3 grid = ak ? dim3((unsigned)(cols / kBlock), (unsigned)(rows / kBlock)) : dim3((unsigned)(rows / kBlock), (unsigned)(cols / kBlock));
+    quant_128x128_kernel<false><<<grid, 256, 0, s>>>((const uint16_t*)w, (int)rows, (int)cols, (uint8_t*)q, nullptr, 0, scale,
+                                                     scale_inv, pow2, ak);
+  }
   return check_launch("quantize_128x128");
 }
 
@@ -1171,7 +1164,8 @@ static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, i
   HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)m, (long long)k);
-  HPFP8_REQUIRE(m < (1 << 30) && k < (1 << 30), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
+  HPFP8_REQUIRE(m < (1 << 30) && k < (1 << 24) && ld_t < (1 << 24), HPFP8_ERR_SHAPE,
+                "%s: dimension too large (at most 2^30 rows, and columns and ld_t below 2^24)", what);
   const int64_t blocks = (m / kBlock) * (k / kBlock);
   if (blocks == 0) return HPFP8_OK;
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
@@ -1181,20 +1175,21 @@ static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, i
                 what, (long long)ld_t);
   HPFP8_REQUIRE(!q || (scale_inv && aligned16(q)), HPFP8_ERR_ARG, "%s: q needs scale_inv and 16-byte alignment", what);
   hipStream_t s = (hipStream_t)stream;
-  const unsigned grid = (unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock);
+  int ak = 0;
+  const dim3 grid = transpose_grid(m / kBlock, k / kBlock, k * 2, q ? 2 : 1, ak);
   const uint16_t* xs = (const uint16_t*)x;
   uint8_t* qt8 = (uint8_t*)q_t;
   uint8_t* q8 = (uint8_t*)q;
   if (q) {
     if (kmajor)
-      quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
+      quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2, ak);
     else
-      quant_128x1_t_kernel<false, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2);
+      quant_128x1_t_kernel<false, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2, ak);
   } else {
     if (kmajor)
-      quant_128x1_t_kernel<true, false><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
+      quant_128x1_t_kernel<true, false><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2, ak);
     else
-      quant_128x1_t_kernel<false, false><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2);
+      quant_128x1_t_kernel<false, false><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr, nullptr, nullptr, pow2, ak);
   }
   return check_launch(what);
 }
@@ -1206,7 +1201,8 @@ int hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, in
   HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(rows % kBlock == 0 && inter % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)rows, (long long)inter);
-  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 30), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
+  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 24) && ld_h < (1 << 24) && ld_t < (1 << 24), HPFP8_ERR_SHAPE,
+                "%s: dimension too large (at most 2^30 rows; width and row strides below 2^24)", what);
   const int64_t blocks = (rows / kBlock) * (inter / kBlock);
   if (blocks == 0) return HPFP8_OK;
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
@@ -1217,13 +1213,14 @@ int hpfp8_swiglu_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t rows, in
   HPFP8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, HPFP8_ERR_SHAPE, "%s: ld_t=%lld must be a multiple of 16 and at least rows",
                 what, (long long)ld_t);
   hipStream_t s = (hipStream_t)stream;
-  const unsigned grid = (unsigned)((blocks + kTilesPerBlock - 1) / kTilesPerBlock);
+  int ak = 0;
+  const dim3 grid = transpose_grid(rows / kBlock, inter / kBlock, ld_h * 2, 2, ak);
   if (fast)
     quant_128x1_t_kernel<true, true, 2><<<grid, 256, 0, s>>>((const uint16_t*)h, ld_h, (int)rows, (int)inter, (uint8_t*)q_t, ld_t,
-                                                            scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0);
+                                                            scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0, ak);
   else
     quant_128x1_t_kernel<true, true, 1><<<grid, 256, 0, s>>>((const uint16_t*)h, ld_h, (int)rows, (int)inter, (uint8_t*)q_t, ld_t,
-                                                            scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0);
+                                                            scale_t, scale_inv_t, (uint8_t*)q, scale, scale_inv, 0, ak);
   return check_launch(what);
 }
 
@@ -1235,7 +1232,8 @@ int hpfp8_swiglu_backward_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t
   HPFP8_REQUIRE(rows >= 0 && inter >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(rows % kBlock == 0 && inter % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)rows, (long long)inter);
-  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 29), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
+  HPFP8_REQUIRE(rows < (1 << 30) && inter < (1 << 23) && ld_h < (1 << 24) && ld_t < (1 << 24), HPFP8_ERR_SHAPE,
+                "%s: dimension too large (at most 2^30 rows; width and row strides below 2^24)", what);
   const int64_t blocks = (rows / kBlock) * (2 * inter / kBlock);
   if (blocks == 0) return HPFP8_OK;
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "%s: tensor too large", what);
@@ -1246,9 +1244,11 @@ int hpfp8_swiglu_backward_quantize_1x128_and_128x1_t_bf16(const void* h, int64_t
                 "%s: ld_h=%lld must be a multiple of 8 and at least twice the width", what, (long long)ld_h);
   HPFP8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, HPFP8_ERR_SHAPE, "%s: ld_t=%lld must be a multiple of 16 and at least rows",
                 what, (long long)ld_t);
-  quant_128x1_t_kernel<true, true, 3><<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+  int ak = 0;
+  const dim3 grid = transpose_grid(rows / kBlock, 2 * inter / kBlock, ld_h * 2, 2, ak);
+  quant_128x1_t_kernel<true, true, 3><<<grid, 256, 0, (hipStream_t)stream>>>(
       (const uint16_t*)h, ld_h, (int)rows, (int)(2 * inter), (uint8_t*)q_t, ld_t, scale_t, scale_inv_t, (uint8_t*)q, scale,
-      scale_inv, 0, nullptr, 0, 0, (const uint16_t*)dact);
+      scale_inv, 0, ak, nullptr, 0, 0, (const uint16_t*)dact);
   return check_launch(what);
 }
 
@@ -1259,7 +1259,8 @@ int hpfp8_quantize_128x1_t_grouped_bf16(const void* x, int64_t total_m, int64_t 
   HPFP8_REQUIRE(total_m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(k % kBlock == 0, HPFP8_ERR_SHAPE, "%s: width %lld is not a multiple of 128", what, (long long)k);
   HPFP8_REQUIRE(experts >= 0 && experts <= 4096, HPFP8_ERR_SHAPE, "%s: bad expert count %d", what, experts);
-  HPFP8_REQUIRE(total_m < (1 << 30) && k < (1 << 30), HPFP8_ERR_SHAPE, "%s: dimension too large", what);
+  HPFP8_REQUIRE(total_m < (1 << 30) && k < (1 << 24) && ld_t < (1 << 24), HPFP8_ERR_SHAPE,
+                "%s: dimension too large (at most 2^30 rows; width and ld_t below 2^24)", what);
   const int64_t padded_blocks = total_m / kBlock + experts;
   const int64_t blocks = padded_blocks * (k / kBlock);
   if (blocks == 0) return HPFP8_OK;
@@ -1271,14 +1272,16 @@ int hpfp8_quantize_128x1_t_grouped_bf16(const void* x, int64_t total_m, int64_t 
                 (long long)(padded_blocks * kBlock));
   HPFP8_REQUIRE(!q || (scale_inv && aligned16(q)), HPFP8_ERR_ARG, "%s: q needs scale_inv and 16-byte alignment", what);
   hipStream_t s = (hipStream_t)stream;
+  int ak = 0;
+  const dim3 grid = transpose_grid(padded_blocks, k / kBlock, k * 2, q ? 2 : 1, ak);
   if (q)
-    quant_128x1_t_kernel<true, true, 0, true><<<(unsigned)blocks, 256, 0, s>>>(
+    quant_128x1_t_kernel<true, true, 0, true><<<grid, 256, 0, s>>>(
         (const uint16_t*)x, k, (int)total_m, (int)k, (uint8_t*)q_t, ld_t, nullptr, scale_inv_t, (uint8_t*)q, nullptr, scale_inv, 0,
-        layout, experts, (int)padded_blocks);
+        ak, layout, experts, (int)padded_blocks);
   else
-    quant_128x1_t_kernel<true, false, 0, true><<<(unsigned)blocks, 256, 0, s>>>(
+    quant_128x1_t_kernel<true, false, 0, true><<<grid, 256, 0, s>>>(
         (const uint16_t*)x, k, (int)total_m, (int)k, (uint8_t*)q_t, ld_t, nullptr, scale_inv_t, nullptr, nullptr, nullptr, 0,
-        layout, experts, (int)padded_blocks);
+        ak, layout, experts, (int)padded_blocks);
   return check_launch(what);
 }
 
@@ -1388,11 +1391,14 @@ int hpfp8_transpose_codes(const void* q, int64_t rows, int64_t cols, int64_t ld,
   HPFP8_REQUIRE(blocks <= 0x7FFFFFFF, HPFP8_ERR_SHAPE, "transpose_codes: tensor too large");
   HPFP8_REQUIRE(q && q_t, HPFP8_ERR_ARG, "transpose_codes: null buffer");
   HPFP8_REQUIRE(aligned16(q) && aligned16(q_t), HPFP8_ERR_ALIGN, "transpose_codes: buffers must be 16-byte aligned");
+  HPFP8_REQUIRE(ld_t < (1 << 24) && ld < (1 << 24), HPFP8_ERR_SHAPE, "transpose_codes: ld and ld_t must be below 2^24");
   HPFP8_REQUIRE(ld >= cols && ld % 16 == 0 && ld_t >= rows && ld_t % 16 == 0, HPFP8_ERR_SHAPE,
                 "transpose_codes: ld=%lld / ld_t=%lld must be multiples of 16 and at least cols / rows", (long long)ld,
                 (long long)ld_t);
-  transpose_codes_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, (int)rows, (int)cols, ld,
-                                                                           (uint8_t*)q_t, ld_t);
+  int ak = 0;
+  const dim3 grid = transpose_grid(rows / kBlock, cols / kBlock, ld, 0, ak);
+  transpose_codes_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, (int)rows, (int)cols, ld, (uint8_t*)q_t,
+                                                                 ld_t, ak);
   return check_launch("transpose_codes");
 }
 
