@@ -27,6 +27,7 @@
 //     along the rows (MoE forward and dgrad: an expert owns a range of rows of a and c and its own b), or
 //     grouped along the contraction (MoE wgrad: an expert owns a range of k-blocks of both operands and
 //     its own c); bf16 or fp32 output, optionally added onto what c holds.
+#include <atomic>
 #include <type_traits>
 
 #include "hpfp8_device.h"
@@ -1048,7 +1049,7 @@ __global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmPar
 
 // 0: the small-tile kernel serves problems with fewer 256 x 256 tiles than half the compute units (and more
 // 128 x 128 tiles than that); 1: never; 2: whenever its forms allow (test hook)
-static int g_small_gemm_mode = 0;
+static std::atomic<int> g_small_gemm_mode{0};   // (atomic: the test hook may be called from any thread)
 
 // Workgroups to launch for `tiles` tiles: one per CU, a multiple of 8 (one share per XCD) unless
 // there are fewer than 8 tiles.
@@ -1066,8 +1067,9 @@ static int persistent_grid(int64_t tiles) {
 }
 
 static bool use_small_kernel(int64_t M, int64_t N) {
-  if (g_small_gemm_mode == 1) return false;
-  if (g_small_gemm_mode == 2) return true;
+  const int mode = g_small_gemm_mode.load(std::memory_order_relaxed);
+  if (mode == 1) return false;
+  if (mode == 2) return true;
   const int64_t big = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   const int64_t small = ((M + kSmallTile - 1) / kSmallTile) * (N / kSmallTile);
   const int cus = persistent_grid((int64_t)1 << 40);
@@ -1254,7 +1256,7 @@ int hpfp8_gemm_blockwise_swiglu_quantize(const void* a, int64_t lda, const float
   return check_launch(what);
 }
 
-void hpfp8_debug_set_small_gemm(int mode) { g_small_gemm_mode = mode == 1 || mode == 2 ? mode : 0; }
+void hpfp8_debug_set_small_gemm(int mode) { g_small_gemm_mode.store(mode == 1 || mode == 2 ? mode : 0, std::memory_order_relaxed); }
 
 int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const void* b, int64_t ldb,
                           const float* sb_inv, int64_t M, int64_t N, int64_t K, const void* bias, void* c,

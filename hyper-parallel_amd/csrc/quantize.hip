@@ -4,6 +4,7 @@
 // 16-bit integers (exact for bf16), amax reduced across lanes with DPP, scale = 448/amax by a
 // full IEEE division, E4M3 conversion with the hardware packed converter after an explicit
 // clamp to +-448, 64/128-bit stores.
+#include <atomic>
 #include <mutex>
 
 #include "hpfp8_device.h"
@@ -143,9 +144,12 @@ __global__ __launch_bounds__(256) void cast_per_tensor_kernel(const uint16_t* __
 // wait ended.  A workgroup that arrives only after scale_inv has been stored (possible only after such a
 // time-out) finds a count above the grid size: its own + 1 has disturbed the stored value, and it stores the value
 // again at its end (the amax word is final by then: the store is ordered after the maximum that justified it).
-// The grid is at most 64 workgroups of 1024 threads (they are always resident together on a chip of 256 CUs):
-// few and large, because every arrival is an atomic on one word, and those serialise across the chip at tens of
-// nanoseconds each (256 arrivals cost more than the second pass they save).
+// The grid is at most 64 workgroups of 1024 threads: few and large, because every arrival is an atomic on one word,
+// and those serialise across the chip at tens of nanoseconds each (256 arrivals cost more than the second pass
+// they save).  On an otherwise idle chip of 256 CUs they are resident together and the wait is a few polls; when
+// they are not (a persistent kernel of another stream holds the CUs, or the device is a partition with fewer CUs than
+// the grid has workgroups) the bounded wait below runs out and the workgroups fall back to the solo maximum, with
+// the same bits.
 constexpr int kFusedMaxBlocks = 64;
 constexpr int kFusedThreads = 1024;
 constexpr int kFusedMaxVec = 8;
@@ -287,8 +291,11 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
 
 // (SYNC3: the `seen > grid` repair of the two-word form cannot occur -- every workgroup arrives exactly once
 // between two clearings.)
-// Polls a waiting workgroup makes before it stops relying on the others (about a microsecond each).
-static uint32_t g_spin_limit = 1u << 22;
+// Polls a waiting workgroup makes before it stops relying on the others (about a microsecond each): a few hundred
+// microseconds at most, two orders of magnitude above what a resident grid needs.  The fallback gives the same
+// bits, so a short wait loses nothing but time in the rare case.  (Atomic: the test hook below may be called from
+// any thread.)
+static std::atomic<uint32_t> g_spin_limit{1u << 8};
 
 // Launches fill + fused kernel; the two words (device, 4 bytes each: amax, and scale_inv as the count) are zeroed
 // first by a kernel (not a memset node, so the sequence can be captured in a graph).  n in (0, kFusedMaxElems].
@@ -302,10 +309,10 @@ static int launch_per_tensor_fused(const void* x, int64_t n, void* q, uint32_t* 
   const uint16_t* xs = (const uint16_t*)x;
   uint8_t* q8 = (uint8_t*)q;
   switch (vec) {
-    case 1: quant_per_tensor_fused_kernel<1><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
-    case 2: quant_per_tensor_fused_kernel<2><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
-    case 4: quant_per_tensor_fused_kernel<4><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
-    default: quant_per_tensor_fused_kernel<8><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit); break;
+    case 1: quant_per_tensor_fused_kernel<1><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit.load(std::memory_order_relaxed)); break;
+    case 2: quant_per_tensor_fused_kernel<2><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit.load(std::memory_order_relaxed)); break;
+    case 4: quant_per_tensor_fused_kernel<4><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit.load(std::memory_order_relaxed)); break;
+    default: quant_per_tensor_fused_kernel<8><<<grid, kFusedThreads, 0, s>>>(xs, n, word, reinterpret_cast<uint32_t*>(scale_inv), q8, scale, g_spin_limit.load(std::memory_order_relaxed)); break;
   }
   return check_launch("quantize_per_tensor");
 }
@@ -639,7 +646,39 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // of 16 KB the 128 rows of a tile column fall on few memory channels, and only the second order keeps all of them busy.
 // All address arithmetic per thread is 32-bit: a tile's first element is a uniform 64-bit pointer, a thread's position
 // inside the tile an unsigned byte offset (a tile spans less than 4 GB: row strides below 2^24 elements).
-template <bool KMAJOR, bool DUAL, int SW = 0, bool GROUPED = false>
+// Column sums of a 128x128 bf16 tile in fp32, in a fixed order (so that a CPU restatement gives the same bits): a
+// thread adds its 8 rows onto +0 in load-slot order (tile rows 4rq, 4rq+1, 4rq+2, 4rq+3, then the same + 64); the
+// four row quads of a wave combine as (q0 + q1) + (q2 + q3); cs[i] then holds, in the wave's first 16 lanes (all of
+// them, in fact), the wave's sum for column cg * 8 + i, which goes to s_cs[wave][column].  After a workgroup barrier
+// column_sum_of_tile() adds the four waves in order.
+__device__ __forceinline__ void tile_column_sums(const uint4 v[8], int cg, int wave, float (*s_cs)[128]) {
+  float cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const uint32_t ws[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      cs[2 * i] += bf16lo(ws[i]);
+      cs[2 * i + 1] += bf16hi(ws[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    cs[i] += __shfl_xor(cs[i], 16);
+    cs[i] += __shfl_xor(cs[i], 32);
+  }
+  if ((threadIdx.x & 63) < 16) {
+    *reinterpret_cast<float4*>(&s_cs[wave][cg * 8]) = make_float4(cs[0], cs[1], cs[2], cs[3]);
+    *reinterpret_cast<float4*>(&s_cs[wave][cg * 8 + 4]) = make_float4(cs[4], cs[5], cs[6], cs[7]);
+  }
+}
+__device__ __forceinline__ float column_sum_of_tile(const float (*s_cs)[128], int col) {
+  return ((s_cs[0][col] + s_cs[1][col]) + s_cs[2][col]) + s_cs[3][col];
+}
+
+// With COLSUM the kernel also writes colsum_part[tr * k + column] = the fp32 sum of the tile's 128 rows per column
+// (tile_column_sums): the per-block partial sums of a bias gradient, from the same read of grad_out.
+template <bool KMAJOR, bool DUAL, int SW = 0, bool GROUPED = false, bool COLSUM = false>
 __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int m, int k,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale_t,
@@ -647,13 +686,16 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
                                                             uint8_t* __restrict__ q, float* __restrict__ scale_r,
                                                             float* __restrict__ scale_inv_r, int pow2, int along_k = 0,
                                                             const int32_t* __restrict__ layout = nullptr, int experts = 0,
-                                                            int padded_blocks = 0, const uint16_t* __restrict__ dact = nullptr) {
+                                                            int padded_blocks = 0, const uint16_t* __restrict__ dact = nullptr,
+                                                            float* __restrict__ colsum_part = nullptr) {
+  static_assert(!COLSUM || (SW == 0 && !GROUPED), "column sums: plain dense source only");
   const int kb = k >> 7, mb = GROUPED ? padded_blocks : m >> 7;
   const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
   const int wave = threadIdx.x >> 6;
   __shared__ uint32_t part[4][64];  // [wave][cg*4 + word]
   __shared__ float s_scale[128];
   __shared__ float s_row[DUAL ? 256 : 2];   // scale, scale_inv of the tile's 128 rows
+  __shared__ __attribute__((aligned(16))) float s_cs[COLSUM ? 4 : 1][128];
   __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
   const int tr = along_k ? blockIdx.y : blockIdx.x, tc = along_k ? blockIdx.x : blockIdx.y;
   // first source row of the tile and how many of its 128 rows exist (dense: tr * 128 and all of them)
@@ -714,6 +756,7 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
       }
     }
   }
+  if (COLSUM) tile_column_sums(v, cg, wave, s_cs);
   // per-column magnitudes over this thread's 8 rows, two columns per word
   uint32_t cm[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -776,6 +819,7 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
     int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
     if (scale_t) scale_t[o] = s;
     scale_inv_t[o] = si;
+    if (COLSUM) colsum_part[(int64_t)tr * k + tc * 128 + col] = column_sum_of_tile(s_cs, col);
   }
   __syncthreads();
   const float4 sa = *reinterpret_cast<const float4*>(&s_scale[cg * 8]), sb = *reinterpret_cast<const float4*>(&s_scale[cg * 8 + 4]);
@@ -793,6 +837,39 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
     c[p].y = hi;
   }
   store_tile_transposed(tile, c, cg, rq, qt + (int64_t)tc * 128 * ld_t + tr * 128, ld_t);
+}
+
+// ---------------------------------------------------------------------------------------------
+// column sums (bias gradient): x[m, k] bf16 -> per 128-row block partial sums fp32 [ceil(m/128), k] -> bf16 / fp32 [k]
+// ---------------------------------------------------------------------------------------------
+// The same tiles, the same order of additions as the COLSUM form of quant_128x1_t_kernel (rows past m count as +0),
+// for the callers that do not run that kernel on grad_out.  k a multiple of 128, any m.
+__global__ __launch_bounds__(256) void column_sum_partial_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int m, int k,
+                                                                 float* __restrict__ colsum_part) {
+  const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4, wave = threadIdx.x >> 6;
+  const int tr = blockIdx.x, tc = blockIdx.y;
+  __shared__ __attribute__((aligned(16))) float s_cs[4][128];
+  const int valid = m - tr * 128;                       // rows of this block that exist (>= 1)
+  const char* sbase = reinterpret_cast<const char*>(x + (int64_t)tr * 128 * ld_src + tc * 128);
+  const uint32_t ld_b = (uint32_t)ld_src * 2u;
+  uint4 v[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p)
+    v[p] = tile_row(rq, p) < valid ? nt_load16(sbase + ((uint32_t)tile_row(rq, p) * ld_b + (uint32_t)cg * 16u)) : make_uint4(0, 0, 0, 0);
+  tile_column_sums(v, cg, wave, s_cs);
+  __syncthreads();
+  if (threadIdx.x < 128) colsum_part[(int64_t)tr * k + tc * 128 + threadIdx.x] = column_sum_of_tile(s_cs, threadIdx.x);
+}
+
+// out[col] = ((0 + part[0][col]) + part[1][col]) + ... in block order, as fp32 and / or rounded once to bf16
+__global__ __launch_bounds__(256) void column_sum_finish_kernel(const float* __restrict__ part, int blocks, int k,
+                                                                uint16_t* __restrict__ out_bf16, float* __restrict__ out_f32) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col >= k) return;
+  float s = 0.f;
+  for (int b = 0; b < blocks; ++b) s += part[(int64_t)b * k + col];
+  if (out_f32) out_f32[col] = s;
+  if (out_bf16) out_bf16[col] = __builtin_bit_cast(uint16_t, (__bf16)s);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1007,7 +1084,7 @@ int hpfp8_quantize_per_tensor_bf16(const void* x, int64_t n, void* q, float* ama
   return hpfp8_cast_per_tensor_bf16(x, n, amax, q, scale, scale_inv, stream);
 }
 
-void hpfp8_debug_set_spin_limit(uint32_t polls) { g_spin_limit = polls; }
+void hpfp8_debug_set_spin_limit(uint32_t polls) { g_spin_limit.store(polls, std::memory_order_relaxed); }
 
 int hpfp8_quantize_per_tensor_sync_bf16(const void* x, int64_t n, void* q, float* amax, float* scale, float* scale_inv,
                                         uint32_t* sync, hpfp8_stream_t stream) {
@@ -1027,10 +1104,10 @@ int hpfp8_quantize_per_tensor_sync_bf16(const void* x, int64_t n, void* q, float
   uint8_t* q8 = (uint8_t*)q;
   hipStream_t s = (hipStream_t)stream;
   switch (vec) {
-    case 1: quant_per_tensor_fused_kernel<1, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
-    case 2: quant_per_tensor_fused_kernel<2, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
-    case 4: quant_per_tensor_fused_kernel<4, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
-    default: quant_per_tensor_fused_kernel<8, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit, amax, scale_inv); break;
+    case 1: quant_per_tensor_fused_kernel<1, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit.load(std::memory_order_relaxed), amax, scale_inv); break;
+    case 2: quant_per_tensor_fused_kernel<2, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit.load(std::memory_order_relaxed), amax, scale_inv); break;
+    case 4: quant_per_tensor_fused_kernel<4, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit.load(std::memory_order_relaxed), amax, scale_inv); break;
+    default: quant_per_tensor_fused_kernel<8, true><<<grid, kFusedThreads, 0, s>>>(xs, n, sync, sync + 64, q8, scale, g_spin_limit.load(std::memory_order_relaxed), amax, scale_inv); break;
   }
   return check_launch(what);
 }
@@ -1160,7 +1237,8 @@ int hpfp8_quantize_128x128_pow2_bf16(const void* w, int64_t rows, int64_t cols, 
 // q != nullptr: also the 1x128 quantization of x itself (codes q, scales scale / scale_inv).
 static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, int64_t m, int64_t k, void* q_t,
                                  int64_t ld_t, float* scale_t, float* scale_inv_t, hpfp8_stream_t stream,
-                                 void* q = nullptr, float* scale = nullptr, float* scale_inv = nullptr, int pow2 = 0) {
+                                 void* q = nullptr, float* scale = nullptr, float* scale_inv = nullptr, int pow2 = 0,
+                                 float* colsum_part = nullptr) {
   HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "%s: negative shape", what);
   HPFP8_REQUIRE(m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE,
                 "%s: shape [%lld, %lld] is not a multiple of 128", what, (long long)m, (long long)k);
@@ -1180,7 +1258,15 @@ static int quantize_128x1_t_impl(const char* what, bool kmajor, const void* x, i
   const uint16_t* xs = (const uint16_t*)x;
   uint8_t* qt8 = (uint8_t*)q_t;
   uint8_t* q8 = (uint8_t*)q;
-  if (q) {
+  if (colsum_part) {
+    HPFP8_REQUIRE(kmajor, HPFP8_ERR_ARG, "%s: the column sums come with the k-block-major scale layout only", what);
+    if (q)
+      quant_128x1_t_kernel<true, true, 0, false, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8,
+                                                                            scale, scale_inv, pow2, ak, nullptr, 0, 0, nullptr, colsum_part);
+    else
+      quant_128x1_t_kernel<true, false, 0, false, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, nullptr,
+                                                                             nullptr, nullptr, pow2, ak, nullptr, 0, 0, nullptr, colsum_part);
+  } else if (q) {
     if (kmajor)
       quant_128x1_t_kernel<true, true><<<grid, 256, 0, s>>>(xs, k, (int)m, (int)k, qt8, ld_t, scale_t, scale_inv_t, q8, scale, scale_inv, pow2, ak);
     else
@@ -1301,6 +1387,45 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
   HPFP8_REQUIRE(m == 0 || k == 0 || q != nullptr, HPFP8_ERR_ARG, "quantize_1x128_and_128x1_t: null buffer");
   return quantize_128x1_t_impl("quantize_1x128_and_128x1_t", kmajor != 0, x, m, k, q_t, ld_t, scale_t, scale_inv_t,
                                stream, q, scale, scale_inv);
+}
+
+int hpfp8_quantize_128x1_t_colsum_bf16(const void* x, int64_t m, int64_t k, void* q, float* scale, float* scale_inv, void* q_t,
+                                       int64_t ld_t, float* scale_t, float* scale_inv_t, int pow2, float* colsum_partial,
+                                       hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(m == 0 || k == 0 || colsum_partial != nullptr, HPFP8_ERR_ARG, "quantize_128x1_t_colsum: null buffer");
+  return quantize_128x1_t_impl("quantize_128x1_t_colsum", true, x, m, k, q_t, ld_t, scale_t, scale_inv_t, stream, q, scale,
+                               scale_inv, pow2 ? 1 : 0, colsum_partial);
+}
+
+int hpfp8_column_sum_finish(const float* partial, int64_t blocks, int64_t cols, void* out_bf16, float* out_f32,
+                            hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(blocks >= 0 && cols >= 0 && blocks < (1 << 30) && cols < (1 << 30), HPFP8_ERR_SHAPE, "column_sum_finish: bad shape");
+  if (cols == 0) return HPFP8_OK;
+  HPFP8_REQUIRE((partial || blocks == 0) && (out_bf16 || out_f32), HPFP8_ERR_ARG, "column_sum_finish: null buffer");
+  column_sum_finish_kernel<<<(unsigned)((cols + 255) / 256), 256, 0, (hipStream_t)stream>>>(partial, (int)blocks, (int)cols,
+                                                                                          (uint16_t*)out_bf16, out_f32);
+  return check_launch("column_sum_finish");
+}
+
+int hpfp8_column_sum_bf16(const void* x, int64_t m, int64_t k, int64_t ld, float* partial, void* out_bf16, float* out_f32,
+                          hpfp8_stream_t stream) {
+  HPFP8_REQUIRE(m >= 0 && k >= 0, HPFP8_ERR_SHAPE, "column_sum: negative shape");
+  HPFP8_REQUIRE(k % kBlock == 0, HPFP8_ERR_SHAPE, "column_sum: width %lld is not a multiple of 128", (long long)k);
+  HPFP8_REQUIRE(m < (1 << 30) && k < (1 << 23) && ld < (1 << 24), HPFP8_ERR_SHAPE, "column_sum: dimension too large");
+  if (k == 0) return HPFP8_OK;
+  const int64_t blocks = (m + kBlock - 1) / kBlock;
+  HPFP8_REQUIRE(out_bf16 || out_f32, HPFP8_ERR_ARG, "column_sum: null output");
+  if (blocks > 0) {
+    HPFP8_REQUIRE(x && partial, HPFP8_ERR_ARG, "column_sum: null buffer");
+    HPFP8_REQUIRE(aligned16(x) && ld >= k && ld % 8 == 0, HPFP8_ERR_ALIGN,
+                  "column_sum: x must be 16-byte aligned with a row stride that is a multiple of 8 and at least k");
+    HPFP8_REQUIRE(k / kBlock <= 65535, HPFP8_ERR_SHAPE, "column_sum: width too large");
+    column_sum_partial_kernel<<<dim3((unsigned)blocks, (unsigned)(k / kBlock)), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)x, ld, (int)m, (int)k, partial);
+    const int rc = check_launch("column_sum");
+    if (rc != HPFP8_OK) return rc;
+  }
+  return hpfp8_column_sum_finish(partial, blocks, k, out_bf16, out_f32, stream);
 }
 
 int hpfp8_quantize_128x1_t_kmajor_pow2_bf16(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t,

@@ -154,12 +154,17 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
         dx = dw = db = None
         goq = sgo = got = sgot = None
         if need_dx and need_dw and not ragged:
-            goq, sgo, got, sgot = ops.quantize_1x128_and_128x1_t(go, kmajor=True, pow2=pow2)   # one read of grad_out
+            if ctx.has_bias:                   # one read of grad_out: both operand forms and the bias gradient
+                goq, sgo, got, sgot, db = ops.quantize_1x128_and_128x1_t(go, kmajor=True, pow2=pow2, column_sum=True)
+            else:
+                goq, sgo, got, sgot = ops.quantize_1x128_and_128x1_t(go, kmajor=True, pow2=pow2)
         else:
             if need_dx:
                 goq, sgo = ops.quantize_1x128(go, kmajor=True, pow2=pow2)
             if need_dw:
                 got, sgot = ops.quantize_128x1_t(_pad_rows(go), kmajor=True, pow2=pow2)
+            if ctx.has_bias:
+                db = ops.column_sum(go)
         if need_dx:
             # dx[M,K] = go[M,N] . W[N,K]: contraction over N, b operand = W^T codes [K,N] whose
             # 128x128 scales are W's with the two strides swapped.
@@ -179,8 +184,6 @@ class _Fp8LinearBlockwise(torch.autograd.Function):
                                                      pow2_scales=pow2)
             else:
                 ops.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=param.main_grad, accumulate=True, pow2_scales=pow2)
-        if ctx.has_bias:
-            db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
         return dx, dw, db, None, None, None, None, None, None
 
 
@@ -236,7 +239,7 @@ class _Fp8LinearPerTensor(torch.autograd.Function):
                 xtq, _, sxt = ops.quantize_per_tensor(_pad_rows(x2).t().contiguous())
                 dw = ops.gemm_per_tensor(gotq, sgot, xtq, sxt)
         if ctx.has_bias:
-            db = go.sum(dim=0, dtype=torch.float32).to(torch.bfloat16)
+            db = ops.column_sum(go)
         return dx, dw, db, None, None
 
 
@@ -364,11 +367,13 @@ def attach_optimizer(optimizer: torch.optim.Optimizer, module: nn.Module):
 class Fp8Linear(nn.Module):
     """Drop-in for torch.nn.Linear (bf16 parameters) whose matmuls run through fp8_linear.
 
-    With ``cache_weight`` (the default) the weight's FP8 form is kept between calls; see `_Fp8WeightCache` for when
-    it is refreshed by itself and when `invalidate_fp8_cache()` must be called."""
+    By default the weight is quantized in every call, which is always right.  ``cache_weight=True`` keeps the
+    weight's FP8 form between calls (the micro-batches of one optimizer step, inference): an opt-in, because some
+    writes to a parameter cannot be seen from here -- see `_Fp8WeightCache` for when the cached form is refreshed by
+    itself and when `invalidate_fp8_cache()` must be called."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, *, recipe: str = "blockwise",
-                 cache_weight: bool = True, apply_grad_on_fp32_main_grad: bool = False, device=None,
+                 cache_weight: bool = False, apply_grad_on_fp32_main_grad: bool = False, device=None,
                  dtype=torch.bfloat16):
         super().__init__()
         self.cache_weight = cache_weight
@@ -674,15 +679,18 @@ _FP8_MLP_DEFAULTS = dict(fast=True, gate_up_fp8=None, down_fp8=None)
 
 class Fp8SwiGLUMLP(nn.Module):
     """A SwiGLU MLP block with bf16 parameters ``gate_up_proj.weight`` [2 * intermediate, hidden] (gate rows
-    first) and ``down_proj.weight`` [hidden, intermediate], computed by `fp8_swiglu_mlp`.  Like `Fp8Linear` it
-    keeps the FP8 forms of its weights until a parameter is written again, so the micro-batches of one optimizer
-    step and inference calls quantize them once."""
+    first) and ``down_proj.weight`` [hidden, intermediate], computed by `fp8_swiglu_mlp`.  With
+    ``cache_weight=True`` it keeps, like `Fp8Linear`, the FP8 forms of its weights until a parameter is written
+    again, so the micro-batches of one optimizer step and inference calls quantize them once (the same opt-in
+    and the same contract: `_Fp8WeightCache`)."""
 
-    def __init__(self, hidden_size: int, intermediate_size: int, *, fast: bool = True, device=None, dtype=torch.bfloat16):
+    def __init__(self, hidden_size: int, intermediate_size: int, *, fast: bool = True, cache_weight: bool = False,
+                 device=None, dtype=torch.bfloat16):
         super().__init__()
         if hidden_size % ops.BLOCK or intermediate_size % ops.BLOCK:
             raise ValueError("hidden_size and intermediate_size must be multiples of 128")
         self.hidden_size, self.intermediate_size, self.fast = hidden_size, intermediate_size, fast
+        self.cache_weight = cache_weight
         self.gate_up_proj = nn.Linear(hidden_size, 2 * intermediate_size, bias=False, device=device, dtype=dtype)
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False, device=device, dtype=dtype)
         self._cache = _Fp8WeightCache(2)
@@ -701,6 +709,8 @@ class Fp8SwiGLUMLP(nn.Module):
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         wgu, wd = self.gate_up_proj.weight, self.down_proj.weight
+        if not self.cache_weight:
+            return fp8_swiglu_mlp(input, wgu, wd, fast=self.fast)
         return fp8_swiglu_mlp(input, wgu, wd, fast=self.fast, gate_up_fp8=self._weight_fp8(0, wgu),
                               down_fp8=self._weight_fp8(1, wd))
 

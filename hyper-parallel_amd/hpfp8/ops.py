@@ -115,11 +115,18 @@ _ONE_PASS_MAX = 1 << 22
 
 
 def _sync_words(device: torch.device) -> Optional[torch.Tensor]:
+    """The 512-byte block through which the one-launch per-tensor quantizer's grid agrees on the maximum, one per
+    (device, stream).  Sharing rule: the block must be zero at launch (the kernel leaves it zero) and two launches
+    must never use it at once.  Eager calls on one stream are ordered by the stream, so they may share it.  A
+    captured graph is different: it would bake the block's address in, and a replay on another stream could then run
+    beside an eager call (or another graph) that uses the same block -- both would write the same slots and the
+    maximum would be silently wrong.  So nothing that is being captured gets the block: under capture the
+    two-launch form runs, whose only scratch is the caller-visible amax word allocated per call."""
+    if torch.cuda.is_current_stream_capturing():
+        return None
     key = (device.index if device.index is not None else torch.cuda.current_device(), _stream())
     t = _SYNC_WORDS.get(key)
     if t is None:
-        if torch.cuda.is_current_stream_capturing():
-            return None          # (creating them would record a fill into the graph; the two-launch form needs none)
         t = _SYNC_WORDS[key] = torch.zeros(128, dtype=torch.int32, device=device)
     return t
 
@@ -358,11 +365,13 @@ def quantize_128x1_t_rows(x: torch.Tensor):
     return qt, scale_inv.t()
 
 
-def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True, pow2: bool = False):
+def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True, pow2: bool = False, column_sum: bool = False):
     """Both operand forms of x[M, K] from one read of it.
 
     Returns (codes[M, K], scale_inv[M, K/128], codes_t[K, M], scale_inv_t[K, M/128]), bit-identical to
     ``quantize_1x128(x, kmajor=kmajor)`` and ``quantize_128x1_t(x, kmajor=kmajor)``.  M and K multiples of 128.
+    With ``column_sum`` (k-block-major scales only) a fifth result: the bf16 sum of x over its rows [K], from the
+    same read -- a bias gradient when x is grad_out -- with the bits of `column_sum(x)`.
     """
     x = _check_bf16(x, "x")
     if x.dim() != 2:
@@ -370,15 +379,45 @@ def quantize_1x128_and_128x1_t(x: torch.Tensor, kmajor: bool = True, pow2: bool 
     m, k = x.shape
     if m % BLOCK or k % BLOCK:
         raise ValueError(f"shape {tuple(x.shape)} is not a multiple of {BLOCK} in both dims")
+    if column_sum and not kmajor:
+        raise ValueError("column_sum comes with the k-block-major scale layout only (kmajor=True)")
     q = torch.empty((m, k), dtype=FP8, device=x.device)
     qt = _empty_codes_t(k, m, x.device)
     s_inv = torch.empty((k // BLOCK, m) if kmajor else (m, k // BLOCK), dtype=torch.float32, device=x.device)
     st_inv = torch.empty((m // BLOCK, k) if kmajor else (k, m // BLOCK), dtype=torch.float32, device=x.device)
+    if column_sum:
+        part = torch.empty((m // BLOCK, k), dtype=torch.float32, device=x.device)
+        _lib.call("hpfp8_quantize_128x1_t_colsum_bf16", _ptr(x), m, k, _ptr(q), None, _ptr(s_inv), _ptr(qt), _ld(qt), None,
+                  _ptr(st_inv), int(pow2), _ptr(part), _stream())
+        total = torch.empty((k,), dtype=torch.bfloat16, device=x.device)
+        _lib.call("hpfp8_column_sum_finish", _ptr(part), m // BLOCK, k, _ptr(total), None, _stream())
+        return q, s_inv.t(), qt, st_inv.t(), total
     _lib.call("hpfp8_quantize_1x128_and_128x1_t_pow2_bf16" if pow2 else "hpfp8_quantize_1x128_and_128x1_t_bf16", _ptr(x),
               m, k, int(kmajor), _ptr(q), None, _ptr(s_inv), _ptr(qt), _ld(qt), None, _ptr(st_inv), _stream())
     if kmajor:
         s_inv, st_inv = s_inv.t(), st_inv.t()
     return q, s_inv, qt, st_inv
+
+
+def column_sum(x: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """Sum of x[M, K] (bf16, K a multiple of 128, any M) over its rows, accumulated in fp32 in a fixed order (per
+    128-row block, then over the blocks) and returned as bf16 (rounded once) or fp32 [K]: the bias gradient of a
+    linear whose grad_out is x.  Same bits as the sum `quantize_1x128_and_128x1_t(..., column_sum=True)` returns."""
+    x = _check_bf16(x, "x")
+    if x.dim() != 2:
+        raise ValueError("x must be 2-D")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("out_dtype must be torch.bfloat16 or torch.float32")
+    m, k = x.shape
+    if k % BLOCK:
+        raise ValueError(f"width {k} is not a multiple of {BLOCK}")
+    blocks = (m + BLOCK - 1) // BLOCK
+    part = torch.empty((blocks, k), dtype=torch.float32, device=x.device)
+    out = torch.empty((k,), dtype=out_dtype, device=x.device)
+    bf = out_dtype == torch.bfloat16
+    _lib.call("hpfp8_column_sum_bf16", _ptr(x), m, k, _ld(x), _ptr(part), _ptr(out) if bf else None,
+              None if bf else _ptr(out), _stream())
+    return out
 
 
 def dequantize_1x128(q: torch.Tensor, scale_inv: torch.Tensor, grad_scale: float = 1.0) -> torch.Tensor:

@@ -97,8 +97,9 @@ int hpfp8_quantize_per_tensor_noalloc_bf16(const void* x, int64_t n, void* q, fl
                                            hpfp8_stream_t stream);
 
 /* Test hook, not part of the path: how many times a workgroup of the one-pass per-tensor quantizer polls for the
- * rest of its grid before it computes the tensor's maximum alone (default 2^22, about seconds).  0 forces that
- * path, which must give the same results. */
+ * rest of its grid before it computes the tensor's maximum alone (default 256 polls, a few hundred microseconds
+ * at most; a resident grid needs a handful).  0 forces that path, which must give the same results.  The value is
+ * process-wide and stored atomically: it may be set from any thread and takes effect with the next launch. */
 void hpfp8_debug_set_spin_limit(uint32_t polls);
 
 /* ---- blockwise quantizers --------------------------------------------------------------------
@@ -143,6 +144,28 @@ int hpfp8_quantize_128x1_t_kmajor_bf16(const void* x, int64_t m, int64_t k, void
 int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, int kmajor, void* q, float* scale,
                                           float* scale_inv, void* q_t, int64_t ld_t, float* scale_t,
                                           float* scale_inv_t, hpfp8_stream_t stream);
+
+/* Bias gradient.  The backward of the linear the reference dispatches (aten::linear at
+ * hyper_parallel/core/shard/_op_dispatch.py:277-283, differentiated by torch autograd) sums grad_out over the tokens
+ * for the bias.  Here that sum comes out of the pass that already reads every element of grad_out:
+ *   hpfp8_quantize_128x1_t_colsum_bf16  hpfp8_quantize_1x128_and_128x1_t_bf16 with kmajor = 1 (or, with q == NULL,
+ *                                       hpfp8_quantize_128x1_t_kmajor_bf16; pow2 != 0: the _pow2 forms), which also
+ *                                       writes colsum_partial[m/128, k] (fp32): per 128-row block and column the sum of
+ *                                       the block's rows;
+ *   hpfp8_column_sum_finish             out[col] = the partial sums of a column added in block order onto +0, as fp32
+ *                                       (out_f32) and / or rounded once to bf16 (out_bf16); either may be NULL;
+ *   hpfp8_column_sum_bf16               both steps for a matrix that is not being quantized (x[m, k], row stride ld
+ *                                       elements, any m, k a multiple of 128; partial[ceil(m/128), k] is caller-owned
+ *                                       scratch), with the same bits as the fused form.
+ * The additions inside a block run in a fixed order (stated with tile_column_sums in csrc/quantize.hip and restated
+ * by the CPU oracle), so the result is reproducible bit for bit. */
+int hpfp8_quantize_128x1_t_colsum_bf16(const void* x, int64_t m, int64_t k, void* q, float* scale, float* scale_inv, void* q_t,
+                                       int64_t ld_t, float* scale_t, float* scale_inv_t, int pow2, float* colsum_partial,
+                                       hpfp8_stream_t stream);
+int hpfp8_column_sum_finish(const float* partial, int64_t blocks, int64_t cols, void* out_bf16, float* out_f32,
+                            hpfp8_stream_t stream);
+int hpfp8_column_sum_bf16(const void* x, int64_t m, int64_t k, int64_t ld, float* partial, void* out_bf16, float* out_f32,
+                          hpfp8_stream_t stream);
 
 /* Power-of-two scales (an optional recipe; the stated one keeps plain fp32 scales): scale_inv is
  * amax_c / 448 rounded up to the next power of two and scale its exact reciprocal, everything else as in
@@ -327,7 +350,8 @@ int hpfp8_gemm_per_tensor(const void* a, int64_t lda, const float* sa_inv, const
 /* Small problems.  When a problem has fewer 256 x 256 output tiles than half the GPU's compute units (cfg-1-sized
  * layers, decode-sized M), hpfp8_gemm_per_tensor and hpfp8_gemm_blockwise (sb_gran = 128, no accumulate) run a
  * kernel with 128 x 128 tiles instead, four times as many workgroups; same arithmetic in the same order, identical
- * results.  Test hook, not part of the path: mode 0 = that rule (default), 1 = never, 2 = whenever the form allows. */
+ * results.  Test hook, not part of the path: mode 0 = that rule (default), 1 = never, 2 = whenever the form allows
+ * (process-wide, stored atomically, takes effect with the next launch). */
 void hpfp8_debug_set_small_gemm(int mode);
 
 /* MoE grouped form (one rank's local experts; no counterpart in the reference, whose expert

@@ -63,6 +63,10 @@ How each function is pinned (tests/test_oracle_pins.py)
       malformed offsets; every expert's piece equals quantize_1x128 of that expert's zero-padded rows transposed;
       the weight gradient equals the float64 product of the dequantized per-expert operands and is unchanged by
       the zero padding.
+  column_sum                : exact integer column sums on integer-valued inputs (any order of additions is exact
+      there, so a dropped or doubled row or a wrong column shows); float64 sums within the fp32 error bound of a
+      sum of that many terms; and hand-derived answers on inputs built so that a different order of the fp32
+      additions rounds differently (2^24 followed by ones), which pins the order stated in its docstring.
 No function here is "parity unpinned" in the mathematical sense; what IS unpinned is parity
 with the reference, because the reference has no FP8 code to compare with.
 """
@@ -82,7 +86,7 @@ __all__ = [
     "dequantize_128x128", "quantize_bucket", "dequantize_bucket",
     "gemm_per_tensor", "gemm_blockwise", "gemm_rowwise_both", "gemm_grouped_blockwise",
     "gemm_dequant_f64", "dequantize_per_tensor_f32", "swiglu_backward",
-    "grouped_layout", "quantize_128x1_t_grouped", "gemm_grouped_wgrad",
+    "grouped_layout", "quantize_128x1_t_grouped", "gemm_grouped_wgrad", "column_sum",
 ]
 
 
@@ -521,6 +525,38 @@ def gemm_grouped_wgrad(got, sgot_inv, xt, sxt_inv, offs, total_m: int):
         cols = slice(b0 * BLOCK, (b0 + nb) * BLOCK)
         out[e], _ = gemm_rowwise_both(got[:, cols], sgot_inv[:, b0:b0 + nb], xt[:, cols], sxt_inv[:, b0:b0 + nb])
     return out, f32_to_bf16_bits(out)
+
+
+def column_sum(x_bits: np.ndarray):
+    """Bias gradient of a linear whose grad_out is x[m, k] (bf16 bit patterns; k a multiple of 128): the sum over the
+    rows, in fp32, in the order the device kernels add (the backward of the aten::linear the reference dispatches at
+    hyper_parallel/core/shard/_op_dispatch.py:277-283 sums grad_out over the tokens in an order torch does not
+    specify; this build fixes one so that the result is reproducible):
+      * rows are taken in blocks of 128 (rows past m count as +0);
+      * inside a block, 16 "row quads" rq = 0..15 each add their 8 rows onto +0 in the order 4rq, 4rq+1, 4rq+2,
+        4rq+3, 64+4rq, ..., 64+4rq+3;
+      * the quads combine four at a time: (q0 + q1) + (q2 + q3) for rq = 4w .. 4w+3, w = 0..3, and the four results
+        as ((w0 + w1) + w2) + w3: the block's partial sum;
+      * the partial sums are added onto +0 in block order; the total is rounded once to bf16.
+    Returns (partial fp32 [ceil(m/128), k], total fp32 [k], total as bf16 bit patterns [k])."""
+    f = np.float32
+    x = bf16_bits_to_f32(np.asarray(x_bits))
+    m, k = x.shape
+    mb = (m + BLOCK - 1) // BLOCK
+    xp = np.zeros((mb * BLOCK, k), dtype=f)
+    xp[:m] = x
+    xt = xp.reshape(mb, 2, 16, 4, k)                    # tile row = half * 64 + 4 * rq + j
+    quad = np.zeros((mb, 16, k), dtype=f)
+    for half in range(2):
+        for j in range(4):
+            quad = (quad + xt[:, half, :, j, :]).astype(f)
+    quad = quad.reshape(mb, 4, 4, k)                    # [block, w, quad within w, column]
+    wsum = ((quad[:, :, 0] + quad[:, :, 1]).astype(f) + (quad[:, :, 2] + quad[:, :, 3]).astype(f)).astype(f)
+    part = (((wsum[:, 0] + wsum[:, 1]).astype(f) + wsum[:, 2]).astype(f) + wsum[:, 3]).astype(f)
+    total = np.zeros((k,), dtype=f)
+    for b in range(mb):
+        total = (total + part[b]).astype(f)
+    return part, total, f32_to_bf16_bits(total)
 
 
 def gemm_dequant_f64(a, sa_rows_inv, b, sb_rows_inv):

@@ -35,6 +35,8 @@ def test_forward_backward_vs_f_linear(gpu, recipe):
     assert rel(y, yr) < tol and rel(gx, x.grad) < tol and rel(gw, w.grad) < tol
     assert rel(gb, b.grad) < 1e-2
     assert gx.shape == x.shape and gw.shape == w.shape and gb.shape == b.shape
+    # the bias gradient is the oracle's fp32 column sum of grad_out, bit for bit, whichever kernel produced it
+    assert np.array_equal(U.bits(gb), O.column_sum(U.bits(go.reshape(-1, 384)))[2])
 
 
 def test_forward_equals_oracle_pipeline(gpu):
@@ -106,7 +108,7 @@ def test_prequantized_weight_and_module_cache(gpu):
         y1.backward(go)
         assert torch.equal(y1, y0) and torch.equal(x.grad, gx0) and torch.equal(w.grad, gw0)
         x.grad = w.grad = None
-    mod = hpfp8.Fp8Linear(384, 256, bias=False, device=gpu)
+    mod = hpfp8.Fp8Linear(384, 256, bias=False, cache_weight=True, device=gpu)
     with torch.no_grad():
         mod.weight.copy_(w)
     a = mod(x.detach())
@@ -130,7 +132,7 @@ def test_prequantized_weight_and_module_cache(gpu):
         hpfp8.fp8_linear(x, w, weight_fp8=wf)
     with pytest.raises(ValueError):
         hpfp8.fp8_linear(x, w, recipe="per_tensor", weight_fp8=hpfp8.quantize_weight(w.detach()))
-    mod = hpfp8.Fp8Linear(384, 256, bias=False, recipe="per_tensor", device=gpu)
+    mod = hpfp8.Fp8Linear(384, 256, bias=False, recipe="per_tensor", cache_weight=True, device=gpu)
     with torch.no_grad():
         mod.weight.copy_(w)
     a = mod(x.detach())
@@ -277,8 +279,13 @@ def test_weight_cache_contract_and_inference_mode(gpu, monkeypatch):
     `requires_grad` does not make forward prepare anything for a backward."""
     import hpfp8
     from hpfp8 import ops
-    mod = hpfp8.Fp8Linear(384, 256, bias=False, device=gpu)
+    plain = hpfp8.Fp8Linear(384, 256, bias=False, device=gpu)   # the default: no cache, so no write can go unseen
     x = U.randn_bf16((128, 384), 51).to(gpu)
+    a = plain(x).detach().clone()
+    plain.weight.data.mul_(2.0)
+    assert plain._fp8 is None and torch.equal(plain(x).detach(), hpfp8.fp8_linear(x, plain.weight.detach()))
+    assert not torch.equal(plain(x).detach(), a)
+    mod = hpfp8.Fp8Linear(384, 256, bias=False, cache_weight=True, device=gpu)
     a = mod(x).detach().clone()
     mod.weight.data.mul_(2.0)                                   # _version does not move
     stale = mod(x).detach()
@@ -298,7 +305,7 @@ def test_weight_cache_contract_and_inference_mode(gpu, monkeypatch):
     mod.load_state_dict(sd)
     assert mod._fp8 is None
     assert not torch.equal(mod(x).detach(), c)
-    mlp = hpfp8.Fp8SwiGLUMLP(256, 384, device=gpu)
+    mlp = hpfp8.Fp8SwiGLUMLP(256, 384, cache_weight=True, device=gpu)
     y0 = mlp(U.randn_bf16((128, 256), 52).to(gpu)).detach().clone()
     mlp.down_proj.weight.data.mul_(0.5)
     hpfp8.invalidate_fp8_caches(mlp)
@@ -594,7 +601,7 @@ def test_swiglu_mlp_module_caches_weights_and_trains(gpu):
     parameter is written, and an SGD step through it lowers a least-squares loss."""
     import hpfp8
     torch.manual_seed(0)
-    mlp = hpfp8.Fp8SwiGLUMLP(256, 384, device=gpu)
+    mlp = hpfp8.Fp8SwiGLUMLP(256, 384, cache_weight=True, device=gpu)
     x = torch.randn((128, 256), device=gpu).to(torch.bfloat16)
     y = mlp(x)
     want = hpfp8.fp8_swiglu_mlp(x, mlp.gate_up_proj.weight, mlp.down_proj.weight)

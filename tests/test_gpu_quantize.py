@@ -666,3 +666,50 @@ def test_tensors_beyond_2_31_elements(gpu):
     dh = hpfp8.ops.swiglu_backward(x, act)
     for r0 in blocks:
         assert torch.equal(dh[r0:r0 + 128], hpfp8.ops.swiglu_backward(x[r0:r0 + 128], act[r0:r0 + 128]))
+
+
+def test_column_sum_bias_gradient_fused_and_standalone(gpu):
+    """The bias gradient (fp32 column sums of grad_out in the oracle's stated order, rounded once to bf16): the
+    standalone kernel on ragged and whole row counts, and the form fused into the dual quantizer, whose codes and
+    scales must stay those of the plain dual quantizer."""
+    import hpfp8
+    from hpfp8 import ops
+    for (m, k), seed in (((1, 128), 1), ((127, 256), 2), ((128, 128), 3), ((300, 384), 4), ((1024, 512), 5)):
+        x = U.laplace_bf16((m, k), seed, 1e-3)
+        part, total, tb = O.column_sum(U.bits(x))
+        got32 = ops.column_sum(x.to(gpu), out_dtype=torch.float32)
+        got16 = ops.column_sum(x.to(gpu))
+        assert np.array_equal(U.f32_bits(got32.cpu().numpy()), U.f32_bits(total)), (m, k)
+        assert np.array_equal(U.bits(got16), tb), (m, k)
+    # a strided source (a column slice of a wider matrix)
+    wide = U.randn_bf16((256, 512), 6).to(gpu)
+    sl = wide[:, 128:384]
+    assert torch.equal(ops.column_sum(sl), ops.column_sum(sl.contiguous()))
+    # 2^24 and ones: the order of the additions is the stated one (see the oracle's pin of the same cases)
+    col = torch.zeros((256, 128), dtype=torch.bfloat16)
+    col[0, 0], col[4, 0], col[8, 0], col[12, 0] = 2.0 ** 24, 1.0, 1.0, 1.0
+    assert float(ops.column_sum(col.to(gpu), out_dtype=torch.float32)[0]) == 2.0 ** 24 + 2
+    for pow2 in (False, True):
+        x = U.laplace_bf16((512, 384), 7, 1e-3).to(gpu)
+        q, s, qt, st, db = ops.quantize_1x128_and_128x1_t(x, kmajor=True, pow2=pow2, column_sum=True)
+        q0, s0, qt0, st0 = ops.quantize_1x128_and_128x1_t(x, kmajor=True, pow2=pow2)
+        assert torch.equal(q.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(qt.view(torch.uint8), qt0.view(torch.uint8))
+        assert torch.equal(s, s0) and torch.equal(st, st0)
+        assert np.array_equal(U.bits(db), O.column_sum(U.bits(x))[2]) and torch.equal(db, ops.column_sum(x))
+    with pytest.raises(ValueError):
+        ops.quantize_1x128_and_128x1_t(x, kmajor=False, column_sum=True)
+    with pytest.raises(ValueError):
+        ops.column_sum(torch.zeros((4, 100), dtype=torch.bfloat16, device=gpu))
+
+
+def test_column_sum_at_full_size_against_float64(gpu):
+    """cfg 2's grad_out shape: the fused bias gradient against torch's float64 column sum (within the fp32 bound of a
+    4096-term sum) and, on a column block, against the oracle bit for bit."""
+    from hpfp8 import ops
+    go = (torch.randn((4096, 36864), device=gpu, generator=torch.Generator(device=gpu).manual_seed(9)) * 1e-3).to(torch.bfloat16)
+    _, _, _, _, db = ops.quantize_1x128_and_128x1_t(go, kmajor=True, column_sum=True)
+    ref = go.double().sum(dim=0)
+    bound = 4096 * 2.0 ** -24 * go.double().abs().sum(dim=0) + ref.abs() * 2.0 ** -8      # fp32 sum + one bf16 rounding
+    assert bool(((db.double() - ref).abs() <= bound).all())
+    sl = go[:, 1280:1536].contiguous()
+    assert np.array_equal(U.bits(db[1280:1536]), O.column_sum(U.bits(sl))[2])

@@ -658,3 +658,48 @@ def test_block_quantizer_against_an_independent_implementation_of_the_same_conve
         pytest.skip(f"power-of-two format not available: {e}")
     q2, _, si2 = O.quantize_128x128(U.bits(w), pow2=True)
     assert np.array_equal(tsi2, si2) and np.array_equal(tq2, q2)
+
+
+# ---- column_sum (bias gradient): facts the oracle did not author ------------------------------------------------
+
+def test_column_sum_is_exact_on_integers_and_bounded_against_float64():
+    rng = np.random.default_rng(7)
+    for m, k in ((1, 128), (127, 128), (128, 256), (300, 128), (513, 384)):
+        ints = rng.integers(-64, 65, size=(m, k)).astype(np.float32)           # bf16-exact, sums far below 2^24
+        bits = O.f32_to_bf16_bits(ints)
+        part, total, tb = O.column_sum(bits)
+        assert part.shape == ((m + 127) // 128, k) and part.dtype == np.float32
+        assert np.array_equal(total, ints.sum(axis=0, dtype=np.int64).astype(np.float32))
+        want_part = np.stack([ints[b * 128:(b + 1) * 128].sum(axis=0, dtype=np.int64) for b in range(part.shape[0])])
+        assert np.array_equal(part, want_part.astype(np.float32))
+        assert np.array_equal(tb, O.f32_to_bf16_bits(total))
+    # real data: within the error bound of an fp32 sum of m terms, n u sum|x| with u = 2^-24
+    x = O.f32_to_bf16_bits((rng.standard_normal((1000, 256)) * 1e-3).astype(np.float32))
+    xf = O.bf16_bits_to_f32(x).astype(np.float64)
+    _, total, _ = O.column_sum(x)
+    assert np.all(np.abs(total - xf.sum(axis=0)) <= 1000 * 2.0 ** -24 * np.abs(xf).sum(axis=0))
+
+
+def test_column_sum_order_is_the_stated_one():
+    """2^24 + 1 rounds back to 2^24 in fp32 (ties to even) while 1 + 1 = 2 survives being added to 2^24: where the
+    ones sit relative to the big value tells the orders of addition apart.  Answers derived by hand from the
+    order in the docstring, for one column each."""
+    big = np.float32(2.0 ** 24)
+
+    def total_of(rows):
+        col = np.zeros((256, 128), dtype=np.float32)
+        for r, v in rows.items():
+            col[r, 0] = v
+        return float(O.column_sum(O.f32_to_bf16_bits(col))[1][0])
+
+    # same row quad (rq = 0: rows 0, 1, 2, 3, 64, ...), added one after the other onto 2^24: every 1 is lost
+    assert total_of({0: big, 1: 1.0, 2: 1.0, 3: 1.0, 64: 1.0}) == 2.0 ** 24
+    # the ones in the neighbouring quad (rq = 1: rows 4..7): they first make 3, which survives (2^24 + 3 -> 2^24 + 4)
+    assert total_of({0: big, 4: 1.0, 5: 1.0, 6: 1.0}) == 2.0 ** 24 + 4
+    # one 1 each in quads 1, 2, 3 of the same group of four: q0 + q1 loses the first, q2 + q3 = 2 survives
+    assert total_of({0: big, 4: 1.0, 8: 1.0, 12: 1.0}) == 2.0 ** 24 + 2
+    # one 1 each in three other groups of four (rows 16, 32, 48): ((w0 + w1) + w2) + w3 loses every one of them
+    assert total_of({0: big, 16: 1.0, 32: 1.0, 48: 1.0}) == 2.0 ** 24
+    # the second block is added as a whole: its three ones make 3 first
+    assert total_of({0: big, 128: 1.0, 129: 1.0, 130: 1.0}) == 2.0 ** 24 + 4
+    # a purely sequential sum over the rows would have returned 2^24 in every case above
