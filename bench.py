@@ -29,52 +29,65 @@ for p in (ROOT, os.path.join(ROOT, "hyper-parallel_amd")):
 M, N, K = 4096, 36864, 7168
 PEAK_FP8_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
-# Bytes per GEMM launch that crossed the L2 <-> memory-fabric boundary come from two rocprofv3 --pmc runs
-# (FETCH_SIZE, calibrated on a copy of known size, + WRITE_SIZE) whose summary is kept in PROFILE; the summary
-# names the tiling of the kernel it was measured on, and the figure is only reported while csrc/gemm.hip still has
-# that tiling (otherwise `traffic` is null until the counters are collected again).
+# Bytes per GEMM launch that crossed the L2 <-> memory-fabric boundary come from rocprofv3 --pmc runs (FETCH_SIZE,
+# calibrated on a copy of known size, + WRITE_SIZE; and the requests among them destined for the memory controller)
+# whose summary is kept in PROFILE together with the sha256 of the kernel source it was measured on; the figure is
+# only reported while csrc/gemm.hip is still that source (otherwise `traffic` is null, with a line on stderr, until
+# the counters are collected again).
 PROFILE = os.path.join(ROOT, "profiles", "bench_cfg2_gemm_blockwise_and_quantizers.md")
 GEMM_SOURCE = os.path.join(ROOT, "hyper-parallel_amd", "csrc", "gemm.hip")
 
 
-def gemm_tiling_signature(path=GEMM_SOURCE):
-    """The constants of csrc/gemm.hip that decide how often operand panels are fetched from beyond L2."""
-    import re
-    text = open(path).read()
-    sig = []
-    for name in ("BM", "BN", "BK", "kRectTiles", "kXcds"):
-        m = re.search(r"\b%s\s*=\s*(\d+)" % name, text)
-        sig.append(f"{name}={m.group(1) if m else '?'}")
-    m = re.search(r"b_stages\(int mode\)\s*\{[^}]*\?\s*(\d+)\s*:\s*(\d+)", text)
-    sig.append(f"b_stages={m.group(2) if m else '?'}")
-    return " ".join(sig)
+def gemm_source_digest(path=GEMM_SOURCE):
+    """sha256 of csrc/gemm.hip: the profile summary records the digest of the source its counters were collected on."""
+    import hashlib
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
 
 
 def gemm_traffic_bytes():
-    """(bytes per launch, or None when the profile is absent or was taken on another tiling; the reason)."""
+    """({"tcc_ea": bytes per launch across the L2 <-> fabric boundary, "dram_path": bytes of those requests that were
+    destined for the memory controller} or None, the reason).  None -- and a loud line on stderr -- when the profile
+    summary is absent or was collected on another version of the kernel source: a stale figure is not reported."""
     import re
     try:
         text = open(PROFILE).read()
     except OSError:
         return None, "no profile summary"
-    m = re.search(r"traffic_bytes=(\d+)\s+gemm_tiling=\"([^\"]*)\"", text)
+    m = re.search(r"traffic_bytes=(\d+)\s+dram_path_bytes=(\d+)\s+gemm_source_sha256=([0-9a-f]{64})", text)
     if not m:
         return None, "profile summary has no traffic line"
-    if m.group(2) != gemm_tiling_signature():
-        return None, f"profile was taken on tiling [{m.group(2)}], the kernel now has [{gemm_tiling_signature()}]"
-    return int(m.group(1)), "profiles/" + os.path.basename(PROFILE)
+    if m.group(3) != gemm_source_digest():
+        why = ("profiles/%s was collected on another version of csrc/gemm.hip (its digest %s..., the source's %s...): "
+               "collect FETCH_SIZE / WRITE_SIZE again" % (os.path.basename(PROFILE), m.group(3)[:12], gemm_source_digest()[:12]))
+        print("bench.py: STALE TRAFFIC FIGURE NOT REPORTED: " + why, file=sys.stderr, flush=True)
+        return None, why
+    return {"tcc_ea": int(m.group(1)), "dram_path": int(m.group(2))}, "profiles/" + os.path.basename(PROFILE)
+
+
+def cpu_draw(gen, shape, kind="randn", chunk=1 << 26):
+    """fp32 values from the CPU generator `gen`, drawn in row chunks (bounded host memory), as one fp32 CPU tensor."""
+    import torch
+    fn = torch.randn if kind == "randn" else torch.rand
+    rows = shape[0]
+    per = max(1, chunk // max(1, int(torch.Size(shape[1:]).numel())))
+    parts = [fn((min(per, rows - r),) + tuple(shape[1:]), generator=gen, dtype=torch.float32) for r in range(0, rows, per)]
+    return parts[0] if len(parts) == 1 else torch.cat(parts)
 
 
 def make_inputs(dev):
+    """cfg 2's tensors, drawn with torch.Generator('cpu').manual_seed(0) in fp32, in this order -- x = randn(M, K), the
+    outlier positions randperm(M * K)[:k], W = randn(N, K) * 0.006 -- then cast to bf16 and copied to the device, so a
+    CPU run and a GPU run of the configuration see identical bytes."""
     import torch
-    g = torch.Generator(device=dev).manual_seed(0)
-    x = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = cpu_draw(g, (M, K))
     k = round(0.001 * M * K)
-    idx = torch.randperm(M * K, generator=g, device=dev)[:k]
+    idx = torch.randperm(M * K, generator=g)[:k]
     x.view(-1)[idx] *= 50.0
     x = x.to(torch.bfloat16)
-    w = (torch.randn((N, K), generator=g, device=dev, dtype=torch.float32) * 0.006).to(torch.bfloat16)
-    return x, w
+    w = (cpu_draw(g, (N, K)) * 0.006).to(torch.bfloat16)
+    return x.to(dev), w.to(dev)
 
 
 def event_ms(pairs):
@@ -133,6 +146,133 @@ def cpu_baseline(x_bits, w_bits, target_seconds=15.0):
     }
 
 
+def cpu_baselines_other_configs():
+    """The CPU legs of configurations 1, 3, 4 and 5 (host cores of this box, the oracle's C restatement with OpenMP;
+    cfg 1 also torch._scaled_mm on CPU): cfg 1 at full size, median of 5; the others on a bounded sample of the same
+    distribution with the factor to the full configuration stated; and, for cfg 5, what the reference does at that
+    site today: the dtype round trip bf16 -> reduce_dtype -> bf16 of
+    hyper_parallel/core/hsdp/hsdp_grad_buffer.py:105-106 and :121-122 (torch on CPU, reduce_dtype = float32)."""
+    import numpy as np
+    import torch
+    from oracle import c_oracle as C
+    from oracle import fp8_oracle as O
+    threads = C.num_threads()
+    torch.set_num_threads(threads)
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    res = {"cores": threads}
+
+    def median_of(fn, n=5):
+        ts = []
+        for _ in range(n):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2]
+
+    # cfg 1, full size, the tensors of the GPU run (CPU generator, seed 0)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = cpu_draw(g, (2048, 1024)).to(torch.bfloat16)
+    w = (cpu_draw(g, (1024, 1024)) * 0.02).to(torch.bfloat16)
+    xb, wb = bits(x), bits(w)
+    fl1 = 2.0 * 2048 * 1024 * 1024
+
+    def oracle_step():
+        xq, _, sx = C.quantize_per_tensor(xb)
+        wq, _, sw = C.quantize_per_tensor(wb)
+        return O.gemm_per_tensor(xq, sx, wq, sw)
+    t_or = median_of(oracle_step)
+    xq, _, sx = C.quantize_per_tensor(xb)
+    wq, _, sw = C.quantize_per_tensor(wb)
+    F8 = torch.float8_e4m3fn
+    xa, wa = torch.from_numpy(xq).view(F8), torch.from_numpy(wq).view(F8)
+    sxt, swt = torch.tensor(float(sx)), torch.tensor(float(sw))
+    c1 = {"oracle_quantize_x_quantize_w_gemm": {"ms": t_or * 1e3, "TFLOP/s": fl1 / t_or / 1e12, "sample": "full size, median of 5"}}
+    try:
+        # (torch's CPU routine for float8 operands takes about 10 s for the full 2048 rows: a quarter of them, x 4)
+        xa4 = xa[:512]
+        t_sm = median_of(lambda: torch._scaled_mm(xa4, wa.t(), scale_a=sxt, scale_b=swt, out_dtype=torch.bfloat16)) * 4
+        c1["torch_scaled_mm_gemm_only"] = {"ms": t_sm * 1e3, "TFLOP/s": fl1 / t_sm / 1e12,
+                                           "sample": "512 of 2048 rows, median of 5, x 4"}
+    except Exception as err:          # (not in every CPU build of torch)
+        c1["torch_scaled_mm_gemm_only"] = f"unavailable: {type(err).__name__}"
+    xg_, wg_ = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    go_ = torch.ones((2048, 1024), dtype=torch.bfloat16)
+
+    def lin_fwd_bwd():
+        torch.nn.functional.linear(xg_, wg_).backward(go_)
+        xg_.grad = wg_.grad = None
+    t_bf = median_of(lin_fwd_bwd)
+    c1["aten_linear_bf16_forward_backward"] = {"ms": t_bf * 1e3, "TFLOP/s": 3 * fl1 / t_bf / 1e12, "sample": "full size, median of 5"}
+    res["cfg1_per_tensor"] = c1
+
+    # cfg 3 (M 4096, N 7168, K 16384): dgrad on the first 256 token rows (x 16), wgrad on the first 1024 columns of x (x 16)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    m, n, k, ms_, ks_ = 4096, 7168, 16384, 256, 1024
+    xs = bits(cpu_draw(g, (m, ks_)).to(torch.bfloat16))
+    u = cpu_draw(g, (m, n), kind="rand") - 0.5
+    go = bits((-(2 ** -0.5) * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999)) * 1e-3).to(torch.bfloat16))
+    wt = bits((cpu_draw(g, (k, n)) * 0.006).to(torch.bfloat16))          # W^T [K, N], drawn directly in that layout
+    t0 = time.perf_counter()
+    wtq, _, swt_ = C.quantize_128x128(wt)
+    t_qw = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    goq, _, sgo = C.quantize_1x128(np.ascontiguousarray(go[:ms_]))
+    C.gemm_blockwise(goq, sgo, wtq, swt_)
+    t_d = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    got, _, sgot = C.quantize_128x1_t(go)
+    xt, _, sxt_ = C.quantize_128x1_t(xs)
+    t_q = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    C.gemm_blockwise(got, sgot, xt, sxt_, sb_per_row=True)
+    t_w = time.perf_counter() - t0
+    fl3 = 2.0 * m * n * k
+    res["cfg3_backward"] = {
+        "dgrad": {"TFLOP/s": fl3 / (t_d * m / ms_) / 1e12, "sample": f"quantize + GEMM of {ms_} of {m} token rows ({t_d:.1f} s), x {m // ms_}"},
+        "wgrad": {"TFLOP/s": fl3 / (t_w * k / ks_) / 1e12, "sample": f"GEMM on {ks_} of {k} columns of x ({t_w:.1f} s), x {k // ks_}"},
+        "requant_t_GB/s": (m * n + m * ks_) * 3 / t_q / 1e9,
+        "quantize_w_128x128_GB/s": k * n * 3 / t_qw / 1e9,
+    }
+    del wt, wtq, go, got, xs, xt
+
+    # cfg 4: 512 rows of one expert against that expert's weight [4096, 7168] (131072 rows in all: x 256)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    we = bits((cpu_draw(g, (4096, 7168)) * 0.006).to(torch.bfloat16))
+    xe = bits(cpu_draw(g, (512, 7168)).to(torch.bfloat16))
+    weq, _, swe = C.quantize_128x128(we)
+    t0 = time.perf_counter()
+    xeq, _, sxe = C.quantize_1x128(xe)
+    C.gemm_blockwise(xeq, sxe, weq, swe)
+    t_e = time.perf_counter() - t0
+    res["cfg4_moe_grouped"] = {"forward": {"TFLOP/s": 2.0 * 512 * 4096 * 7168 / t_e / 1e12,
+                                           "sample": f"quantize + GEMM of 512 rows of one expert ({t_e:.1f} s), x 256 for the 131072 routed rows"}}
+    del we, weq
+
+    # cfg 5: 2^25 of the 2^29 elements (x 16); and the reference's own cast round trip at this site on 2^27 (x 4)
+    nel = 1 << 25
+    flat = bits((torch.randn(nel, generator=g) * 1e-4).to(torch.bfloat16)).reshape(-1, 128)
+    t0 = time.perf_counter()
+    cq, _, csi = C.quantize_1x128(flat)
+    t_q5 = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    C.dequantize_1x128(cq, csi)
+    t_d5 = time.perf_counter() - t0
+    nb5 = nel * 3 + nel // 128 * 4
+    big = (torch.randn(1 << 27, generator=g) * 1e-4).to(torch.bfloat16)
+    t0 = time.perf_counter()
+    back = big.to(torch.float32).to(torch.bfloat16)
+    t_rt = time.perf_counter() - t0
+    res["cfg5_bucket"] = {
+        "quantize_GB/s": nb5 / t_q5 / 1e9, "dequantize_GB/s": nb5 / t_d5 / 1e9,
+        "sample": f"2^25 of 2^29 elements (x 16): {t_q5:.2f} s + {t_d5:.2f} s",
+        "reference_cast_round_trip_bf16_fp32_bf16": {"GB/s": (1 << 27) * 12 / t_rt / 1e9,
+                                                     "sample": f"torch on CPU, 2^27 of 2^29 elements (x 4): {t_rt:.2f} s; 2 + 4 bytes "
+                                                               "per element cast in, 4 + 2 cast back"},
+    }
+    del back, big
+    return res
+
+
 def _time(fn, iters=30, warm=40):
     import torch
     for _ in range(warm):
@@ -145,6 +285,66 @@ def _time(fn, iters=30, warm=40):
     s1.record()
     torch.cuda.synchronize()
     return s0.elapsed_time(s1) / iters
+
+
+CACHE_BYTES = 256 << 20         # the Infinity Cache between the L2s and HBM
+
+
+def _n_sets(bytes_per_set):
+    """How many copies of a kernel's buffers to rotate through so that a launch finds none of its data in the
+    Infinity Cache: the copies together hold more than 2.5 times its size."""
+    return max(2, int(2.5 * CACHE_BYTES // max(1, bytes_per_set)) + 1)
+
+
+def _time_rot(launch, nsets, iters=30, warm=40):
+    """Like _time for launch(i), which must use buffer set i % nsets."""
+    import torch
+    for i in range(warm):
+        launch(i % nsets)
+    torch.cuda.synchronize()
+    s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s0.record()
+    for i in range(iters):
+        launch(i % nsets)
+    s1.record()
+    torch.cuda.synchronize()
+    return s0.elapsed_time(s1) / iters
+
+
+def quantizer_rows(src, dev, prefix=""):
+    """Every quantizer form of one bf16 source [m, k] through the C ABI on preallocated buffers that rotate beyond the
+    Infinity Cache (source copies and outputs alike): {name: {ms, GB/s, frac_hbm}}."""
+    import torch
+    from hpfp8 import _lib
+    from hpfp8.ops import _padded_ld
+    m, k = src.shape
+    FP8 = torch.float8_e4m3fn
+    st = torch.cuda.current_stream().cuda_stream
+    ld_t = _padded_ld(m)
+    n = _n_sets(m * k * 4)
+    xs = [src] + [src.clone() for _ in range(n - 1)]
+    q = [torch.empty((m, k), dtype=FP8, device=dev) for _ in range(n)]
+    qt = [torch.empty((k, ld_t), dtype=FP8, device=dev) for _ in range(n)]
+    s1 = torch.empty((k // 128, m), dtype=torch.float32, device=dev)
+    s2 = torch.empty((m // 128, k), dtype=torch.float32, device=dev)
+    part = torch.empty((m // 128, k), dtype=torch.float32, device=dev)
+    db = torch.empty((k,), dtype=torch.bfloat16, device=dev)
+    P = lambda t: t.data_ptr()
+    sc = m * k // 128 * 4
+    out = {}
+    out[prefix + "quantize_1x128"] = _gb(m * k * 3 + sc, _time_rot(lambda i: _lib.call(
+        "hpfp8_quantize_1x128_kmajor_bf16", P(xs[i]), m, k, P(q[i]), None, P(s1), st), n))
+    out[prefix + "requant_t"] = _gb(m * k * 3 + sc, _time_rot(lambda i: _lib.call(
+        "hpfp8_quantize_128x1_t_kmajor_bf16", P(xs[i]), m, k, P(qt[i]), ld_t, None, P(s2), st), n))
+    out[prefix + "quantize_both_forms"] = _gb(m * k * 4 + 2 * sc, _time_rot(lambda i: _lib.call(
+        "hpfp8_quantize_1x128_and_128x1_t_bf16", P(xs[i]), m, k, 1, P(q[i]), None, P(s1), P(qt[i]), ld_t, None, P(s2), st), n))
+
+    def with_bias(i):
+        _lib.call("hpfp8_quantize_128x1_t_colsum_bf16", P(xs[i]), m, k, P(q[i]), None, P(s1), P(qt[i]), ld_t, None, P(s2), 0,
+                  P(part), st)
+        _lib.call("hpfp8_column_sum_finish", P(part), m // 128, k, P(db), None, st)
+    out[prefix + "quantize_both_forms_and_bias_gradient"] = _gb(m * k * 4 + 3 * sc, _time_rot(with_bias, n))
+    return out
 
 
 def _tf(flops, ms):
@@ -174,38 +374,47 @@ def zipf_counts(experts, total, seed=0):
 def other_configs_compact(dev):
     """The other four benchmark configurations, each kernel with its own roofline fraction (HIP events around
     back-to-back launches after a warm-up): cfg 1 per-tensor quantize + GEMM, cfg 3 backward GEMMs and transposed
-    requantizers, cfg 4 MoE grouped GEMMs and the whole grouped layer, cfg 5 bucket quantize / dequantize."""
+    requantizers, cfg 4 MoE grouped GEMMs and the whole grouped layer, cfg 5 bucket quantize / dequantize.  Every
+    HBM-bound kernel whose tensors would fit the Infinity Cache runs on buffers that rotate beyond it.  cfg 1 and 3
+    are drawn with the CPU generator (seed 0, one generator per configuration, tensors in the order listed in the
+    benchmark's description); cfg 4's 2.4e9 and cfg 5's 5.4e8 values are drawn on the GPU (same distributions, seed
+    0), where they take a second instead of a minute."""
     import torch
     import hpfp8
     from hpfp8 import ops
-    res = {}
+    res = {"data_generator": {"cfg1": "cpu seed 0", "cfg2": "cpu seed 0", "cfg3": "cpu seed 0",
+                              "cfg4": "gpu seed 0 (deviation: 2.4e9 values)", "cfg5": "gpu seed 0 (deviation: 5.4e8 values)"}}
     g = torch.Generator(device=dev).manual_seed(0)
     # cfg 1: per-tensor linear 2048 x 1024 x 1024 (launch-bound: times include the launches)
-    x = torch.randn((2048, 1024), generator=g, device=dev).to(torch.bfloat16)
-    w = (torch.randn((1024, 1024), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    g1 = torch.Generator(device="cpu").manual_seed(0)
+    x = cpu_draw(g1, (2048, 1024)).to(torch.bfloat16).to(dev)
+    w = (cpu_draw(g1, (1024, 1024)) * 0.02).to(torch.bfloat16).to(dev)
     xq, _, sx = hpfp8.quantize_per_tensor(x)
     wq, _, sw = hpfp8.quantize_per_tensor(w)
     # (timed through the C ABI with outputs allocated beforehand: at this size the Python wrappers' allocations
-    # would be most of the time)
+    # would be most of the time; 64 copies of x and of its codes, 384 MB, so that no launch finds its data in a cache)
     from hpfp8 import _lib
     st = torch.cuda.current_stream().cuda_stream
-    q1 = torch.empty((2048, 1024), dtype=torch.uint8, device=dev)
+    n1 = 64
+    x1 = [x] + [x.clone() for _ in range(n1 - 1)]
+    q1 = [torch.empty((2048, 1024), dtype=torch.uint8, device=dev) for _ in range(n1)]
+    xq1 = [xq] + [xq.clone() for _ in range(n1 - 1)]
     w3 = torch.zeros(3, dtype=torch.float32, device=dev)
-    c1 = torch.empty((2048, 1024), dtype=torch.bfloat16, device=dev)
+    c1 = [torch.empty((2048, 1024), dtype=torch.bfloat16, device=dev) for _ in range(n1)]
     pw = w3.data_ptr()
     sync = torch.zeros(128, dtype=torch.int32, device=dev)
-    quant = lambda: _lib.call("hpfp8_quantize_per_tensor_sync_bf16", x.data_ptr(), x.numel(), q1.data_ptr(), pw, pw + 4, pw + 8,
-                              sync.data_ptr(), st)
-    gemm = lambda: _lib.call("hpfp8_gemm_per_tensor", xq.data_ptr(), 1024, sx.data_ptr(), wq.data_ptr(), 1024, sw.data_ptr(),
-                             2048, 1024, 1024, None, c1.data_ptr(), 1024, 0, st)
-    t_q = _time(quant, iters=200, warm=100)
-    t_g = _time(gemm, iters=200, warm=100)
-    t_both = _time(lambda: (quant(), gemm()), iters=200, warm=100)
+    quant = lambda i: _lib.call("hpfp8_quantize_per_tensor_sync_bf16", x1[i].data_ptr(), x.numel(), q1[i].data_ptr(), pw, pw + 4,
+                                pw + 8, sync.data_ptr(), st)
+    gemm = lambda i: _lib.call("hpfp8_gemm_per_tensor", xq1[i].data_ptr(), 1024, sx.data_ptr(), wq.data_ptr(), 1024, sw.data_ptr(),
+                               2048, 1024, 1024, None, c1[i].data_ptr(), 1024, 0, st)
+    t_q = _time_rot(quant, n1, iters=200, warm=100)
+    t_g = _time_rot(gemm, n1, iters=200, warm=100)
+    t_both = _time_rot(lambda i: (quant(i), gemm(i)), n1, iters=200, warm=100)
     res["cfg1_per_tensor"] = {"quantize_x": _gb(x.numel() * 3, t_q), "gemm": _tf(2.0 * 2048 * 1024 * 1024, t_g),
                               "quantize_x_plus_gemm_us": t_both * 1e3,
-                              "note": "launch-bound: two launches (one-pass amax + cast, 128 x 128-tile GEMM), "
-                                      "times include the launches"}
-    del x, w, xq, wq, q1, c1
+                              "note": "launch-bound: two launches (one-pass amax + cast, 128 x 128-tile GEMM), times "
+                                      "include the launches; buffers rotate over 64 copies"}
+    del x, w, xq, wq, q1, c1, x1, xq1
     # cfg 2's layer as an inference MLP block: the gate/up GEMM with SwiGLU + the 1x128 quantizer as its epilogue
     # (no bf16 gate/up tensor), then the down projection
     x = torch.randn((4096, 7168), generator=g, device=dev).to(torch.bfloat16)
@@ -236,29 +445,40 @@ def other_configs_compact(dev):
     torch.cuda.empty_cache()
     # cfg 3: o_proj backward, M = 4096 tokens, W[7168, 16384]
     m, n, k = 4096, 7168, 16384
-    x = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
-    u = torch.rand((m, n), generator=g, device=dev) - 0.5
-    go = (-(2 ** -0.5) * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999)) * 1e-3).to(torch.bfloat16)
-    w = (torch.randn((n, k), generator=g, device=dev) * 0.006).to(torch.bfloat16)
+    g3 = torch.Generator(device="cpu").manual_seed(0)
+    x = cpu_draw(g3, (m, k)).to(torch.bfloat16).to(dev)
+    u = cpu_draw(g3, (m, n), kind="rand") - 0.5
+    go = (-(2 ** -0.5) * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999)) * 1e-3).to(torch.bfloat16).to(dev)
+    w = (cpu_draw(g3, (n, k)) * 0.006).to(torch.bfloat16).to(dev)
+    del u
     wq, sw, wqt = hpfp8.quantize_128x128(w, with_transpose=True)
     goq, sgo = hpfp8.quantize_1x128(go, kmajor=True)
     got, sgot = hpfp8.quantize_128x1_t(go, kmajor=True)
     xt, sxt = hpfp8.quantize_128x1_t(x, kmajor=True)
     fl = 2.0 * m * n * k
-    res["cfg3_backward"] = {
+    main_grad = torch.zeros((n, k), dtype=torch.float32, device=dev)
+    r3 = {
         "dgrad_gemm": _tf(fl, _time(lambda: hpfp8.gemm_blockwise(goq, sgo, wqt, sw.t()))),
         "wgrad_gemm": _tf(fl, _time(lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1))),
-        "requant_t_x": _gb(m * k * 3 + k * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(x, kmajor=True))),
-        "requant_t_grad_out": _gb(m * n * 3 + n * (m // 128) * 4, _time(lambda: hpfp8.quantize_128x1_t(go, kmajor=True))),
-        "quantize_grad_out": _gb(m * n * 3 + m * (n // 128) * 4, _time(lambda: hpfp8.quantize_1x128(go, kmajor=True))),
-        "quantize_both_forms_x": _gb(m * k * 4 + 2 * m * (k // 128) * 4,
-                                     _time(lambda: hpfp8.quantize_1x128_and_128x1_t(x, kmajor=True))),
-        "quantize_both_forms_grad_out": _gb(m * n * 4 + 2 * m * (n // 128) * 4,
-                                            _time(lambda: hpfp8.quantize_1x128_and_128x1_t(go, kmajor=True))),
-        "quantize_w_with_transpose": _gb(n * k * 4 + (n // 128) * (k // 128) * 4,
-                                         _time(lambda: hpfp8.quantize_128x128(w, with_transpose=True))),
+        "wgrad_gemm_into_fp32_main_grad": _tf(fl, _time(
+            lambda: hpfp8.gemm_blockwise(got, sgot, xt, sxt, sb_gran=1, out=main_grad, accumulate=True))),
     }
-    del x, go, w, wq, wqt, goq, got, xt, u
+    del main_grad, wq, wqt, goq, got, xt
+    torch.cuda.empty_cache()
+    r3.update(quantizer_rows(x, dev, "x_"))
+    r3.update(quantizer_rows(go, dev, "grad_out_"))
+    # the weight with its transposed codes (470 MB per launch: beyond the cache by itself; two sets all the same)
+    from hpfp8.ops import _padded_ld
+    ldw = _padded_ld(n)
+    ws = [w, w.clone()]
+    wqs = [torch.empty((n, k), dtype=torch.float8_e4m3fn, device=dev) for _ in range(2)]
+    wts = [torch.empty((k, ldw), dtype=torch.float8_e4m3fn, device=dev) for _ in range(2)]
+    sws = torch.empty((n // 128, k // 128), dtype=torch.float32, device=dev)
+    r3["quantize_w_with_transpose"] = _gb(n * k * 4 + (n // 128) * (k // 128) * 4, _time_rot(lambda i: _lib.call(
+        "hpfp8_quantize_128x128_bf16", ws[i].data_ptr(), n, k, wqs[i].data_ptr(), wts[i].data_ptr(), ldw, None, sws.data_ptr(), st), 2))
+    r3["note"] = "quantizer rows: source copies and outputs rotate over more than 640 MB (Infinity Cache: 256 MB)"
+    res["cfg3_backward"] = r3
+    del x, go, w, ws, wqs, wts
     torch.cuda.empty_cache()
     # cfg 4: MoE grouped, 32 experts, 131072 routed rows, Zipf(1.1) counts, two empty experts
     e, n, k, total = 32, 4096, 7168, 131072
@@ -646,7 +866,8 @@ def main():
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_tflops / PEAK_FP8_TFLOPS,
-            "traffic": traffic,
+            "traffic": traffic["tcc_ea"] if traffic else None,
+            "traffic_dram_path": traffic["dram_path"] if traffic else None,
             "traffic_source": traffic_source,
             "ms": t_g,
         },
@@ -671,6 +892,8 @@ def main():
         out["more"] = more_measurements(dev)
     if host_copies is not None:
         out["cpu_baseline"] = cpu_baseline(*host_copies)
+        if not args.headline_only:
+            out["cpu_baseline"]["other_configs"] = cpu_baselines_other_configs()
     print(json.dumps(out))
 
 

