@@ -856,6 +856,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5))) void q
 }
 
 // ---------------------------------------------------------------------------------------------
+// traffic model of the transposing quantizers (measurement aid)
+// ---------------------------------------------------------------------------------------------
+// The memory accesses of quant_128x1_t_kernel and nothing else: a workgroup loads its 128x128 bf16 tile with the
+// same instructions, folds the loaded words together so that the stores depend on them, and writes 128 rows of 128
+// bytes where the transposed codes would go (and, with q, the 128 rows of 128 bytes of the row-major codes): no
+// amax, no scales, no conversion, no LDS, no barrier.  What it reaches is what the access pattern allows on the
+// machine; the distance of the real kernel to it is what the arithmetic and the LDS transposition cost.
+__global__ __launch_bounds__(256) void transpose_traffic_model_kernel(const uint16_t* __restrict__ x, int64_t ld_src, int k,
+                                                                      uint8_t* __restrict__ qt, int64_t ld_t,
+                                                                      uint8_t* __restrict__ q, int along_k) {
+  const int cg = threadIdx.x & 15, rq = threadIdx.x >> 4;
+  const int tr = along_k ? blockIdx.y : blockIdx.x, tc = along_k ? blockIdx.x : blockIdx.y;
+  const char* sbase = reinterpret_cast<const char*>(x + (int64_t)tr * 128 * ld_src + tc * 128);
+  const uint32_t ld_b = (uint32_t)ld_src * 2u;
+  uint4 v[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) v[p] = nt_load16(sbase + ((uint32_t)tile_row(rq, p) * ld_b + (uint32_t)cg * 16u));
+  uint4 acc = v[0];
+#pragma unroll
+  for (int p = 1; p < 8; ++p) {
+    acc.x ^= v[p].x; acc.y ^= v[p].y; acc.z ^= v[p].z; acc.w ^= v[p].w;
+  }
+  char* dst = reinterpret_cast<char*>(qt + (int64_t)tc * 128 * ld_t + tr * 128);
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass)
+    nt_store16(dst + ((uint32_t)(pass * 32 + (threadIdx.x >> 3)) * (uint32_t)ld_t + (uint32_t)(threadIdx.x & 7) * 16u), acc);
+  if (q) {
+    char* qbase = reinterpret_cast<char*>(q + (int64_t)tr * 128 * k + tc * 128);
+#pragma unroll
+    for (int p = 0; p < 8; ++p)
+      nt_store8(qbase + ((uint32_t)tile_row(rq, p) * (uint32_t)k + (uint32_t)cg * 8u), make_uint2(acc.x ^ v[p].x, acc.y ^ v[p].y));
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // column sums (bias gradient): x[m, k] bf16 -> per 128-row block partial sums fp32 [ceil(m/128), k] -> bf16 / fp32 [k]
 // ---------------------------------------------------------------------------------------------
 // The same tiles, the same order of additions as the COLSUM form of quant_128x1_t_kernel (rows past m count as +0),
@@ -1403,6 +1438,19 @@ int hpfp8_quantize_1x128_and_128x1_t_bf16(const void* x, int64_t m, int64_t k, i
   HPFP8_REQUIRE(m == 0 || k == 0 || q != nullptr, HPFP8_ERR_ARG, "quantize_1x128_and_128x1_t: null buffer");
   return quantize_128x1_t_impl("quantize_1x128_and_128x1_t", kmajor != 0, x, m, k, q_t, ld_t, scale_t, scale_inv_t,
                                stream, q, scale, scale_inv);
+}
+
+int hpfp8_debug_transpose_traffic_model(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t, void* q,
+                                        hpfp8_stream_t stream) {
+  const char* what = "debug_transpose_traffic_model";
+  HPFP8_REQUIRE(m > 0 && k > 0 && m % kBlock == 0 && k % kBlock == 0, HPFP8_ERR_SHAPE, "%s: shape must be positive multiples of 128", what);
+  HPFP8_REQUIRE(m < (1 << 30) && k < (1 << 24) && ld_t < (1 << 24) && ld_t >= m && ld_t % 16 == 0, HPFP8_ERR_SHAPE, "%s: bad shape", what);
+  HPFP8_REQUIRE(x && q_t && aligned16(x) && aligned16(q_t) && (!q || aligned16(q)), HPFP8_ERR_ARG, "%s: bad buffer", what);
+  int ak = 0;
+  const dim3 grid = transpose_grid(m / kBlock, k / kBlock, k * 2, q ? 2 : 1, ak);
+  transpose_traffic_model_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, k, (int)k, (uint8_t*)q_t, ld_t,
+                                                                       (uint8_t*)q, ak);
+  return check_launch(what);
 }
 
 int hpfp8_quantize_128x1_t_colsum_bf16(const void* x, int64_t m, int64_t k, void* q, float* scale, float* scale_inv, void* q_t,

@@ -42,6 +42,7 @@ SIGNATURES = {
     "hpfp8_quantize_128x128_bf16": [_vp, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
     "hpfp8_quantize_128x1_t_colsum_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, ctypes.c_int, _vp, _vp],
     "hpfp8_column_sum_finish": [_vp, _i64, _i64, _vp, _vp, _vp],
+    "hpfp8_debug_transpose_traffic_model": [_vp, _i64, _i64, _vp, _i64, _vp, _vp],
     "hpfp8_column_sum_bf16": [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_1x128_kmajor_pow2_bf16": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
     "hpfp8_quantize_128x128_pow2_bf16": [_vp, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp],

@@ -96,6 +96,13 @@ int hpfp8_quantize_per_tensor_sync_bf16(const void* x, int64_t n, void* q, float
 int hpfp8_quantize_per_tensor_noalloc_bf16(const void* x, int64_t n, void* q, float* scale, float* scale_inv,
                                            hpfp8_stream_t stream);
 
+/* Measurement aid, not part of the path: the memory traffic of hpfp8_quantize_128x1_t_kmajor_bf16 (q == NULL) or of
+ * hpfp8_quantize_1x128_and_128x1_t_bf16 (q != NULL) and nothing else -- the same tile loads, in the same tile order,
+ * and stores of the same sizes at the same addresses, whose contents are meaningless.  bench.py times it beside the
+ * real kernels: what it reaches is what the access pattern allows on the machine. */
+int hpfp8_debug_transpose_traffic_model(const void* x, int64_t m, int64_t k, void* q_t, int64_t ld_t, void* q,
+                                        hpfp8_stream_t stream);
+
 /* Test hook, not part of the path: how many times a workgroup of the one-pass per-tensor quantizer polls for the
  * rest of its grid before it computes the tensor's maximum alone (default 256 polls, a few hundred microseconds
  * at most; a resident grid needs a handful).  0 forces that path, which must give the same results.  The value is
