@@ -311,7 +311,7 @@ def _time_rot(launch, nsets, iters=30, warm=40):
     return s0.elapsed_time(s1) / iters
 
 
-def quantizer_rows(src, dev, prefix=""):
+def quantizer_rows(src, dev, prefix="", iters=30, warm=40):
     """Every quantizer form of one bf16 source [m, k] through the C ABI on preallocated buffers that rotate beyond the
     Infinity Cache (source copies and outputs alike): {name: {ms, GB/s, frac_hbm}}."""
     import torch
@@ -332,24 +332,25 @@ def quantizer_rows(src, dev, prefix=""):
     P = lambda t: t.data_ptr()
     sc = m * k // 128 * 4
     out = {}
-    out[prefix + "quantize_1x128"] = _gb(m * k * 3 + sc, _time_rot(lambda i: _lib.call(
-        "hpfp8_quantize_1x128_kmajor_bf16", P(xs[i]), m, k, P(q[i]), None, P(s1), st), n))
-    out[prefix + "requant_t"] = _gb(m * k * 3 + sc, _time_rot(lambda i: _lib.call(
-        "hpfp8_quantize_128x1_t_kmajor_bf16", P(xs[i]), m, k, P(qt[i]), ld_t, None, P(s2), st), n))
-    out[prefix + "quantize_both_forms"] = _gb(m * k * 4 + 2 * sc, _time_rot(lambda i: _lib.call(
-        "hpfp8_quantize_1x128_and_128x1_t_bf16", P(xs[i]), m, k, 1, P(q[i]), None, P(s1), P(qt[i]), ld_t, None, P(s2), st), n))
+    T = lambda fn: _time_rot(fn, n, iters=iters, warm=warm)
+    out[prefix + "quantize_1x128"] = _gb(m * k * 3 + sc, T(lambda i: _lib.call(
+        "hpfp8_quantize_1x128_kmajor_bf16", P(xs[i]), m, k, P(q[i]), None, P(s1), st)))
+    out[prefix + "requant_t"] = _gb(m * k * 3 + sc, T(lambda i: _lib.call(
+        "hpfp8_quantize_128x1_t_kmajor_bf16", P(xs[i]), m, k, P(qt[i]), ld_t, None, P(s2), st)))
+    out[prefix + "quantize_both_forms"] = _gb(m * k * 4 + 2 * sc, T(lambda i: _lib.call(
+        "hpfp8_quantize_1x128_and_128x1_t_bf16", P(xs[i]), m, k, 1, P(q[i]), None, P(s1), P(qt[i]), ld_t, None, P(s2), st)))
 
     def with_bias(i):
         _lib.call("hpfp8_quantize_128x1_t_colsum_bf16", P(xs[i]), m, k, P(q[i]), None, P(s1), P(qt[i]), ld_t, None, P(s2), 0,
                   P(part), st)
         _lib.call("hpfp8_column_sum_finish", P(part), m // 128, k, P(db), None, st)
     out[prefix + "quantize_both_forms_and_bias_gradient"] = dict(
-        _gb(m * k * 4 + 3 * sc, _time_rot(with_bias, n)), note="two launches: the quantizer, then the sum over the 128-row blocks")
+        _gb(m * k * 4 + 3 * sc, T(with_bias)), note="two launches: the quantizer, then the sum over the 128-row blocks")
     # what the two transposing access patterns allow on this machine: the same loads and stores with nothing between them
-    out[prefix + "requant_t_traffic_model"] = _gb(m * k * 3, _time_rot(lambda i: _lib.call(
-        "hpfp8_debug_transpose_traffic_model", P(xs[i]), m, k, P(qt[i]), ld_t, None, st), n))
-    out[prefix + "quantize_both_forms_traffic_model"] = _gb(m * k * 4, _time_rot(lambda i: _lib.call(
-        "hpfp8_debug_transpose_traffic_model", P(xs[i]), m, k, P(qt[i]), ld_t, P(q[i]), st), n))
+    out[prefix + "requant_t_traffic_model"] = _gb(m * k * 3, T(lambda i: _lib.call(
+        "hpfp8_debug_transpose_traffic_model", P(xs[i]), m, k, P(qt[i]), ld_t, None, st)))
+    out[prefix + "quantize_both_forms_traffic_model"] = _gb(m * k * 4, T(lambda i: _lib.call(
+        "hpfp8_debug_transpose_traffic_model", P(xs[i]), m, k, P(qt[i]), ld_t, P(q[i]), st)))
     return out
 
 
@@ -529,6 +530,23 @@ def other_configs_compact(dev):
                           "dequantize": _gb(nbytes, _time(lambda: hpfp8.dequantize_bucket(codes, si)))}
     del flat, codes, si
     torch.cuda.empty_cache()
+    return res
+
+
+def cfg3_quantizers_only(dev, iters=8, warm=4):
+    """--cfg3-quantizers: nothing but the quantizer rows of configuration 3 (x[4096, 16384] and grad_out[4096, 7168],
+    drawn as in the full run, every form, on rotating buffers), with few launches: the command the counter runs of
+    profiles/ use, so that their per-kernel rows hold these shapes only."""
+    import torch
+    m, n, k = 4096, 7168, 16384
+    g3 = torch.Generator(device="cpu").manual_seed(0)
+    x = cpu_draw(g3, (m, k)).to(torch.bfloat16).to(dev)
+    u = cpu_draw(g3, (m, n), kind="rand") - 0.5
+    go = (-(2 ** -0.5) * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.4999999)) * 1e-3).to(torch.bfloat16).to(dev)
+    res = quantizer_rows(x, dev, "x_", iters=iters, warm=warm)
+    del x
+    torch.cuda.empty_cache()
+    res.update(quantizer_rows(go, dev, "grad_out_", iters=iters, warm=warm))
     return res
 
 
@@ -748,6 +766,8 @@ def main():
                     help="also time the layers around the kernels, the optional recipe and the fused bucket forms "
                          "(adds a 'more' key; the other four configurations are always under 'other_configs')")
     ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
+    ap.add_argument("--cfg3-quantizers", action="store_true",
+                    help="run only the quantizer rows of configuration 3 (for counter collection) and print them")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU's share of the path; this build has no multi-GPU leg "
@@ -761,6 +781,9 @@ def main():
     lib = _lib.load()
     assert lib.hpfp8_check_device() == 0, lib.hpfp8_last_error().decode()
     dev = torch.device("cuda:0")
+    if args.cfg3_quantizers:
+        print(json.dumps({"cfg3_quantizers": cfg3_quantizers_only(dev)}))
+        return
     x, w = make_inputs(dev)
 
     # preallocated outputs: nothing is allocated inside the timed region
