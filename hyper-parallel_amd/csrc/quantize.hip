@@ -913,12 +913,20 @@ __global__ __launch_bounds__(256) void column_sum_partial_kernel(const uint16_t*
 }
 
 // out[col] = ((0 + part[0][col]) + part[1][col]) + ... in block order, as fp32 and / or rounded once to bf16
-__global__ __launch_bounds__(256) void column_sum_finish_kernel(const float* __restrict__ part, int blocks, int k,
-                                                                uint16_t* __restrict__ out_bf16, float* __restrict__ out_f32) {
-  const int col = blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(64) void column_sum_finish_kernel(const float* __restrict__ part, int blocks, int k,
+                                                               uint16_t* __restrict__ out_bf16, float* __restrict__ out_f32) {
+  const int col = blockIdx.x * 64 + threadIdx.x;
   if (col >= k) return;
   float s = 0.f;
-  for (int b = 0; b < blocks; ++b) s += part[(int64_t)b * k + col];
+  int b = 0;
+  for (; b + 16 <= blocks; b += 16) {      // sixteen loads in flight, added in block order (the order is the contract)
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = part[(int64_t)(b + u) * k + col];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) s += v[u];
+  }
+  for (; b < blocks; ++b) s += part[(int64_t)b * k + col];
   if (out_f32) out_f32[col] = s;
   if (out_bf16) out_bf16[col] = __builtin_bit_cast(uint16_t, (__bf16)s);
 }
@@ -1466,7 +1474,7 @@ int hpfp8_column_sum_finish(const float* partial, int64_t blocks, int64_t cols, 
   HPFP8_REQUIRE(blocks >= 0 && cols >= 0 && blocks < (1 << 30) && cols < (1 << 30), HPFP8_ERR_SHAPE, "column_sum_finish: bad shape");
   if (cols == 0) return HPFP8_OK;
   HPFP8_REQUIRE((partial || blocks == 0) && (out_bf16 || out_f32), HPFP8_ERR_ARG, "column_sum_finish: null buffer");
-  column_sum_finish_kernel<<<(unsigned)((cols + 255) / 256), 256, 0, (hipStream_t)stream>>>(partial, (int)blocks, (int)cols,
+  column_sum_finish_kernel<<<(unsigned)((cols + 63) / 64), 64, 0, (hipStream_t)stream>>>(partial, (int)blocks, (int)cols,
                                                                                           (uint16_t*)out_bf16, out_f32);
   return check_launch("column_sum_finish");
 }
