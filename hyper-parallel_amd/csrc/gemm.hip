@@ -870,13 +870,17 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_kernel(const GemmParams p) 
 // so the two give identical results.  Per-tensor and 128x128-block scale forms, dense, bf16 or fp32 output, bias.
 constexpr int kSmallThreads = 256;
 constexpr int kSmallTile = 128;
-constexpr int kSmallStageBytes = 2 * kSmallTile * BK;   // a tile + b tile
 constexpr int kSmallStages = 5;
 
-template <int MODE, bool OUT_F32>
+// TM: rows of the tile, 128 or 64.  With 64 (wave tile 32 x 64) a problem has twice as many workgroups: the form for
+// problems whose 128 x 128 tiles would leave compute units idle (cfg 1: 128 tiles on 256 compute units).
+template <int MODE, bool OUT_F32, int TM = 128>
 __global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmParams p) {
   static_assert(MODE == kScaleTensor || MODE == kScaleBlock, "per-tensor or block scales");
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[kSmallStages * kSmallStageBytes];
+  static_assert(TM == 128 || TM == 64, "tile rows");
+  constexpr int kStageBytes = (TM + kSmallTile) * BK;     // a tile + b tile
+  constexpr int NA = TM / 32;                             // a transfers per wave and k-block; also m-subtiles per wave
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kSmallStages * kStageBytes];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
@@ -884,8 +888,8 @@ __global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmPar
   const int kblocks = p.K / BK;
   const int tiles_n = p.N / kSmallTile;
   const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
-  const int row0 = tm * kSmallTile, n0 = tn * kSmallTile;
-  const int rows_valid = p.M - row0 < kSmallTile ? p.M - row0 : kSmallTile;
+  const int row0 = tm * TM, n0 = tn * kSmallTile;
+  const int rows_valid = p.M - row0 < TM ? p.M - row0 : TM;
 
   // transfers: as in gemm_kernel, a wave moves 8 rows x 128 B per instruction, four per operand tile and k-block;
   // the resources start at the tile's first row and end with the tensor (rows past it read as zero); k-blocks
@@ -904,42 +908,46 @@ __global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmPar
   for (int i = 0; i < 4; ++i) {
     const int r = (wave * 4 + i) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ row_swizzle(r);
-    a_off[i] = (uint32_t)r * (uint32_t)p.lda + chunk * 16 - i * 1024;
     b_off[i] = (uint32_t)r * (uint32_t)p.ldb + chunk * 16 - i * 1024;
+    const int ra = (wave * NA + (i < NA ? i : 0)) * 8 + (lane >> 3);
+    const int chunk_a = (lane & 7) ^ row_swizzle(ra);
+    a_off[i] = (uint32_t)ra * (uint32_t)p.lda + chunk_a * 16 - (i < NA ? i : 0) * 1024;
   }
   auto issue_stage = [&](int kb, int stage) {
     const bool ok = kb < kblocks;
     const __amdgpu_buffer_rsrc_t ra = ok ? rs_a : rs_none, rb = ok ? rs_b : rs_none;
-    uint8_t* sa_base = lds + stage * kSmallStageBytes + wave * 4096;
-    uint8_t* sb_base = sa_base + kSmallTile * BK;
+    uint8_t* sa_base = lds + stage * kStageBytes + wave * (NA * 1024);
+    uint8_t* sb_base = lds + stage * kStageBytes + TM * BK + wave * 4096;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[0], kb * BK, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[1], kb * BK, 1024, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[2], kb * BK, 2048, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[3], kb * BK, 3072, 0);
+    if (NA == 4) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[2], kb * BK, 2048, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)sa_base, 16, a_off[3], kb * BK, 3072, 0);
+    }
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[0], kb * BK, 0, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[1], kb * BK, 1024, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[2], kb * BK, 2048, 0);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)sb_base, 16, b_off[3], kb * BK, 3072, 0);
   };
   const int pc0 = (2 * g) ^ row_swizzle(l16);
-  const int a_frag = (wm * 64 + l16) * BK, b_frag = kSmallTile * BK + (wn * 64 + l16) * BK;
+  const int a_frag = (wm * (TM / 2) + l16) * BK, b_frag = TM * BK + (wn * 64 + l16) * BK;
 
   // scales of the block form: this lane's four rows of a (clamped: rows past M are never stored), the tile's
   // one 128-row block of b
-  const float* sa_row[4];
+  const float* sa_row[NA];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int r = row0 + wm * 64 + j * 16 + l16;
+  for (int j = 0; j < NA; ++j) {
+    const int r = row0 + wm * (TM / 2) + j * 16 + l16;
     sa_row[j] = p.sa + (int64_t)(r < p.M ? r : p.M - 1) * p.sa_sm;
   }
   const float* sb_blk = p.sb + (int64_t)(n0 >> 7) * p.sb_sn;
 
   const v4f zero = {0.f, 0.f, 0.f, 0.f};
-  v4f acc[4][4];
+  v4f acc[4][NA];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = zero;
+    for (int j = 0; j < NA; ++j) acc[i][j] = zero;
 
   // Transfers run four k-blocks ahead (five stages); the block form's scales are fetched three k-blocks ahead
   // into a ring of registers, so that waiting for them never waits for a transfer that is not needed yet
@@ -951,7 +959,7 @@ __global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmPar
       const int kk = kb < kblocks ? kb : kblocks - 1;
       raw[4] = sb_blk[(int64_t)kk * p.sb_sk];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) raw[j] = sa_row[j][(int64_t)kk * p.sa_sk];
+      for (int j = 0; j < NA; ++j) raw[j] = sa_row[j][(int64_t)kk * p.sa_sk];
     }
   };
   issue_stage(0, 0);
@@ -969,39 +977,43 @@ __global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmPar
     // all but the youngest transfers of three k-blocks (and, block form, the scale loads issued between them)
     // have landed: this k-block's tiles of this wave; after the barrier everyone's, and everyone has left the
     // stage that is refilled next
-    if (MODE == kScaleBlock) asm volatile("s_waitcnt vmcnt(34)\n\ts_barrier" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
+    // (in flight and allowed to stay so: the transfers of three k-blocks, NA + 4 each, and in the block form the scale
+    // loads of two, NA + 1 each)
+    if (MODE == kScaleBlock && NA == 4) asm volatile("s_waitcnt vmcnt(34)\n\ts_barrier" ::: "memory");
+    else if (MODE == kScaleBlock) asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
+    else if (NA == 4) asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
     load_scales(kb + 3, s_ring[(Q + 3) & 3]);
     asm volatile("" ::: "memory");       // (keeps the scale loads ahead of the transfers, as the wait above counts them)
     issue_stage(kb + 4, st_issue);
-    const uint8_t* base = lds + st * kSmallStageBytes;
+    const uint8_t* base = lds + st * kStageBytes;
     st = st == kSmallStages - 1 ? 0 : st + 1;
     st_issue = st_issue == kSmallStages - 1 ? 0 : st_issue + 1;
-    v8i xf[4], wf[4];
+    v8i xf[NA], wf[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xf[j] = frag_read(base + a_frag + j * 16 * BK, pc0);
+    for (int j = 0; j < NA; ++j) xf[j] = frag_read(base + a_frag + j * 16 * BK, pc0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) wf[i] = frag_read(base + b_frag + i * 16 * BK, pc0);
     if (MODE == kScaleTensor) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NA; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
     } else {
-      v4f part[4][4];
+      v4f part[4][NA];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NA; ++j)
           part[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf[j], zero, 0, 0, 0, 0, 0, 0);
-      float s[4];
+      float s[NA];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) s[j] = s_ring[Q][j] * s_ring[Q][4];
+      for (int j = 0; j < NA; ++j) s[j] = s_ring[Q][j] * s_ring[Q][4];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NA; ++j)
 #pragma unroll
           for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(part[i][j][r], s[j], acc[i][j][r]);
     }
@@ -1018,8 +1030,8 @@ __global__ __launch_bounds__(kSmallThreads) void gemm_small_kernel(const GemmPar
   float tensor_scale = 1.f;
   if (MODE == kScaleTensor) tensor_scale = p.sa[0] * p.sb[0];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int r = wm * 64 + j * 16 + l16;
+  for (int j = 0; j < NA; ++j) {
+    const int r = wm * (TM / 2) + j * 16 + l16;
     if (r >= rows_valid) continue;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1079,7 +1091,15 @@ static bool use_small_kernel(int64_t M, int64_t N) {
 template <int MODE>
 static int launch_small(const GemmParams& p, int out_type, hipStream_t stream) {
   const int64_t tiles = (((int64_t)p.M + kSmallTile - 1) / kSmallTile) * (p.N / kSmallTile);
-  dim3 grid((unsigned)tiles), block(kSmallThreads);
+  dim3 block(kSmallThreads);
+  // fewer 128 x 128 tiles than compute units: tiles of 64 rows, twice as many workgroups (the same results)
+  if (tiles < persistent_grid((int64_t)1 << 40)) {
+    dim3 grid((unsigned)((((int64_t)p.M + 63) / 64) * (p.N / kSmallTile)));
+    if (out_type == HPFP8_OUT_F32) gemm_small_kernel<MODE, true, 64><<<grid, block, 0, stream>>>(p);
+    else gemm_small_kernel<MODE, false, 64><<<grid, block, 0, stream>>>(p);
+    return check_launch("gemm (small tiles)");
+  }
+  dim3 grid((unsigned)tiles);
   if (out_type == HPFP8_OUT_F32) gemm_small_kernel<MODE, true><<<grid, block, 0, stream>>>(p);
   else gemm_small_kernel<MODE, false><<<grid, block, 0, stream>>>(p);
   return check_launch("gemm (small tiles)");

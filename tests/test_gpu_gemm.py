@@ -718,12 +718,13 @@ def small_gemm_mode():
 
 
 @pytest.mark.parametrize("shape", [(2048, 1024, 1024), (1, 128, 128), (130, 384, 256), (64, 2304, 512), (257, 128, 1152),
-                                   (1000, 640, 384)])
+                                   (1000, 640, 384), (2048, 2304, 256), (4100, 1024, 384)])
 def test_small_tile_kernel_equals_the_large_tile_kernel_and_the_oracle(gpu, shape, small_gemm_mode):
-    """The 128 x 128-tile kernel (problems with few tiles: BASELINE configuration 1, decode-sized M) does the same
+    """The small-tile kernel (problems with few tiles: BASELINE configuration 1, decode-sized M) does the same
     arithmetic in the same order as the 256 x 256-tile kernel: identical bits for the block and the per-tensor
     form, fp32 and bf16 output, with and without bias, ragged M; and the fp32 output agrees with the oracle as the
-    large kernel's does."""
+    large kernel's does.  Both of its tile heights are covered: 64 rows where 128 x 128 tiles would be fewer than the
+    256 compute units (the first six shapes), 128 rows otherwise (288 and 264 such tiles in the last two)."""
     import hpfp8
     m, n, k = shape
     x = U.randn_bf16((m, k), 40 + m, 1.0, 0.001, 30.0).to(gpu)
