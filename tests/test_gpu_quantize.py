@@ -67,6 +67,21 @@ def test_golden_fixtures(gpu):
     assert np.array_equal(U.codes(qt), P["t128x1_codes"]) and eq_f32(s, P["t128x1_scale"]) and eq_f32(si, P["t128x1_scale_inv"])
 
 
+@pytest.mark.parametrize("pow2", [False, True])
+def test_128x128_two_blocks_per_workgroup(gpu, pow2):
+    # from 4096 blocks on, with an even number of block columns and no transposed copy, a workgroup quantizes two
+    # neighbouring blocks: same bits as the oracle and as the one-block kernel (which the transposing call uses)
+    import hpfp8
+    x = U.randn_bf16((16384, 4096), 21, 0.05, 0.002, 300.0)
+    xb = U.bits(x)
+    xg = x.to(gpu)
+    rq, rs, rsi = O.quantize_128x128(xb, pow2=True) if pow2 else C.quantize_128x128(xb)
+    q, si, s = hpfp8.quantize_128x128(xg, want_scale=True, pow2=pow2)
+    assert np.array_equal(U.codes(q), rq) and eq_f32(s, rs) and eq_f32(si, rsi)
+    q1, si1, qt1, s1 = hpfp8.quantize_128x128(xg, with_transpose=True, want_scale=True, pow2=pow2)
+    assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(si, si1) and torch.equal(s, s1)
+
+
 @pytest.mark.parametrize("shape,seed,std,of,om", [
     ((2048, 1024), 0, 1.0, 0.0, 1.0),          # cfg 1 activations
     ((1024, 1024), 1, 0.02, 0.0, 1.0),         # cfg 1 weights
