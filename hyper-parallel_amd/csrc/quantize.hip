@@ -210,7 +210,10 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
   if (SYNC3) {
     if (threadIdx.x < 64) {              // the first wave: lane l watches slot l
       const uint32_t lane = threadIdx.x;
-      if (lane == 0) __hip_atomic_store(amax_word + blockIdx.x, kSlotValid | m, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      // (Relaxed accesses: a slot's value is all that is communicated -- nothing else is published with it, nothing
+      // else of another workgroup's is read after it -- so no cache needs writing back or invalidating; a release or
+      // an acquire at device scope does that to the XCD's whole L2.)
+      if (lane == 0) __hip_atomic_store(amax_word + blockIdx.x, kSlotValid | m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       uint32_t spins = 0, slot = 0;
       bool all = false;
       while (true) {
@@ -219,7 +222,6 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
         if (all || spins++ >= spin_limit) break;
         __builtin_amdgcn_s_sleep(1);
       }
-      __atomic_thread_fence(__ATOMIC_ACQUIRE);
       uint32_t mx = (slot & kSlotValid) ? (slot & 0xFFFFu) : 0u;
       mx = row16_max_u32(mx);
       mx = umax(mx, (uint32_t)__shfl_xor((int)mx, 16));
@@ -268,12 +270,12 @@ __global__ __launch_bounds__(kFusedThreads) void quant_per_tensor_fused_kernel(c
       if (scale_out) *scale_out = scale;
       if (scale_inv_out) *scale_inv_out = scale_inv;
     }
-    // this workgroup has read the slots for the last time (before the barrier above); the last one to say so clears
-    // them for the next launch
+    // this workgroup has read the slots for the last time (before the barrier above: the values had arrived, they
+    // were used); the last one to say so clears them for the next launch
     if (threadIdx.x < 64) {
       uint32_t last = 0;
       if (threadIdx.x == 0)
-        last = __hip_atomic_fetch_add(count_word, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) + 1u == grid ? 1u : 0u;
+        last = __hip_atomic_fetch_add(count_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u == grid ? 1u : 0u;
       last = (uint32_t)__shfl((int)last, 0);
       if (last) {
         __hip_atomic_store(amax_word + threadIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
